@@ -1,0 +1,229 @@
+/* C ABI of libsocket_hip.so: SOCKET's sparse-decode hot path on MI355X (gfx950).
+ *
+ * Every entry point takes raw device pointers, explicit sizes and element
+ * strides, and a HIP stream handle passed as void* (hipStream_t; NULL = the
+ * default stream).  Outputs and workspaces are allocated by the caller; the
+ * library allocates nothing, keeps no state besides cached device limits, and
+ * is re-entrant.  Kernels are enqueued on `stream` and the call returns without
+ * synchronising.  The return value is a status: 0 on success, a negative
+ * SOCKET_ERR_* otherwise; on error nothing was launched.
+ *
+ * Citations name the reference interface each entry point replaces, as
+ * path:line inside the SOCKET checkout.
+ *
+ * Shapes use B batch, Hq query heads, Hkv key/value heads, G = Hq / Hkv,
+ * D head dim, T context length, Tcap cache capacity (row pitch of the hash
+ * cache), L hash tables, P hyperplanes per table (code < 2^P), R entries per
+ * soft-hash table (R >= 2^P), M top-k budget.
+ *
+ * Packed code format (this library's own; the reference keeps int16 codes
+ * [B,Hkv,T,L]): c = 32 / P codes per 32-bit word, NW = ceil(L / c) words per
+ * key; table l lives in word l / c at bit offset (l % c) * P; unused high bits
+ * are zero.  Words are stored table-major per KV head: uint32 [B,Hkv,NW,Tcap],
+ * so consecutive tokens of one word index are consecutive in memory.
+ */
+#ifndef SOCKET_HIP_H_
+#define SOCKET_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SOCKET_ABI_VERSION 1
+
+/* status codes */
+#define SOCKET_OK 0
+#define SOCKET_ERR_NULL (-1)        /* a required pointer is NULL */
+#define SOCKET_ERR_SHAPE (-2)       /* sizes inconsistent or out of range */
+#define SOCKET_ERR_UNSUPPORTED (-3) /* dtype / head dim / table size not built */
+#define SOCKET_ERR_ALIGN (-4)       /* pointer or pitch not aligned as required */
+#define SOCKET_ERR_WORKSPACE (-5)   /* workspace smaller than *_workspace_bytes */
+#define SOCKET_ERR_LAUNCH (-6)      /* hipGetLastError() after the launch */
+
+/* element types of q / k / v / out */
+#define SOCKET_F32 0
+#define SOCKET_BF16 1
+#define SOCKET_F16 2
+
+int socket_abi_version(void);
+const char* socket_status_string(int status);
+/* Compute-unit count and LDS bytes per workgroup of the current device. */
+int socket_device_query(int* cu_count, int* max_lds_bytes);
+
+/* ------------------------------------------------------------------------
+ * K1  key hashing (+ fused value norm)
+ * ---------------------------------------------------------------------- */
+
+/* NW for (L, P); 0 if P is outside [1,16] or L < 1. */
+int socket_words_per_key(int L, int P);
+
+/* planes [L,P,D] (SOCKET_F32/BF16/F16) -> bf16 [NW*32, D]: row w*32+p is the
+ * hyperplane whose sign becomes bit p of packed word w, zero rows for unused
+ * bits.  Done once per layer.  Replaces the weights tensor of pack_bits,
+ * GPT-FAST/model.py:403-407, by ordering the contraction's columns. */
+int socket_permute_planes(const void* planes, int planes_dtype, int L, int P, int D,
+                          void* planes_words, void* stream);
+
+/* Hash S new keys per (b, kv head) and store their packed codes and value
+ * norms at cache positions pos0(b)+s, s in [0,S): pos0(b) = pos_b ? pos_b[b] : t0.
+ * k, v address element [0,0,0,0] of the new rows with the given element strides
+ * (last dim contiguous); v may be NULL (then v_norm is not written).
+ * bit = (k . plane >= 0) from an MFMA bf16 contraction with fp32 accumulation.
+ * Replaces Attention.hard_hash_keys + pack_bits, GPT-FAST/model.py:403-413, the
+ * value norm at GPT-FAST/model.py:450 and the k_hard / v_norm writes of
+ * KVCache.update, GPT-FAST/model.py:222-226.
+ * Requires D == 128, 16-byte aligned rows. */
+int socket_hash_keys(const void* k, const void* v, int dtype,
+                     int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                     int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                     const void* planes_words, uint32_t* codes, uint16_t* v_norm,
+                     const int32_t* pos_b, int t0,
+                     int B, int Hkv, int S, int D, int L, int P, int64_t Tcap,
+                     void* stream);
+
+/* Packed words -> int16 codes with arbitrary output strides (elements) over
+ * (b, h, l, t) for tokens [t0, t0+T).  out[b,h,l,t-t0].  Gives the reference's
+ * k_hard layouts: [B,S,Hkv,L] (GPT-FAST/model.py:413) or [B,H,L,T]
+ * (pipeline/train_quest/modeling/modeling_llama.py:615). */
+int socket_unpack_codes(const uint32_t* codes, int16_t* out, int B, int Hkv, int L, int P,
+                        int t0, int T, int64_t Tcap,
+                        int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l,
+                        int64_t out_stride_t, void* stream);
+
+/* int16 codes with arbitrary strides over (b, h, l, t) -> packed words at
+ * positions [t0, t0+T) of the cache. */
+int socket_pack_codes(const int16_t* in, int64_t in_stride_b, int64_t in_stride_h,
+                      int64_t in_stride_l, int64_t in_stride_t,
+                      uint32_t* codes, int B, int Hkv, int L, int P, int t0, int T,
+                      int64_t Tcap, void* stream);
+
+/* ------------------------------------------------------------------------
+ * K2  soft-collision scorer
+ * ---------------------------------------------------------------------- */
+
+/* Native scorer on the packed cache.  For every b, kv head, token t < T and
+ * each of the G query heads h of that kv head:
+ *   scores[b,h,t] = t < len(b) ? (sum_{l<L} q_probs[b,h,l,code_l(b,kv,t)]) * v_norm[b,kv,t] : -inf
+ * with the sum taken over l ascending in fp32 (the order of the loop at
+ * GPT-FAST/kernels/soft_hash_collision.cu:45-53), len(b) = lens ? lens[b] : T.
+ * q_probs: fp32 [B,Hq,L,R] contiguous (q_dtype must be SOCKET_F32).
+ * scores: fp32, row (b,h) at scores + (b*Hq+h)*score_stride.
+ * Codes are read once per kv head, not once per query head.
+ * Replaces the relayout at GPT-FAST/model.py:490-509 and the scorer call at
+ * GPT-FAST/kernels/sparse.py:42-55.
+ * Requires Tcap % 4 == 0, score_stride % 4 == 0, 16-byte aligned pointers,
+ * R a power of two, 2^P <= R, G <= 8. */
+int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
+                        const uint16_t* v_norm, const int32_t* lens, float* scores,
+                        int B, int Hq, int Hkv, int L, int P, int R, int T, int64_t Tcap,
+                        int64_t score_stride, void* stream);
+
+/* The reference extension's entry point on its own layout:
+ * q_probs f32 [B,H,1,L,R], key_buckets i16 [B,H,L,T], allowed bool [B,H,1,T],
+ * v_hist f32 [B,H,1,T] -> out f32 [B,H,1,T], all contiguous.
+ * Replaces ext.soft_hash_collision, GPT-FAST/kernels/soft_hash_collision_loader.py:14-74
+ * (kernel GPT-FAST/kernels/soft_hash_collision.cu:25-54). */
+int socket_soft_hash_collision(const float* q_probs, const int16_t* key_buckets,
+                               const uint8_t* allowed, const float* v_hist, float* out,
+                               int B, int H, int L, int R, int T, void* stream);
+
+/* fp16 variant: q_probs f16 [B,H,L,R], v_norm f16 [B,H,T], any L.
+ * Replaces soft_hash_score, GPT-FAST/kernels/soft_hash_score/soft_hash_score_bindings.cpp:10-36
+ * (kernel GPT-FAST/kernels/soft_hash_score/soft_hash_score.cu:7-42). */
+int socket_soft_hash_score_f16(const uint16_t* q_probs, const int16_t* key_buckets,
+                               const uint16_t* v_norm, const uint8_t* allowed, float* out,
+                               int B, int H, int L, int R, int T, void* stream);
+
+/* ------------------------------------------------------------------------
+ * K3  top-k select and index list
+ * ---------------------------------------------------------------------- */
+
+/* Per row (b,h) of fp32 scores: the m = min(budget(b), len(b)) largest entries
+ * of scores[0:len(b)] in descending score order, equal scores by ascending
+ * index, written as int32 after the sink/window part so that the row of
+ * sparse_list is [sink | window | heavy | -1 padding up to list_width]:
+ *   sink   = 0 .. min(sink,len)-1
+ *   window = max(len - min(window,len), min(sink,len)) .. len-1
+ *   (both empty -> the single index len-1)
+ * and sparse_len[b,h] = entries before the padding.  len(b) = lens ? lens[b] : T,
+ * budget(b) = budgets ? budgets[b] : M.  With write_base == 0 only the heavy
+ * part is written, starting at column 0.
+ * Replaces torch.topk + the list assembly of build_sparse_list_decode,
+ * GPT-FAST/kernels/sparse.py:57-95.  NaN scores rank above +inf, -0.0 equals +0.0.
+ * Requires M <= SOCKET_TOPK_MAX_M. */
+#define SOCKET_TOPK_MAX_M 16384
+int socket_select_list(const float* scores, int64_t score_stride, const int32_t* lens,
+                       const int32_t* budgets, int B, int Hq, int T, int M, int sink,
+                       int window, int write_base, int32_t* sparse_list, int64_t list_stride,
+                       int list_width, int32_t* sparse_len, void* stream);
+
+/* ------------------------------------------------------------------------
+ * K4  sparse flash-decode
+ * ---------------------------------------------------------------------- */
+
+/* Stage 1: for split s of query head (b,h), attend over list entries
+ * [s*block_seq, min(len, (s+1)*block_seq)) of the kv head h / G; entries < 0
+ * are skipped.  Writes mid_o[b,h,s,:] = acc / sum_exp (fp32 [B,Hq,nsplit,D]) and
+ * mid_lse[b,h,s] = max + log(sum_exp) (fp32 [B,Hq,nsplit]); a split with no
+ * live row gets mid_lse = -inf, mid_o = 0; splits at or beyond len are left
+ * untouched.  Strides are in elements; the last dim of q, k, v is contiguous.
+ * Replaces sparse_decode_stage1, kernels/socket_triton_kernels.py:167-205
+ * (kernel :31-118).  D in {16,32,64,128}; q,k,v of one dtype. */
+int socket_attend_stage1(const void* q, const void* k, const void* v, int dtype,
+                         int64_t q_stride_b, int64_t q_stride_h,
+                         int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                         int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                         const int32_t* sparse_list, int64_t list_stride_b, int64_t list_stride_h,
+                         const int32_t* sparse_len, int64_t len_stride_b, int64_t len_stride_h,
+                         float* mid_o, float* mid_lse,
+                         int B, int Hq, int Hkv, int D, int kv_rows, int nsplit, int block_seq,
+                         void* stream);
+
+/* Stage 2: merge the ceil(len / block_seq) splits of every (b,h) into
+ * out[b,h,:] (out_dtype); len == 0 gives NaN like the reference's 0/0.
+ * Replaces sparse_decode_stage2, kernels/socket_triton_kernels.py:208-235
+ * (kernel :121-164). */
+int socket_attend_stage2(const float* mid_o, const float* mid_lse,
+                         const int32_t* sparse_len, int64_t len_stride_b, int64_t len_stride_h,
+                         void* out, int out_dtype, int64_t out_stride_b, int64_t out_stride_h,
+                         int B, int Hq, int D, int nsplit, int block_seq, void* stream);
+
+/* Split size (list entries per workgroup) socket_sparse_attention uses for a
+ * list of width max_len, and its workspace need. */
+int socket_sparse_attention_block_seq(int B, int Hq, int max_len);
+size_t socket_sparse_attention_workspace_bytes(int B, int Hq, int D, int max_len);
+
+/* Stage 1 + stage 2 with the split size chosen by the library; max_len is the
+ * width of sparse_list (an upper bound of every sparse_len, so no device->host
+ * read of the lengths is needed).
+ * Replaces sparse_attention_fwd, kernels/socket_triton_kernels.py:238-258. */
+int socket_sparse_attention(const void* q, const void* k, const void* v, int dtype,
+                            int64_t q_stride_b, int64_t q_stride_h,
+                            int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                            int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                            const int32_t* sparse_list, int64_t list_stride_b, int64_t list_stride_h,
+                            const int32_t* sparse_len, int64_t len_stride_b, int64_t len_stride_h,
+                            void* out, int64_t out_stride_b, int64_t out_stride_h,
+                            void* workspace, size_t workspace_bytes,
+                            int B, int Hq, int Hkv, int D, int kv_rows, int max_len, void* stream);
+
+/* Dense split-K flash-decode over rows [0, len(b)) of the cache (the
+ * comparator the sparse path is timed against; the reference's dense decode is
+ * Attention.forward, GPT-FAST/model.py:562-589).  K/V rows are read once per kv
+ * head and shared by its G query heads. */
+size_t socket_dense_decode_workspace_bytes(int B, int Hq, int D, int T);
+int socket_dense_decode(const void* q, const void* k, const void* v, int dtype,
+                        int64_t q_stride_b, int64_t q_stride_h,
+                        int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                        int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                        const int32_t* lens, void* out, int64_t out_stride_b, int64_t out_stride_h,
+                        void* workspace, size_t workspace_bytes,
+                        int B, int Hq, int Hkv, int D, int T, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SOCKET_HIP_H_ */

@@ -1,0 +1,129 @@
+// Shared device/host helpers for the SOCKET sparse-decode kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/socket_hip.h"
+
+#define SOCKET_WAVE 64
+
+// Validate a condition on the host before any launch; the entry point returns
+// the given status instead of launching a kernel on operands it cannot handle.
+#define SOCKET_REQUIRE(cond, status) \
+  do {                               \
+    if (!(cond)) return (status);    \
+  } while (0)
+
+#define SOCKET_LAUNCH_CHECK()                                    \
+  do {                                                           \
+    hipError_t e__ = hipGetLastError();                          \
+    if (e__ != hipSuccess) return SOCKET_ERR_LAUNCH;             \
+  } while (0)
+
+static inline int socket_dtype_bytes(int dt) {
+  return dt == SOCKET_F32 ? 4 : (dt == SOCKET_BF16 || dt == SOCKET_F16) ? 2 : 0;
+}
+
+static inline bool socket_aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
+// ---- element conversions -------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {  // round to nearest even
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+  _Float16 x;
+  __builtin_memcpy(&x, &h, 2);
+  return (float)x;
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 x = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
+  uint16_t h;
+  __builtin_memcpy(&h, &x, 2);
+  return h;
+}
+
+// Order-preserving map float -> uint32 used by the top-k select: larger float
+// <=> larger key.  -0.0 is folded onto +0.0 and every NaN onto the largest key,
+// which is how a stable descending sort of floats ranks them.
+__device__ __forceinline__ uint32_t score_to_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;
+  if (u == 0x80000000u) u = 0u;
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+struct DType_f32 {
+  typedef float storage;
+  static constexpr int kEnum = SOCKET_F32;
+  static constexpr int kPer16B = 4;
+};
+struct DType_bf16 {
+  typedef uint16_t storage;
+  static constexpr int kEnum = SOCKET_BF16;
+  static constexpr int kPer16B = 8;
+};
+struct DType_f16 {
+  typedef uint16_t storage;
+  static constexpr int kEnum = SOCKET_F16;
+  static constexpr int kPer16B = 8;
+};
+
+// Unpack one 16-byte vector of elements into floats.
+template <class DT>
+__device__ __forceinline__ void unpack16(const uint4& raw, float* out);
+
+template <>
+__device__ __forceinline__ void unpack16<DType_f32>(const uint4& raw, float* out) {
+  out[0] = __uint_as_float(raw.x);
+  out[1] = __uint_as_float(raw.y);
+  out[2] = __uint_as_float(raw.z);
+  out[3] = __uint_as_float(raw.w);
+}
+template <>
+__device__ __forceinline__ void unpack16<DType_bf16>(const uint4& raw, float* out) {
+  out[0] = __uint_as_float(raw.x << 16);
+  out[1] = __uint_as_float(raw.x & 0xffff0000u);
+  out[2] = __uint_as_float(raw.y << 16);
+  out[3] = __uint_as_float(raw.y & 0xffff0000u);
+  out[4] = __uint_as_float(raw.z << 16);
+  out[5] = __uint_as_float(raw.z & 0xffff0000u);
+  out[6] = __uint_as_float(raw.w << 16);
+  out[7] = __uint_as_float(raw.w & 0xffff0000u);
+}
+template <>
+__device__ __forceinline__ void unpack16<DType_f16>(const uint4& raw, float* out) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = f16_bits_to_f32((uint16_t)(w[i] & 0xffffu));
+    out[2 * i + 1] = f16_bits_to_f32((uint16_t)(w[i] >> 16));
+  }
+}
+
+template <class DT>
+__device__ __forceinline__ void store_elem(void* base, int64_t idx, float v);
+template <>
+__device__ __forceinline__ void store_elem<DType_f32>(void* base, int64_t idx, float v) {
+  ((float*)base)[idx] = v;
+}
+template <>
+__device__ __forceinline__ void store_elem<DType_bf16>(void* base, int64_t idx, float v) {
+  ((uint16_t*)base)[idx] = f32_to_bf16_bits(v);
+}
+template <>
+__device__ __forceinline__ void store_elem<DType_f16>(void* base, int64_t idx, float v) {
+  ((uint16_t*)base)[idx] = f32_to_f16_bits(v);
+}
+
+// Cached device limits (read once per process; the library keeps no other state).
+struct SocketDeviceLimits {
+  int cu_count;
+  int max_lds_per_block;
+};
+const SocketDeviceLimits& socket_device_limits();

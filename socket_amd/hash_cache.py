@@ -1,0 +1,193 @@
+"""The HIP-native decode path: packed per-KV-head hash cache and the
+score -> select -> attend step on it.
+
+This is what the attention hook calls instead of the reference's per-step
+relayout (GPT-FAST/model.py:490-509), scorer + torch.topk + list assembly
+(GPT-FAST/kernels/sparse.py:16-95) and K/V prefix copies
+(GPT-FAST/model.py:541-542).  HBM layout per layer:
+
+  k_cache, v_cache  [B, Hkv, Tcap, D]   model dtype      (as KVCache, model.py:175-176)
+  codes             [B, Hkv, NW, Tcap]  uint32 (int32 tensor), packed bucket codes,
+                                        table-major; replaces k_hard [B,Hkv,T,L] int16
+  v_norm            [B, Hkv, Tcap]      float16          (as KVCache, model.py:182)
+  lens              [B]                 int32, device    (replaces the 0-d prefill_len)
+
+Nothing on the step path reads a length back to the host.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from ._lib import check, dtype_enum, lib, ptr, stream_ptr
+from .socket_kernels import sparse_attention_fwd
+from .sparse import select_list
+
+
+def words_per_key(L: int, P: int) -> int:
+    nw = lib().socket_words_per_key(int(L), int(P))
+    if nw <= 0:
+        raise RuntimeError(f"unsupported hash shape L={L}, P={P} (need L >= 1, 1 <= P <= 16)")
+    return nw
+
+
+@torch.no_grad()
+def permute_planes(planes_lpd: torch.Tensor) -> torch.Tensor:
+    """[L,P,D] hyperplanes -> bf16 [NW*32, D] in packed-bit column order."""
+    assert planes_lpd.is_cuda and planes_lpd.dim() == 3
+    L, P, D = planes_lpd.shape
+    planes_lpd = planes_lpd.contiguous()
+    out = torch.empty((words_per_key(L, P) * 32, D), dtype=torch.bfloat16, device=planes_lpd.device)
+    check("socket_permute_planes", lib().socket_permute_planes(
+        ptr(planes_lpd), dtype_enum(planes_lpd.dtype), L, P, D, ptr(out), stream_ptr(planes_lpd.device)))
+    return out
+
+
+@torch.no_grad()
+def hash_keys_into(k: torch.Tensor, v: Optional[torch.Tensor], planes_words: torch.Tensor,
+                   codes: torch.Tensor, v_norm: Optional[torch.Tensor], L: int, P: int,
+                   t0: int = 0, pos_b: Optional[torch.Tensor] = None, layout: str = "bhsd") -> None:
+    """Hash new keys (and take value norms) into the packed cache at positions
+    t0 + s (or pos_b[b] + s).  `k`/`v` are [B,Hkv,S,D] (layout "bhsd") or
+    [B,S,Hkv,D] ("bshd"), any strides with a contiguous last dim."""
+    assert k.is_cuda and codes.is_cuda and codes.dtype == torch.int32 and codes.is_contiguous()
+    if layout == "bhsd":
+        B, Hkv, S, D = k.shape
+        ks = (k.stride(0), k.stride(1), k.stride(2))
+        vs = (v.stride(0), v.stride(1), v.stride(2)) if v is not None else (0, 0, 0)
+    elif layout == "bshd":
+        B, S, Hkv, D = k.shape
+        ks = (k.stride(0), k.stride(2), k.stride(1))
+        vs = (v.stride(0), v.stride(2), v.stride(1)) if v is not None else (0, 0, 0)
+    else:
+        raise ValueError(layout)
+    assert k.stride(-1) == 1 and (v is None or (v.stride(-1) == 1 and v.shape == k.shape and v.dtype == k.dtype))
+    NW, Tcap = codes.shape[2], codes.shape[3]
+    assert codes.shape[0] == B and codes.shape[1] == Hkv and NW == words_per_key(L, P)
+    if v is not None:
+        assert v_norm is not None and v_norm.dtype == torch.float16 and v_norm.is_contiguous()
+        assert tuple(v_norm.shape) == (B, Hkv, Tcap)
+    if pos_b is not None:
+        assert pos_b.dtype == torch.int32 and pos_b.is_cuda and pos_b.numel() == B
+    if S == 0:
+        return
+    check("socket_hash_keys", lib().socket_hash_keys(
+        ptr(k), ptr(v), dtype_enum(k.dtype), *ks, *vs, ptr(planes_words), ptr(codes), ptr(v_norm),
+        ptr(pos_b), int(t0), B, Hkv, S, D, int(L), int(P), Tcap, stream_ptr(k.device)))
+
+
+@torch.no_grad()
+def unpack_codes(codes: torch.Tensor, L: int, P: int, t0: int, T: int, layout: str = "bhlt") -> torch.Tensor:
+    """Packed words -> int16 codes in one of the reference's layouts:
+    "bhlt" [B,Hkv,L,T] (modeling_llama.py:615) or "bthl" [B,T,Hkv,L] (model.py:413)."""
+    B, Hkv, NW, Tcap = codes.shape
+    if layout == "bhlt":
+        out = torch.empty((B, Hkv, L, T), dtype=torch.int16, device=codes.device)
+        st = (out.stride(0), out.stride(1), out.stride(2), out.stride(3))
+    elif layout == "bthl":
+        out = torch.empty((B, T, Hkv, L), dtype=torch.int16, device=codes.device)
+        st = (out.stride(0), out.stride(2), out.stride(3), out.stride(1))
+    else:
+        raise ValueError(layout)
+    if T > 0:
+        check("socket_unpack_codes", lib().socket_unpack_codes(
+            ptr(codes), ptr(out), B, Hkv, int(L), int(P), int(t0), int(T), Tcap, *st,
+            stream_ptr(codes.device)))
+    return out
+
+
+@torch.no_grad()
+def pack_codes_into(codes_i16_bhlt: torch.Tensor, codes: torch.Tensor, P: int, t0: int = 0) -> None:
+    """int16 [B,Hkv,L,T] (any strides) -> packed words at cache positions [t0, t0+T)."""
+    B, Hkv, L, T = codes_i16_bhlt.shape
+    assert codes_i16_bhlt.dtype == torch.int16 and codes.dtype == torch.int32 and codes.is_contiguous()
+    c = codes_i16_bhlt
+    if T > 0:
+        check("socket_pack_codes", lib().socket_pack_codes(
+            ptr(c), c.stride(0), c.stride(1), c.stride(2), c.stride(3), ptr(codes), B, Hkv, L, int(P),
+            int(t0), T, codes.shape[3], stream_ptr(codes.device)))
+
+
+@torch.no_grad()
+def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
+                 lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Soft-collision scores [B,Hq,T] fp32 (row pitch padded to a multiple of 4)
+    from q_probs fp32 [B,Hq,L,R] and the packed cache."""
+    assert q_probs.is_cuda and q_probs.dim() == 4
+    if q_probs.dtype != torch.float32:
+        q_probs = q_probs.float()
+    q_probs = q_probs.contiguous()
+    B, Hq, L, R = q_probs.shape
+    _, Hkv, NW, Tcap = codes.shape
+    assert codes.dtype == torch.int32 and codes.is_contiguous() and codes.shape[0] == B
+    assert v_norm.dtype == torch.float16 and v_norm.is_contiguous() and tuple(v_norm.shape) == (B, Hkv, Tcap)
+    assert NW == words_per_key(L, P), "codes were packed for a different (L, P)"
+    pitch = (T + 3) // 4 * 4
+    if out is None:
+        out = torch.empty((B, Hq, pitch), dtype=torch.float32, device=q_probs.device)
+    else:
+        assert out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (B, Hq, pitch)
+    if lens is not None:
+        assert lens.dtype == torch.int32 and lens.is_cuda and lens.numel() == B
+    check("socket_score_packed", lib().socket_score_packed(
+        ptr(q_probs), 0, ptr(codes), ptr(v_norm), ptr(lens), ptr(out), B, Hq, Hkv, L, int(P), R, int(T),
+        Tcap, pitch, stream_ptr(q_probs.device)))
+    return out[:, :, :T]
+
+
+@torch.no_grad()
+def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Tensor,
+                       v_cache: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
+                       sink: int, window: int, M: int, lens: Optional[torch.Tensor] = None,
+                       budgets: Optional[torch.Tensor] = None,
+                       return_details: bool = False):
+    """One decode step of sparse attention for one layer: score every cached key,
+    select top-M + sink + window, attend over the selected rows.
+
+    q [B,Hq,D]; q_probs [B,Hq,L,R]; T = number of cached tokens to consider (an
+    upper bound when `lens` gives per-sequence lengths).  Returns out [B,Hq,D].
+    """
+    scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens)
+    sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets)
+    out = sparse_attention_fwd(q, k_cache, v_cache, sparse_list, sparse_len)
+    if return_details:
+        return out, scores, sparse_list, sparse_len
+    return out
+
+
+class SocketHashCache:
+    """Per-layer K/V + hash cache in the layout above, with in-place append."""
+
+    def __init__(self, max_batch_size: int, max_seq_length: int, n_kv_heads: int, head_dim: int,
+                 L: int, P: int, dtype=torch.bfloat16, device="cuda"):
+        B, H, D = max_batch_size, n_kv_heads, head_dim
+        Tcap = (max_seq_length + 7) // 8 * 8
+        self.L, self.P, self.NW, self.Tcap = L, P, words_per_key(L, P), Tcap
+        self.k_cache = torch.zeros((B, H, Tcap, D), dtype=dtype, device=device)
+        self.v_cache = torch.zeros((B, H, Tcap, D), dtype=dtype, device=device)
+        self.codes = torch.zeros((B, H, self.NW, Tcap), dtype=torch.int32, device=device)
+        self.v_norm = torch.zeros((B, H, Tcap), dtype=torch.float16, device=device)
+        self.lens = torch.zeros((B,), dtype=torch.int32, device=device)
+        self.planes_words: Optional[torch.Tensor] = None
+
+    def set_planes(self, planes_lpd: torch.Tensor) -> None:
+        assert tuple(planes_lpd.shape[:2]) == (self.L, self.P)
+        self.planes_words = permute_planes(planes_lpd.to(self.k_cache.device))
+
+    @torch.no_grad()
+    def append(self, pos0: int, k_bshd: torch.Tensor, v_bshd: torch.Tensor) -> None:
+        """Write S new tokens at positions [pos0, pos0+S) for every sequence:
+        K/V rows, packed codes and value norms (KVCache.update,
+        GPT-FAST/model.py:187-229, with the hashing of :449-450 folded in)."""
+        assert self.planes_words is not None, "call set_planes() first"
+        B, S, H, D = k_bshd.shape
+        assert B == self.k_cache.shape[0], "append expects the cache's full batch"
+        if pos0 < 0 or pos0 + S > self.Tcap:
+            raise RuntimeError(
+                f"KVCache.update out-of-bounds: positions [{pos0},{pos0 + S - 1}] but cache T={self.Tcap}")
+        self.k_cache[:, :, pos0:pos0 + S].copy_(k_bshd.permute(0, 2, 1, 3))
+        self.v_cache[:, :, pos0:pos0 + S].copy_(v_bshd.permute(0, 2, 1, 3))
+        hash_keys_into(self.k_cache[:, :, pos0:pos0 + S], self.v_cache[:, :, pos0:pos0 + S],
+                       self.planes_words, self.codes, self.v_norm, self.L, self.P, t0=pos0)
+        self.lens.clamp_(min=pos0 + S)

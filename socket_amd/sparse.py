@@ -1,0 +1,122 @@
+"""Index-list builder with the reference's signature, plus the sparse
+flash-decode entry points re-exported as the reference's module does
+(GPT-FAST/kernels/sparse.py holds both: `build_sparse_list_decode` at :16-95 and
+a copy of the decode kernels at :98-329).
+
+`build_sparse_list_decode` takes the reference's operand layout (int16 codes per
+query head, [B,H,L,T]) and returns the same `(sparse_list, sparse_len)`.  The
+scorer and the top-k + list assembly are HIP kernels; heavy entries are in
+descending score order with equal scores ordered by ascending index.  For the
+layout the HIP path is designed around (packed codes per KV head, no relayout),
+use `socket_amd.hash_cache`.
+"""
+from __future__ import annotations
+
+import torch
+
+from ._lib import SOCKET_TOPK_MAX_M, check, lib, ptr, stream_ptr
+from .socket_kernels import (  # noqa: F401  (re-exported, as in the reference module)
+    attention_mask_to_allowed_prob,
+    sparse_attention_fwd,
+    sparse_decode_stage1,
+    sparse_decode_stage2,
+)
+
+_SOFT_HASH_EXT = None
+
+
+def _get_soft_hash_ext():
+    global _SOFT_HASH_EXT
+    if _SOFT_HASH_EXT is None:
+        from .soft_hash_collision_loader import load_soft_hash_collision
+        _SOFT_HASH_EXT = load_soft_hash_collision(3)
+    return _SOFT_HASH_EXT
+
+
+def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=None, budgets=None,
+                write_base: bool = True, list_width=None):
+    """Top-M + [sink | window | heavy] assembly on fp32 score rows [B,H,T]
+    (row pitch = scores.stride(1)).  Returns (sparse_list int32 [B,H,width],
+    sparse_len int32 [B,H]).  `lens`/`budgets`: optional int32 [B] device tensors
+    (per-sequence context length and top-k budget)."""
+    assert scores.is_cuda and scores.dtype == torch.float32 and scores.dim() == 3
+    assert scores.stride(2) == 1 and scores.stride(0) == scores.shape[1] * scores.stride(1)
+    B, H, T = scores.shape
+    M = int(M)
+    if M > SOCKET_TOPK_MAX_M:
+        raise RuntimeError(f"top-k budget {M} exceeds the supported maximum {SOCKET_TOPK_MAX_M}")
+    if list_width is None:
+        s_e, w_e = max(0, min(sink, T)), max(0, min(window, T))
+        nbase = 0
+        if write_base:
+            nbase = s_e + (T - max(T - w_e, s_e) if w_e > 0 else 0)
+            nbase = max(nbase, 1)
+        list_width = nbase + min(M, T)
+    sparse_list = torch.empty((B, H, list_width), dtype=torch.int32, device=scores.device)
+    sparse_len = torch.empty((B, H), dtype=torch.int32, device=scores.device)
+    if list_width == 0:
+        return sparse_list, sparse_len.zero_()
+    check("socket_select_list", lib().socket_select_list(
+        ptr(scores), scores.stride(1), ptr(lens), ptr(budgets), B, H, T, M, int(sink), int(window),
+        1 if write_base else 0, ptr(sparse_list), list_width, list_width, ptr(sparse_len),
+        stream_ptr(scores.device)))
+    return sparse_list, sparse_len
+
+
+@torch.no_grad()
+def build_sparse_list_decode(
+    q_probs: torch.Tensor,       # [B,H,L,R] fp16/bf16/fp32
+    k_hard_bhlt: torch.Tensor,   # [B,H,L,T] int16/int32
+    v_norm_bht: torch.Tensor,    # [B,H,T] fp16/bf16/fp32
+    allowed_bht: torch.Tensor,   # [B,H,T] bool
+    sink: int,
+    window: int,
+    M: int,
+    KC: int = 8,
+    BLOCK_N: int = 512,
+    num_warps: int = 8,
+    num_stages: int = 2,
+):
+    """GPT-FAST/kernels/sparse.py:16-95.  KC, BLOCK_N, num_warps, num_stages are
+    accepted and ignored, as in the reference (:38)."""
+    assert q_probs.is_cuda and k_hard_bhlt.is_cuda and v_norm_bht.is_cuda and allowed_bht.is_cuda
+    assert q_probs.dtype in (torch.float16, torch.bfloat16, torch.float32)
+    assert allowed_bht.dtype == torch.bool
+    B, H, L, R = q_probs.shape
+    _, _, L2, T = k_hard_bhlt.shape
+    assert L2 == L
+    device = q_probs.device
+    M_eff = min(M, T)
+    if M_eff > 0:
+        ext = _get_soft_hash_ext()
+        q_probs_f32 = q_probs.float().unsqueeze(2).contiguous()
+        key_buckets = k_hard_bhlt if k_hard_bhlt.dtype == torch.int16 else k_hard_bhlt.to(torch.int16)
+        key_buckets = key_buckets.contiguous()
+        allowed_ext = allowed_bht.unsqueeze(2).contiguous()
+        v_hist = v_norm_bht.float().unsqueeze(2).contiguous()
+        scores = ext.soft_hash_collision(q_probs_f32, key_buckets, allowed_ext, v_hist).squeeze(2)
+        heavy_idx, _ = select_list(scores, 0, 0, M_eff, write_base=False)
+        # disallowed positions carry -inf and may still be selected when fewer
+        # than M_eff positions are allowed: they become -1 (:62-68)
+        ok = torch.gather(allowed_bht, -1, heavy_idx.clamp(0, T - 1).long())
+        heavy_idx = heavy_idx.masked_fill(~ok, -1)
+    else:
+        heavy_idx = torch.empty((B, H, 0), device=device, dtype=torch.int32)
+
+    sink = max(0, min(sink, T))
+    window = max(0, min(window, T))
+    parts = []
+    if sink > 0:
+        parts.append(torch.arange(sink, device=device, dtype=torch.int32))
+    if window > 0:
+        win_start = max(T - window, sink)
+        if win_start < T:
+            parts.append(torch.arange(win_start, T, device=device, dtype=torch.int32))
+    base = torch.cat(parts, dim=0) if parts else torch.tensor([T - 1], device=device, dtype=torch.int32)
+    base = base.view(1, 1, -1).expand(B, H, -1)
+    base_ok = torch.gather(allowed_bht, -1, base.long())
+    base = base.masked_fill(~base_ok, -1)
+
+    sparse_list = torch.cat([base, heavy_idx], dim=-1).contiguous()
+    sparse_len = torch.full((B, H), sparse_list.shape[-1], device=device, dtype=torch.int32)
+    return sparse_list, sparse_len

@@ -1,0 +1,420 @@
+"""HIP kernels vs the CPU oracle, through the C ABI (socket_amd -> ctypes -> libsocket_hip.so).
+
+Bars: top-k / lists bit-exact on identical fp32 scores (ties -> lower index);
+scores within 1e-5 relative (the packed scorer sums in the reference's order,
+so it is in fact compared for equality as well where stated); attention within
+2e-2 absolute for bf16/fp16 inputs and 2e-5 for fp32 inputs.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import socket_oracle as orc
+from socket_amd import hash_cache, socket_kernels, sparse
+from socket_amd.soft_hash_collision_loader import load_soft_hash_collision, soft_hash_score
+from socket_amd.workloads import WORKLOADS, make_inputs, scaled
+
+pytestmark = pytest.mark.gpu
+
+ATOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def _rand_codes(g, B, H, L, T, P):
+    return torch.randint(0, 1 << P, (B, H, L, T), generator=g, dtype=torch.int32).to(torch.int16)
+
+
+def _packed_cache(codes_i16_bhlt, P, Tcap, dev):
+    """oracle-packed words -> device int32 [B,Hkv,NW,Tcap]"""
+    words = orc.pack_code_words(codes_i16_bhlt.numpy(), P)  # uint32 [B,H,NW,T]
+    B, H, NW, T = words.shape
+    full = np.zeros((B, H, NW, Tcap), dtype=np.uint32)
+    full[..., :T] = words
+    return torch.from_numpy(full.view(np.int32)).to(dev)
+
+
+# ---------------------------------------------------------------- K2 scorer
+@pytest.mark.parametrize("B,Hq,Hkv,L,P,T", [
+    (1, 8, 2, 32, 8, 1000),      # G=4, P=8 (4 codes / word)
+    (2, 8, 2, 60, 10, 4099),     # G=4, P=10, ragged tail
+    (1, 4, 4, 7, 10, 513),       # G=1, L not a multiple of codes/word
+    (1, 4, 2, 5, 6, 300),        # G=2, runtime-P kernel
+    (1, 14, 2, 48, 10, 2500),    # G=7 (padded to 8)
+    (4, 32, 8, 60, 10, 20000),   # enough work for the 8-tokens-per-lane variant
+])
+def test_score_packed_matches_oracle(dev, B, Hq, Hkv, L, P, T):
+    g = torch.Generator().manual_seed(B * 1000 + L * 10 + P)
+    R = 1 << P
+    G = Hq // Hkv
+    q_probs = torch.rand(B, Hq, L, R, generator=g)
+    codes = _rand_codes(g, B, Hkv, L, T, P)
+    v_norm = (torch.rand(B, Hkv, T, generator=g) * 10).to(torch.float16)
+    lens = torch.randint(T // 2, T + 1, (B,), generator=g, dtype=torch.int32)
+    Tcap = (T + 64 + 7) // 8 * 8
+    vn_full = torch.zeros(B, Hkv, Tcap, dtype=torch.float16)
+    vn_full[..., :T] = v_norm
+    got = hash_cache.score_packed(q_probs.to(dev), _packed_cache(codes, P, Tcap, dev), vn_full.to(dev),
+                                  T, P, lens=lens.to(dev)).cpu()
+    allowed = (torch.arange(T)[None, None, :] < lens[:, None, None]).expand(B, Hq, T)
+    want = orc.collision_score(q_probs, codes.repeat_interleave(G, dim=1), allowed,
+                               v_norm.float().repeat_interleave(G, dim=1))
+    assert torch.equal(got, want), f"max abs diff {(got - want).abs().nan_to_num(0).max()}"
+
+
+def test_score_packed_collision_counts(dev):
+    """Known answer: one-hot q_probs at the query's own codes -> score = (#tables
+    whose code equals the query's) * v_norm, an exact small integer multiple."""
+    g = torch.Generator().manual_seed(7)
+    B, Hq, Hkv, L, P, T = 1, 4, 1, 60, 10, 3000
+    R = 1 << P
+    qcode = torch.randint(0, R, (B, Hq, L), generator=g)
+    q_probs = torch.zeros(B, Hq, L, R).scatter_(-1, qcode.unsqueeze(-1), 1.0)
+    codes = _rand_codes(g, B, Hkv, L, T, P)
+    codes[0, 0, :, 17] = qcode[0, 2].to(torch.int16)          # key 17 collides with head 2 in every table
+    codes[0, 0, :30, 99] = qcode[0, 0, :30].to(torch.int16)   # key 99: >= 30 tables of head 0
+    v_norm = torch.full((B, Hkv, T), 2.0, dtype=torch.float16)
+    Tcap = 3008
+    vn = torch.zeros(B, Hkv, Tcap, dtype=torch.float16); vn[..., :T] = v_norm
+    got = hash_cache.score_packed(q_probs.to(dev), _packed_cache(codes, P, Tcap, dev), vn.to(dev), T, P).cpu()
+    count = (codes.long().unsqueeze(1) == qcode.unsqueeze(-1)).sum(2)   # [B,Hq,T]
+    assert torch.equal(got, count.float() * 2.0)
+    assert got[0, 2, 17] == 120.0 and got[0, 0, 99] >= 60.0
+
+
+@pytest.mark.parametrize("L,R,T", [(32, 256, 777), (60, 1024, 4096), (3, 32768, 100)])
+def test_reference_layout_scorer(dev, L, R, T):
+    g = torch.Generator().manual_seed(L + T)
+    B, H = 2, 3
+    q_probs = torch.rand(B, H, L, R, generator=g)
+    codes = torch.randint(0, R, (B, H, L, T), generator=g, dtype=torch.int32).to(torch.int16)
+    allowed = torch.rand(B, H, T, generator=g) > 0.2
+    v_hist = torch.rand(B, H, T, generator=g) * 5
+    ext = load_soft_hash_collision(3)
+    got = ext.soft_hash_collision(q_probs.unsqueeze(2).contiguous().to(dev), codes.to(dev),
+                                  allowed.unsqueeze(2).contiguous().to(dev),
+                                  v_hist.unsqueeze(2).contiguous().to(dev)).squeeze(2).cpu()
+    assert torch.equal(got, orc.collision_score(q_probs, codes, allowed, v_hist))
+    got16 = soft_hash_score(q_probs.half().to(dev), codes.to(dev), v_hist.half().to(dev), allowed.to(dev)).cpu()
+    assert torch.equal(got16, orc.collision_score_vnorm16(q_probs.half(), codes, v_hist.half(), allowed))
+
+
+def test_loader_errors(dev):
+    ext = load_soft_hash_collision()
+    with pytest.raises(ValueError):
+        load_soft_hash_collision(2)
+    q = torch.rand(1, 1, 1, 2, 16, device=dev)
+    kb = torch.zeros(1, 1, 2, 8, dtype=torch.int16, device=dev)
+    al = torch.ones(1, 1, 1, 8, dtype=torch.bool, device=dev)
+    vh = torch.ones(1, 1, 1, 8, device=dev)
+    with pytest.raises(RuntimeError, match="float32"):
+        ext.soft_hash_collision(q.half(), kb, al, vh)
+    with pytest.raises(RuntimeError, match="int16"):
+        ext.soft_hash_collision(q, kb.int(), al, vh)
+    with pytest.raises(RuntimeError, match="shape mismatch"):
+        ext.soft_hash_collision(q, kb, al[..., :4].contiguous(), vh)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ext.soft_hash_collision(q.cpu(), kb, al, vh)
+
+
+# ---------------------------------------------------------------- K3 select
+def _check_select(scores, sink, window, M, dev, lens=None, budgets=None):
+    B, H, T = scores.shape
+    pitch = (T + 3) // 4 * 4
+    buf = torch.full((B, H, pitch), float("nan"))
+    buf[..., :T] = scores
+    sl, ln = sparse.select_list(buf.to(dev)[..., :T], sink, window, M,
+                                lens=None if lens is None else lens.to(dev),
+                                budgets=None if budgets is None else budgets.to(dev))
+    sl, ln = sl.cpu(), ln.cpu()
+    for b in range(B):
+        n = T if lens is None else int(lens[b])
+        m = min(M if budgets is None else min(int(budgets[b]), M), n)
+        base = torch.from_numpy(orc.base_indices(n, sink, window))
+        for h in range(H):
+            heavy = orc.topk_lower_index_first(scores[b, h, :n], m).to(torch.int32)
+            want = torch.cat([base, heavy])
+            assert int(ln[b, h]) == want.numel()
+            assert torch.equal(sl[b, h, :want.numel()], want), (b, h)
+            assert (sl[b, h, want.numel():] == -1).all()
+
+
+@pytest.mark.parametrize("T,M", [(5000, 128), (131072, 2048), (300, 300), (64, 1), (4097, 4000)])
+def test_select_random_scores(dev, T, M):
+    g = torch.Generator().manual_seed(T + M)
+    scores = torch.randn(2, 3, T, generator=g).abs() * 7
+    _check_select(scores, 4, 64, M, dev)
+
+
+def test_select_ties_and_special_values(dev):
+    g = torch.Generator().manual_seed(3)
+    T = 20000
+    s = torch.randint(0, 50, (1, 6, T), generator=g).float()     # heavy ties, few distinct values
+    s[0, 1] = 1.0                                                 # all equal -> indices 0..M-1
+    s[0, 2, ::3] = float("-inf")                                  # masked keys
+    s[0, 3, 5] = float("nan"); s[0, 3, 77] = float("inf")         # NaN ranks first, then +inf
+    s[0, 4] = torch.randn(T, generator=g)                         # negative values
+    s[0, 4, 10] = 0.0; s[0, 4, 11] = -0.0                         # signed zeros compare equal
+    s[0, 5] = torch.where(torch.arange(T) % 2 == 0, 3.0, 2.0)     # one huge tie class straddling M
+    for M in (1, 700, 5000):
+        _check_select(s, 4, 16, M, dev)
+
+
+def test_select_ragged_lengths_and_budgets(dev):
+    g = torch.Generator().manual_seed(11)
+    B, H, T = 4, 2, 9000
+    scores = torch.rand(B, H, T, generator=g)
+    lens = torch.tensor([9000, 130, 4097, 1], dtype=torch.int32)
+    budgets = torch.tensor([180, 500, 81, 3], dtype=torch.int32)
+    _check_select(scores, 4, 128, 500, dev, lens=lens, budgets=budgets)
+
+
+def test_select_base_enumeration(dev):
+    """List arithmetic for every small T (sparse.py:70-95), including the
+    'empty base -> [T-1]' rule."""
+    for T in range(1, 12):
+        for sink, window in ((0, 0), (2, 3), (4, 0), (0, 5), (20, 20)):
+            scores = torch.arange(T, dtype=torch.float32).flip(0).view(1, 1, T).contiguous()
+            _check_select(scores, sink, window, 3, dev)
+
+
+@pytest.mark.parametrize("T,M,sink,window", [(700, 64, 4, 32), (50, 80, 4, 64), (9, 0, 2, 2)])
+def test_build_sparse_list_decode_reference_layout(dev, T, M, sink, window):
+    g = torch.Generator().manual_seed(T)
+    B, H, L, P = 2, 4, 12, 8
+    R = 1 << P
+    q_probs = torch.rand(B, H, L, R, generator=g).to(torch.bfloat16)
+    codes = _rand_codes(g, B, H, L, T, P)
+    v_norm = torch.rand(B, H, T, generator=g).to(torch.float16)
+    allowed = torch.rand(B, H, T, generator=g) > 0.1
+    allowed[1, 2, T // 4:] = False          # fewer allowed keys than M on one row
+    sl, ln = sparse.build_sparse_list_decode(q_probs.to(dev), codes.to(dev), v_norm.to(dev), allowed.to(dev),
+                                             sink=sink, window=window, M=M)
+    wl, wn = orc.build_sparse_list_decode(q_probs, codes, v_norm, allowed, sink, window, M)
+    assert sl.dtype == torch.int32 and ln.dtype == torch.int32
+    assert torch.equal(sl.cpu(), wl) and torch.equal(ln.cpu(), wn)
+
+
+# ---------------------------------------------------------------- K4 attend
+def _attend_case(dev, dtype, B, Hq, Hkv, D, S, Kt, seed, neg_frac=0.0, ragged=False):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Hq, D, generator=g).to(dtype)
+    k = torch.randn(B, Hkv, S, D, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, S, D, generator=g).to(dtype)
+    sl = torch.randint(0, S, (B, Hq, Kt), generator=g, dtype=torch.int32)   # duplicates on purpose
+    if neg_frac:
+        sl[torch.rand(B, Hq, Kt, generator=g) < neg_frac] = -1
+    ln = torch.full((B, Hq), Kt, dtype=torch.int32)
+    if ragged:
+        ln = torch.randint(1, Kt + 1, (B, Hq), generator=g, dtype=torch.int32)
+    return q, k, v, sl, ln
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D", [128, 64])
+def test_sparse_attention_vs_textbook(dev, dtype, D):
+    q, k, v, sl, ln = _attend_case(dev, dtype, 2, 8, 2, D, 3000, 777, seed=D, neg_frac=0.05, ragged=True)
+    got = socket_kernels.sparse_attention_fwd(q.to(dev), k.to(dev), v.to(dev), sl.to(dev), ln.to(dev))
+    assert got.dtype == dtype
+    want = orc.sparse_attend_textbook(q, k, v, sl, ln)
+    assert (got.cpu().double() - want).abs().max() <= ATOL[dtype]
+
+
+def test_sparse_attention_small_head_dims(dev):
+    for D in (16, 32):
+        q, k, v, sl, ln = _attend_case(dev, torch.bfloat16, 1, 4, 2, D, 500, 100, seed=D)
+        got = socket_kernels.sparse_attention_fwd(q.to(dev), k.to(dev), v.to(dev), sl.to(dev), ln.to(dev))
+        want = orc.sparse_attend_textbook(q, k, v, sl, ln)
+        assert (got.cpu().double() - want).abs().max() <= 2e-2
+
+
+def test_stage1_stage2_match_reference_blocking(dev):
+    """Stage outputs in the reference's own split geometry (block_seq = 256)."""
+    q, k, v, sl, ln = _attend_case(dev, torch.float32, 1, 4, 2, 128, 2000, 600, seed=5, ragged=True)
+    block_seq = 256
+    max_len = int(ln.max())
+    ns = (max_len + block_seq - 1) // block_seq
+    mid_o = torch.full((1, 4, ns, 128), float("nan"), device=dev)
+    mid_l = torch.full((1, 4, ns), float("nan"), device=dev)
+    socket_kernels.sparse_decode_stage1(q.to(dev), k.to(dev), v.to(dev), sl.to(dev), ln.to(dev), max_len,
+                                        mid_o, mid_l, block_seq)
+    wo, wl = orc.sparse_decode_stage1(q, k, v, sl, ln, max_len, block_seq)
+    written = ~torch.isnan(wl)
+    assert torch.equal(~torch.isnan(mid_l.cpu()), written)        # untouched splits stay untouched
+    assert torch.allclose(mid_l.cpu()[written], wl[written], rtol=1e-5, atol=1e-5)
+    assert torch.allclose(mid_o.cpu()[written], wo[written], rtol=1e-4, atol=1e-5)
+    out = torch.empty(1, 4, 128, device=dev)
+    socket_kernels.sparse_decode_stage2(mid_o, mid_l, ln.to(dev), out, block_seq)
+    want = orc.sparse_decode_stage2(wo, wl, ln, torch.float32, block_seq)
+    assert torch.allclose(out.cpu(), want, rtol=1e-4, atol=1e-5)
+
+
+def test_attention_special_cases(dev):
+    g = torch.Generator().manual_seed(9)
+    B, Hq, Hkv, D, S = 1, 8, 2, 128, 1500
+    q = torch.randn(B, Hq, D, generator=g)
+    k = torch.randn(B, Hkv, S, D, generator=g)
+    v = torch.randn(B, Hkv, S, D, generator=g)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    # list = arange(S)  ==  dense attention (library routine)
+    full = torch.arange(S, dtype=torch.int32).view(1, 1, S).expand(B, Hq, S).contiguous()
+    ln = torch.full((B, Hq), S, dtype=torch.int32)
+    got = socket_kernels.sparse_attention_fwd(qd, kd, vd, full.to(dev), ln.to(dev)).cpu()
+    sdpa = torch.nn.functional.scaled_dot_product_attention(
+        q.unsqueeze(2), k.repeat_interleave(4, 1), v.repeat_interleave(4, 1)).squeeze(2)
+    assert torch.allclose(got, sdpa, atol=2e-5)
+    dense = socket_kernels.dense_decode_fwd(qd, kd, vd, torch.tensor([S], dtype=torch.int32, device=dev)).cpu()
+    assert torch.allclose(dense, sdpa, atol=2e-5)
+    # single index -> that V row (GQA map kv = h // G)
+    one = torch.full((B, Hq, 1), 123, dtype=torch.int32)
+    got = socket_kernels.sparse_attention_fwd(qd, kd, vd, one.to(dev), torch.ones(B, Hq, dtype=torch.int32, device=dev)).cpu()
+    assert torch.allclose(got, v[:, :, 123].repeat_interleave(4, 1), atol=1e-6)
+    # a duplicated index doubles its weight
+    dup = torch.tensor([5, 9, 9], dtype=torch.int32).view(1, 1, 3).expand(B, Hq, 3).contiguous()
+    got = socket_kernels.sparse_attention_fwd(qd, kd, vd, dup.to(dev), torch.full((B, Hq), 3, dtype=torch.int32, device=dev)).cpu()
+    kk = k.repeat_interleave(4, 1); vv = v.repeat_interleave(4, 1)
+    lg = torch.stack([(q * kk[:, :, 5]).sum(-1), (q * kk[:, :, 9]).sum(-1)], -1) / math.sqrt(D)
+    w = torch.softmax(lg + torch.tensor([0.0, math.log(2.0)]), -1)
+    want = w[..., :1] * vv[:, :, 5] + w[..., 1:] * vv[:, :, 9]
+    assert torch.allclose(got, want, atol=1e-5)
+    # empty list -> NaN (0/0), as the reference
+    got = socket_kernels.sparse_attention_fwd(qd, kd, vd, dup.to(dev), torch.zeros(B, Hq, dtype=torch.int32, device=dev))
+    assert torch.isnan(got).all()
+
+
+def test_strided_kv_views(dev):
+    """K/V as views of a larger cache (non-contiguous in dims 0-2)."""
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(2, 4, 128, generator=g).to(torch.bfloat16)
+    cache_k = torch.randn(2, 2, 900, 128, generator=g).to(torch.bfloat16)
+    cache_v = torch.randn(2, 2, 900, 128, generator=g).to(torch.bfloat16)
+    sl = torch.randint(0, 500, (2, 4, 64), generator=g, dtype=torch.int32)
+    ln = torch.full((2, 4), 64, dtype=torch.int32)
+    kd, vd = cache_k.to(dev)[:, :, :500], cache_v.to(dev)[:, :, :500]
+    assert not kd.is_contiguous()
+    got = socket_kernels.sparse_attention_fwd(q.to(dev), kd, vd, sl.to(dev), ln.to(dev))
+    want = orc.sparse_attend_textbook(q, cache_k[:, :, :500], cache_v[:, :, :500], sl, ln)
+    assert (got.cpu().double() - want).abs().max() <= 2e-2
+
+
+def test_dense_decode_ragged(dev):
+    g = torch.Generator().manual_seed(33)
+    B, Hq, Hkv, D, T = 3, 14, 2, 128, 5000     # G = 7
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, T, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, T, D, generator=g).to(torch.bfloat16)
+    lens = torch.tensor([5000, 17, 2049], dtype=torch.int32)
+    got = socket_kernels.dense_decode_fwd(q.to(dev), k.to(dev), v.to(dev), lens.to(dev))
+    want = orc.dense_attend(q, k, v, lens)
+    assert (got.cpu().double() - want).abs().max() <= 2e-2
+
+
+# ---------------------------------------------------------------- K1 hash
+@pytest.mark.parametrize("dtype,L,P,S", [(torch.bfloat16, 60, 10, 1000), (torch.float32, 32, 8, 333),
+                                         (torch.float16, 7, 5, 65), (torch.bfloat16, 48, 10, 1)])
+def test_hash_keys_vs_oracle(dev, dtype, L, P, S):
+    g = torch.Generator().manual_seed(L * P + S)
+    B, Hkv, D, t0 = 2, 3, 128, 24
+    Tcap = (t0 + S + 15) // 8 * 8
+    k = torch.randn(B, S, Hkv, D, generator=g).to(dtype)          # [B,S,Hkv,D] as the reference hashes them
+    v = torch.randn(B, S, Hkv, D, generator=g).to(dtype)
+    planes = torch.randn(L, P, D, generator=g)
+    NW = orc.words_per_key(L, P)
+    codes = torch.full((B, Hkv, NW, Tcap), -1, dtype=torch.int32, device=dev)
+    vn = torch.full((B, Hkv, Tcap), -1.0, dtype=torch.float16, device=dev)
+    pw = hash_cache.permute_planes(planes.to(dev))
+    assert torch.equal(pw.cpu(), orc.permute_planes_for_words(planes.to(torch.bfloat16)))
+    hash_cache.hash_keys_into(k.to(dev), v.to(dev), pw, codes, vn, L, P, t0=t0, layout="bshd")
+    got = hash_cache.unpack_codes(codes, L, P, t0, S, layout="bthl").cpu()      # [B,S,Hkv,L]
+    # untouched cache positions stay untouched
+    assert (codes[..., :t0] == -1).all() and (codes[..., t0 + S:] == -1).all()
+    assert (vn[..., :t0] == -1).all() and (vn[..., t0 + S:] == -1).all()
+    # the kernel contracts bf16 operands with fp32 accumulation
+    kb, pb = k.to(torch.bfloat16), planes.to(torch.bfloat16)
+    proj = orc.projections_f64(kb, pb)                                            # [B,S,Hkv,L,P]
+    want_bits = proj >= 0
+    got_bits = ((got.long().unsqueeze(-1) >> torch.arange(P - 1, -1, -1)) & 1).bool()
+    margin = 1e-3 * kb.double().norm(dim=-1)[..., None, None] * pb.double().norm(dim=-1)
+    decided = proj.abs() > margin
+    assert decided.float().mean() > 0.98
+    assert torch.equal(got_bits[decided], want_bits[decided])
+    # and against the reference's own formulation run in the input dtype, on the same decided bits
+    ref_codes = orc.hard_hash_keys(k, planes)                                      # int16 [B,S,Hkv,L]
+    ref_bits = ((ref_codes.long().unsqueeze(-1) >> torch.arange(P - 1, -1, -1)) & 1).bool()
+    assert torch.equal(got_bits[decided], ref_bits[decided])
+    # value norm: fp32 reduce, fp16 store (1 ulp of fp16 for the different summation order)
+    want_vn = orc.value_norm(v).permute(0, 2, 1)                                   # [B,Hkv,S]
+    got_vn = vn[..., t0:t0 + S].cpu()
+    assert torch.allclose(got_vn.float(), want_vn.float(), rtol=1e-3, atol=0)
+
+
+def test_hash_identity_planes_and_sign_flip(dev):
+    """planes = +-unit vectors -> bits are the sign bits of key coordinates;
+    hash(a*k) = hash(k) for a > 0; hash(-k) = ~hash(k) when no projection is 0."""
+    L, P, D, S = 8, 10, 128, 200
+    g = torch.Generator().manual_seed(1)
+    planes = torch.zeros(L, P, D)
+    coord = torch.randperm(D, generator=g)[:L * P].view(L, P)
+    sign = torch.where(torch.rand(L, P, generator=g) > 0.5, 1.0, -1.0)
+    planes.view(-1, D).scatter_(1, coord.view(-1, 1), sign.view(-1, 1))
+    k = torch.randn(1, S, 1, D, generator=g).to(torch.bfloat16)
+    NW = orc.words_per_key(L, P)
+    pw = hash_cache.permute_planes(planes.to(dev))
+
+    def run(x):
+        codes = torch.zeros((1, 1, NW, 208), dtype=torch.int32, device=dev)
+        hash_cache.hash_keys_into(x.to(dev), None, pw, codes, None, L, P, layout="bshd")
+        return hash_cache.unpack_codes(codes, L, P, 0, S, layout="bthl").cpu()
+
+    got = run(k)
+    bits = (k.float()[0, :, 0][:, coord] * sign) >= 0                      # [S,L,P]
+    assert torch.equal(got[0, :, 0], orc.pack_bits(bits))
+    assert torch.equal(run(k * 3), got)
+    assert torch.equal(run(-k)[0, :, 0].int(), (~got[0, :, 0].int()) & ((1 << P) - 1))
+
+
+def test_pack_unpack_round_trip(dev):
+    g = torch.Generator().manual_seed(2)
+    for L, P in ((60, 10), (32, 8), (5, 16), (33, 1), (7, 11)):
+        T = 301
+        codes = _rand_codes(g, 2, 3, L, T, min(P, 15))
+        NW = orc.words_per_key(L, P)
+        words = torch.zeros((2, 3, NW, 304), dtype=torch.int32, device=dev)
+        hash_cache.pack_codes_into(codes.to(dev), words, P, t0=2)
+        want = orc.pack_code_words(codes.numpy(), P)
+        assert np.array_equal(words[..., 2:2 + T].cpu().numpy().view(np.uint32), want)
+        back = hash_cache.unpack_codes(words, L, P, 2, T).cpu()
+        assert torch.equal(back, codes)
+
+
+# ---------------------------------------------------------------- whole step
+@pytest.mark.parametrize("name,T", [("c1", 4096), ("c2", 8192)])
+def test_decode_step_end_to_end(dev, name, T):
+    """hash -> score -> select -> attend on a BASELINE configuration (C2 with a
+    shorter context so the oracle finishes in seconds)."""
+    w = scaled(WORKLOADS[name], T=T, M=min(WORKLOADS[name].M, T // 8))
+    inp = make_inputs(w, device="cpu")
+    cache = hash_cache.SocketHashCache(w.B, T, w.Hkv, w.D, w.L, w.P, dtype=w.dtype, device=dev)
+    cache.set_planes(inp.planes)
+    cache.append(0, inp.k.permute(0, 2, 1, 3).to(dev), inp.v.permute(0, 2, 1, 3).to(dev))
+    out, scores, sl, ln = hash_cache.sparse_decode_step(
+        inp.q.to(dev), inp.q_probs.to(dev), cache.k_cache, cache.v_cache, cache.codes, cache.v_norm,
+        T, w.P, w.sink, w.window, w.M, return_details=True)
+    # oracle on the device's own codes / norms (hash parity is covered separately)
+    codes = hash_cache.unpack_codes(cache.codes, w.L, w.P, 0, T).cpu()
+    vnorm = cache.v_norm[..., :T].cpu()
+    allowed = torch.ones(w.B, w.Hq, T, dtype=torch.bool)
+    wl, wn, wscores = orc.build_sparse_list_decode(
+        inp.q_probs, codes.repeat_interleave(w.G, 1), vnorm.repeat_interleave(w.G, 1), allowed,
+        w.sink, w.window, w.M, return_scores=True)
+    rel = ((scores.cpu() - wscores).abs() / wscores.abs().clamp_min(1e-30)).max()
+    assert rel <= 1e-5
+    # top-k exact on the device's own scores, and (scores being equal) on the oracle's
+    wl2 = torch.cat([wl[..., :wl.shape[-1] - w.M], orc.topk_lower_index_first(scores.cpu(), w.M).int()], -1)
+    assert torch.equal(sl.cpu(), wl2) and torch.equal(ln.cpu(), wn)
+    assert torch.equal(sl.cpu(), wl)
+    want = orc.sparse_attend_textbook(inp.q, inp.k, inp.v, wl, wn)
+    assert (out.cpu().double() - want).abs().max() <= ATOL[w.dtype]
+    # planted heavy keys are found: most of them are inside the selected set
+    # (a sanity check of the whole chain, not a parity bar)
+    assert out.dtype == w.dtype
