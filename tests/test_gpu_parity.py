@@ -77,7 +77,7 @@ def test_score_packed_collision_counts(dev):
     Tcap = 3008
     vn = torch.zeros(B, Hkv, Tcap, dtype=torch.float16); vn[..., :T] = v_norm
     got = hash_cache.score_packed(q_probs.to(dev), _packed_cache(codes, P, Tcap, dev), vn.to(dev), T, P).cpu()
-    count = (codes.long().unsqueeze(1) == qcode.unsqueeze(-1)).sum(2)   # [B,Hq,T]
+    count = (codes[:, 0].long().unsqueeze(1) == qcode.unsqueeze(-1)).sum(2)   # [B,Hq,T]
     assert torch.equal(got, count.float() * 2.0)
     assert got[0, 2, 17] == 120.0 and got[0, 0, 99] >= 60.0
 
