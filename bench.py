@@ -1,0 +1,384 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-decode hot path on one MI355X.
+
+A step is one decode step of one attention layer on synthetic inputs of the
+configured shape, resident in HBM before timing starts: hash the newly appended
+key of every (sequence, kv head), score every cached key, select the top-k +
+sink + window list, and attend over the listed rows.  The default workload is
+configuration 3 (batch 4, 32/8 heads, head dim 128, 131072-token bf16 cache,
+L=60 x P=10, top-k 2048 + 4 sink + 256 window).
+
+Prints one JSON line: `value` is microseconds per layer per step for the sparse
+path; `roofline` prices the scorer (the kernel moving the most bytes) against
+HBM peak; `kernels` does the same for every kernel; `dense` is the dense
+flash-decode comparator on the same GPU; `cpu_baseline` is the CPU oracle timed
+on the host's cores on a slice of the same workload.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c5]
+                  [--only score|select|attend|hash|dense] [--no-cpu] [--no-parity]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+# HBM bytes per launch of the scorer from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of `bench.py --only score` (see profiles/), keyed by workload; None until
+# a counter run for that workload has been recorded there.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(w, lens=None, budgets=None):
+    """Per-launch algorithmic bytes of each kernel on the packed format."""
+    cpw = 32 // w.P
+    wc = 4 * ((w.L + cpw - 1) // cpw)
+    G = w.Hq // w.Hkv
+    if lens is None:
+        tok = w.B * w.T
+        sel = w.B * w.Hq * (4 * w.T + 4 * w.M)
+        kt = w.B * (w.sink + w.window + w.M)
+    else:
+        tok = int(lens.sum())
+        sel = int((w.Hq * (4 * lens.long() + 4 * budgets.long())).sum())
+        kt = int((w.sink + w.window + budgets.long()).sum())
+    return {
+        "hash": w.B * w.Hkv * w.new_keys * (2 * 2 * w.D + wc + 2),
+        "score": w.Hkv * tok * (wc + 2 + 4 * G),
+        "score_f32": w.Hkv * tok * (wc + 2 + 4 * G),
+        "score_f32_table": w.Hkv * tok * (wc + 2 + 4 * G),
+        "select": sel,
+        "attend": w.Hq * kt * (4 * w.D + 4) + w.B * w.Hq * 4 * w.D,
+        "dense": w.Hkv * tok * 4 * w.D,
+    }
+
+
+def time_launches(fn, iters, warmup=3):
+    """Average duration in microseconds of `fn` (which enqueues on torch's current
+    stream) measured with HIP events recorded on that same stream."""
+    for _ in range(warmup):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) * 1000.0 / iters
+
+
+def copy_ceiling_gbs(dev):
+    """Measured device-to-device copy rate (read + write bytes) of a 1 GiB buffer."""
+    n = 1 << 28
+    a = torch.empty(n, dtype=torch.float32, device=dev).normal_()
+    b = torch.empty_like(a)
+    us = time_launches(lambda: b.copy_(a), 10)
+    del a, b
+    return 2 * n * 4 / us / 1e3
+
+
+def cpu_baseline(w, inp_cpu, codes_cpu, vnorm_cpu, seconds_budget=20.0):
+    """The CPU oracle on a slice of the workload: sequence 0, the first two kv
+    heads (2*G query heads), full context; scaled to the whole layer."""
+    from oracle import socket_oracle as orc
+
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    G = w.Hq // w.Hkv
+    nkv = min(2, w.Hkv)
+    T = int(inp_cpu["len0"])
+    M = int(inp_cpu["m0"])
+    q = inp_cpu["q"][:1, :nkv * G]
+    qp = inp_cpu["q_probs"][:1, :nkv * G].float().contiguous()
+    k = inp_cpu["k"][:1, :nkv, :T]
+    v = inp_cpu["v"][:1, :nkv, :T]
+    codes = codes_cpu[:1, :nkv, :, :T].repeat_interleave(G, 1)
+    vn = vnorm_cpu[:1, :nkv, :T].repeat_interleave(G, 1)
+    allowed = torch.ones(1, nkv * G, T, dtype=torch.bool)
+
+    def once():
+        t0 = time.perf_counter()
+        scores = orc.collision_score(qp, codes, allowed, vn.float())
+        t1 = time.perf_counter()
+        heavy = orc.topk_lower_index_first(scores, M).to(torch.int32)
+        base = torch.from_numpy(orc.base_indices(T, w.sink, w.window)).view(1, 1, -1).expand(1, nkv * G, -1)
+        sl = torch.cat([base, heavy], -1).contiguous()
+        ln = torch.full((1, nkv * G), sl.shape[-1], dtype=torch.int32)
+        t2 = time.perf_counter()
+        orc.sparse_attend_textbook(q, k, v, sl, ln)
+        t3 = time.perf_counter()
+        return t1 - t0, t2 - t1, t3 - t2
+
+    once()
+    reps = []
+    t_start = time.perf_counter()
+    while len(reps) < 5 or (time.perf_counter() - t_start < seconds_budget and len(reps) < 15):
+        reps.append(once())
+    med = [statistics.median(r[i] for r in reps) for i in range(3)]
+    # keys scored by the whole layer / keys scored by the sample
+    scale = (w.Hkv * float(inp_cpu["tok_total"])) / (nkv * T)
+    total_us = sum(med) * 1e6 * scale
+    return {
+        "value": round(total_us, 1),
+        "unit": "us/layer/step",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"sequence 0, {nkv} of {w.Hkv} kv heads ({nkv * G} query heads), context {T}, "
+                  f"median of {len(reps)} reps, scaled x{scale:.2f} to the whole layer",
+        "stage_us_scaled": {"score": round(med[0] * 1e6 * scale, 1), "select": round(med[1] * 1e6 * scale, 1),
+                            "attend": round(med[2] * 1e6 * scale, 1)},
+        "cpu_model": _cpu_model(),
+    }
+
+
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c5"])
+    ap.add_argument("--only", default=None, choices=["score", "score_f32", "select", "attend", "hash", "dense"])
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-parity", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every (sequence, kv head) "
+              "pair is independent; see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(2)
+
+    from socket_amd import hash_cache, socket_kernels, sparse
+    from socket_amd.workloads import WORKLOADS, make_inputs
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = WORKLOADS[args.workload]
+    t_gen = time.perf_counter()
+    inp = make_inputs(w, device=dev, device_rng=True)
+    torch.cuda.synchronize()
+    t_gen = time.perf_counter() - t_gen
+
+    B, Hq, Hkv, D, T = w.B, w.Hq, w.Hkv, w.D, w.T
+    NW = hash_cache.words_per_key(w.L, w.P)
+    Tcap = (T + 7) // 8 * 8
+    codes = torch.zeros((B, Hkv, NW, Tcap), dtype=torch.int32, device=dev)
+    v_norm = torch.zeros((B, Hkv, Tcap), dtype=torch.float16, device=dev)
+    planes_words = hash_cache.permute_planes(inp.planes)
+    lens, budgets = inp.lens, inp.budgets
+    abytes = algorithmic_bytes(w, None if lens is None else lens.cpu(), None if budgets is None else budgets.cpu())
+
+    # ---- prefill hash of the whole cache (K1 at scale) -----------------------------
+    def prefill_hash():
+        hash_cache.hash_keys_into(inp.k, inp.v, planes_words, codes, v_norm, w.L, w.P, t0=0, layout="bhsd")
+
+    prefill_us = time_launches(prefill_hash, 3, warmup=1)
+    rows = B * Hkv * T
+    prefill_flops = 2.0 * rows * D * NW * 32          # columns actually contracted (incl. pad bits)
+    prefill_bytes = rows * (2 * 2 * D + 4 * NW + 2)
+    hash_report = {
+        "prefill_ms": round(prefill_us / 1e3, 3),
+        "rows": rows,
+        "mfma_tflops": round(prefill_flops / prefill_us / 1e6, 1),
+        "mfma_frac": round(prefill_flops / prefill_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "hbm_gbs": round(prefill_bytes / prefill_us / 1e3, 1),
+        "hbm_frac": round(prefill_bytes / prefill_us / 1e3 / HBM_PEAK_GBS, 4),
+    }
+
+    # ---- the step --------------------------------------------------------------------
+    pitch = (T + 3) // 4 * 4
+    scores_buf = torch.empty((B, Hq, pitch), dtype=torch.float32, device=dev)
+    new_pos = None
+    if lens is not None:
+        new_pos = (lens - w.new_keys).to(torch.int32)
+
+    def k_hash():
+        # the newly appended key(s) of every (sequence, kv head) land on the last
+        # position(s), so the context length is the same every step
+        hash_cache.hash_keys_into(inp.k_new, inp.v_new, planes_words, codes, v_norm, w.L, w.P,
+                                  t0=T - w.new_keys, pos_b=new_pos, layout="bshd")
+
+    # the soft-hash table in the dtype the model produces it in: the reference's
+    # soft_hash runs in the model dtype (GPT-FAST/model.py:392-401), bf16 here
+    q_table = inp.q_probs.to(torch.bfloat16) if w.dtype == torch.bfloat16 else inp.q_probs
+    q_table_f32 = q_table.float()
+
+    def k_score():
+        return hash_cache.score_packed(q_table, codes, v_norm, T, w.P, lens=lens, out=scores_buf)
+
+    def k_score_f32():
+        return hash_cache.score_packed(q_table_f32, codes, v_norm, T, w.P, lens=lens, out=scores_buf)
+
+    def k_select(scores):
+        return sparse.select_list(scores, w.sink, w.window, w.M, lens=lens, budgets=budgets)
+
+    def k_attend(sl, ln):
+        return socket_kernels.sparse_attention_fwd(inp.q, inp.k, inp.v, sl, ln)
+
+    dense_lens = lens if lens is not None else torch.full((B,), T, dtype=torch.int32, device=dev)
+
+    def k_dense():
+        return socket_kernels.dense_decode_fwd(inp.q, inp.k, inp.v, dense_lens)
+
+    def step():
+        k_hash()
+        s = k_score()
+        sl, ln = k_select(s)
+        return k_attend(sl, ln)
+
+    scores = k_score()
+    sl, ln = k_select(scores)
+    out = k_attend(sl, ln)
+    torch.cuda.synchronize()
+
+    iters = max(args.steps, 1)
+    if args.only:
+        fn = {"score": k_score, "score_f32": k_score_f32, "select": lambda: k_select(scores), "attend": lambda: k_attend(sl, ln),
+              "hash": k_hash, "dense": k_dense}[args.only]
+        us = time_launches(fn, iters, warmup=args.warmup)
+        print(json.dumps({"only": args.only, "workload": w.name, "us": round(us, 2),
+                          "gbs": round(abytes[args.only] / us / 1e3, 1), "iters": iters}))
+        return
+
+    # ---- parity gates on the full-size run (device-side checks, not timed) --------------
+    parity = None
+    if not args.no_parity:
+        parity = {}
+        s0 = scores[0, :8]
+        n0 = T if lens is None else int(lens[0])
+        m0 = w.M if budgets is None else int(budgets[0])
+        order = torch.sort(s0[:, :n0], dim=-1, descending=True, stable=True).indices[:, :m0].to(torch.int32)
+        nbase = int(ln[0, 0]) - m0
+        parity["topk_exact_rows_checked"] = 8
+        parity["topk_exact"] = bool(torch.equal(sl[0, :8, nbase:nbase + m0], order))
+        # attention vs an fp32 gather-softmax over the same list, one sequence
+        idx = sl[0, :, :int(ln[0, 0])].long()
+        G = Hq // Hkv
+        kk = inp.k[0].repeat_interleave(G, 0).gather(1, idx.unsqueeze(-1).expand(-1, -1, D)).float()
+        vv = inp.v[0].repeat_interleave(G, 0).gather(1, idx.unsqueeze(-1).expand(-1, -1, D)).float()
+        att = torch.softmax((kk @ inp.q[0].float().unsqueeze(-1)).squeeze(-1) / D ** 0.5, -1)
+        ref = (att.unsqueeze(1) @ vv).squeeze(1)
+        parity["attend_max_abs_err"] = float((out[0].float() - ref).abs().max())
+        # scores vs an fp32 gather-sum in table order on the unpacked codes, one kv head
+        c16 = hash_cache.unpack_codes(codes[:1, :1].contiguous(), w.L, w.P, 0, n0).long()[0, 0]   # [L,T]
+        acc = torch.zeros(n0, dtype=torch.float32, device=dev)
+        for l in range(w.L):
+            acc = acc + q_table_f32[0, 0, l].gather(0, c16[l])
+        ref_s = acc * v_norm[0, 0, :n0].float()
+        parity["score_max_rel_err"] = float(((scores[0, 0, :n0] - ref_s).abs() / ref_s.abs().clamp_min(1e-30)).max())
+        del kk, vv, c16
+
+    # ---- per-kernel timings ------------------------------------------------------------------
+    per = {
+        "hash": time_launches(k_hash, iters),
+        "score": time_launches(k_score, iters),
+        "score_f32_table": time_launches(k_score_f32, iters),
+        "select": time_launches(lambda: k_select(scores), iters),
+        "attend": time_launches(lambda: k_attend(sl, ln), iters),
+        "dense": time_launches(k_dense, max(iters // 2, 5)),
+    }
+    kernels = {k: {"us": round(v, 2), "algorithmic_MB": round(abytes[k] / 1e6, 2),
+                   "gbs": round(abytes[k] / v / 1e3, 1), "hbm_frac": round(abytes[k] / v / 1e3 / HBM_PEAK_GBS, 4)}
+               for k, v in per.items()}
+
+    # ---- the timed region: exactly K steps -----------------------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    sparse_us = ms_per_step * 1e3
+    sparse_bytes = abytes["score"] + abytes["select"] + abytes["attend"]
+    kernel_sum_us = per["score"] + per["select"] + per["attend"]
+
+    ceiling = copy_ceiling_gbs(dev)
+
+    result = {
+        "metric": "sparse-attn us/layer/step at 128k ctx (score+select+attend+hash-append), % of HBM peak"
+                  if w.name == "c3" else "sparse-attn us/layer/step (score+select+attend+hash-append), % of HBM peak",
+        "value": round(sparse_us, 2),
+        "unit": "us/layer/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: B{B} Hq{Hq}/Hkv{Hkv} D{D} T{T} bf16 KV cache, L{w.L}xP{w.P} packed codes, "
+                               f"{str(q_table.dtype).split('.')[-1]} soft-hash table, "
+                               f"top-k {w.M} + sink {w.sink} + window {w.window}"
+                               + (", ragged lengths" if w.ragged else ""),
+                   "layers_timed": 1, "new_keys_hashed_per_step": B * Hkv * w.new_keys},
+        "roofline": {"kernel": "score_packed_kernel", "bound": "hbm",
+                     "achieved": round(abytes["score"] / per["score"] / 1e3, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(abytes["score"] / per["score"] / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(w.name)},
+        "kernels": kernels,
+        "sparse_total": {"algorithmic_MB": round(sparse_bytes / 1e6, 2), "kernel_sum_us": round(kernel_sum_us, 2),
+                         "hbm_frac_of_kernel_sum": round(sparse_bytes / kernel_sum_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "hbm_frac_of_step": round(sparse_bytes / sparse_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "speedup_vs_dense": round(per["dense"] / sparse_us, 3),
+                         "attend_block_seq": None},
+        "hash_prefill": hash_report,
+        "copy_ceiling_gbs": round(ceiling, 1),
+        "parity": parity,
+        "wall_ms_timed_region": round(wall_ms, 2),
+        "input_generation_s": round(t_gen, 1),
+    }
+    from socket_amd._lib import lib
+    result["sparse_total"]["attend_block_seq"] = lib().socket_sparse_attention_block_seq(B, Hq, sl.shape[-1])
+
+    if not args.no_cpu:
+        n0 = T if lens is None else int(lens[0])
+        m0 = w.M if budgets is None else int(budgets[0])
+        nkv = min(2, Hkv)
+        G = Hq // Hkv
+        inp_cpu = {"q": inp.q.cpu(), "q_probs": inp.q_probs[:1, :nkv * G].cpu(), "k": inp.k[:1, :nkv].cpu(),
+                   "v": inp.v[:1, :nkv].cpu(), "len0": n0, "m0": m0,
+                   "tok_total": B * T if lens is None else int(lens.sum())}
+        codes_cpu = hash_cache.unpack_codes(codes[:1, :nkv].contiguous(), w.L, w.P, 0, n0).cpu()
+        result["cpu_baseline"] = cpu_baseline(w, inp_cpu, codes_cpu, v_norm[:1, :nkv].cpu())
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -109,13 +109,15 @@ int socket_pack_codes(const int16_t* in, int64_t in_stride_b, int64_t in_stride_
  *   scores[b,h,t] = t < len(b) ? (sum_{l<L} q_probs[b,h,l,code_l(b,kv,t)]) * v_norm[b,kv,t] : -inf
  * with the sum taken over l ascending in fp32 (the order of the loop at
  * GPT-FAST/kernels/soft_hash_collision.cu:45-53), len(b) = lens ? lens[b] : T.
- * q_probs: fp32 [B,Hq,L,R] contiguous (q_dtype must be SOCKET_F32).
+ * q_probs: [B,Hq,L,R] contiguous, q_dtype SOCKET_F32 or SOCKET_BF16 (bf16 values are
+ * widened exactly, as the reference's q_probs.float() does).
  * scores: fp32, row (b,h) at scores + (b*Hq+h)*score_stride.
  * Codes are read once per kv head, not once per query head.
  * Replaces the relayout at GPT-FAST/model.py:490-509 and the scorer call at
  * GPT-FAST/kernels/sparse.py:42-55.
  * Requires Tcap % 4 == 0, score_stride % 4 == 0, 16-byte aligned pointers,
- * R a power of two, 2^P <= R, G <= 8. */
+ * R a power of two >= 8, 2^P <= R, G <= 8, and the tables of one packed word
+ * (32/P tables x R entries x G values) must fit in LDS. */
 int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
                         const uint16_t* v_norm, const int32_t* lens, float* scores,
                         int B, int Hq, int Hkv, int L, int P, int R, int T, int64_t Tcap,

@@ -12,7 +12,9 @@
 //    interleaved ([table][bucket][g]), so one LDS gather returns the terms of
 //    all G heads.  Partial sums stay in registers across slices, which keeps the
 //    reference's summation order.  Codes are read once per kv head, 16 bytes per
-//    lane, fully coalesced.
+//    lane, fully coalesced, one word ahead of their use.  The table may be fp32
+//    or bf16 (a bf16 soft-hash producer loses nothing and halves the LDS bytes
+//    per gather, which is what bounds this kernel).
 //  * collision_i16_kernel: the reference's own operand layout (int16 codes per
 //    query head), for drop-in callers.
 #include "socket_common.h"
@@ -22,27 +24,139 @@ namespace {
 // ---------------------------------------------------------------------------
 // native packed scorer
 // ---------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+
+struct TabF32 {
+  typedef float elem;
+  static constexpr int kEnum = SOCKET_F32;
+};
+struct TabBF16 {
+  typedef uint16_t elem;
+  static constexpr int kEnum = SOCKET_BF16;
+};
+
+// acc[g] += entry[g] for one LDS entry of GP table elements.
 template <int GP>
-struct LdsEntry;  // GP floats, stored with the widest LDS access available
-template <>
-struct LdsEntry<1> { float v[1]; };
-template <>
-struct __attribute__((aligned(8))) LdsEntry<2> { float v[2]; };
-template <>
-struct __attribute__((aligned(16))) LdsEntry<4> { float v[4]; };
-template <>
-struct __attribute__((aligned(16))) LdsEntry<8> { float v[8]; };
+__device__ __forceinline__ void accumulate_entry(float* acc, const float* entry_lds) {
+  if (GP == 1) {
+    acc[0] += entry_lds[0];
+  } else if (GP == 2) {
+    const float2 e = *reinterpret_cast<const float2*>(entry_lds);
+    acc[0] += e.x;
+    acc[1] += e.y;
+  } else {
+#pragma unroll
+    for (int v = 0; v < GP / 4; ++v) {
+      const float4 e = reinterpret_cast<const float4*>(entry_lds)[v];
+      acc[4 * v + 0] += e.x;
+      acc[4 * v + 1] += e.y;
+      acc[4 * v + 2] += e.z;
+      acc[4 * v + 3] += e.w;
+    }
+  }
+}
+
+// bf16 entries: widening to fp32 and the add are one v_dot2_f32_bf16 per head,
+// acc += lo * 1 + hi * 0 (or the other way round).  The dot unit's final rounding
+// is not always that of the fp32 adder, so a sum of L terms can differ from the
+// sequential fp32 sum in the last few ulp (measured below 2e-6 relative; the
+// fp32-table path uses plain adds and reproduces the reference sum exactly).  The
+// (1,0) / (0,1) selectors are passed in as run-time values held in scalar
+// registers: written as literals the compiler folds them into an inline operand
+// constant, and with that encoding the instruction picked the wrong half.
+struct Bf16Select {
+  uint32_t lo, hi;  // bf16 pairs (1.0, 0.0) and (0.0, 1.0)
+};
+__device__ __forceinline__ float add_bf16(float acc, uint32_t pair, uint32_t selector) {
+  bf16x2_t a, one;
+  __builtin_memcpy(&a, &pair, 4);
+  __builtin_memcpy(&one, &selector, 4);
+  return __builtin_amdgcn_fdot2_f32_bf16(a, one, acc, false);
+}
+
+template <int GP>
+__device__ __forceinline__ void accumulate_entry(float* acc, const float* entry_lds, const Bf16Select&) {
+  accumulate_entry<GP>(acc, entry_lds);
+}
+
+template <int GP>
+__device__ __forceinline__ void accumulate_entry(float* acc, const uint16_t* entry_lds, const Bf16Select& sel) {
+  if (GP == 1) {
+    acc[0] += bf16_bits_to_f32(entry_lds[0]);
+  } else if (GP == 2) {
+    const uint32_t e = *reinterpret_cast<const uint32_t*>(entry_lds);
+    acc[0] = add_bf16(acc[0], e, sel.lo);
+    acc[1] = add_bf16(acc[1], e, sel.hi);
+  } else if (GP == 4) {
+    const uint2 e = *reinterpret_cast<const uint2*>(entry_lds);
+    acc[0] = add_bf16(acc[0], e.x, sel.lo);
+    acc[1] = add_bf16(acc[1], e.x, sel.hi);
+    acc[2] = add_bf16(acc[2], e.y, sel.lo);
+    acc[3] = add_bf16(acc[3], e.y, sel.hi);
+  } else {
+    const uint4 e = *reinterpret_cast<const uint4*>(entry_lds);
+    acc[0] = add_bf16(acc[0], e.x, sel.lo);
+    acc[1] = add_bf16(acc[1], e.x, sel.hi);
+    acc[2] = add_bf16(acc[2], e.y, sel.lo);
+    acc[3] = add_bf16(acc[3], e.y, sel.hi);
+    acc[4] = add_bf16(acc[4], e.z, sel.lo);
+    acc[5] = add_bf16(acc[5], e.z, sel.hi);
+    acc[6] = add_bf16(acc[6], e.w, sel.lo);
+    acc[7] = add_bf16(acc[7], e.w, sel.hi);
+  }
+}
+
+// One 16-byte vector of table elements per head (GP heads) -> the same elements
+// regrouped entry-major: out word stream holds entry e = {head 0..GP-1}.
+template <int GP, class TT>
+__device__ __forceinline__ void interleave_heads(const uint4 (&x)[GP], uint4 (&out)[GP]) {
+  constexpr int EPV = 16 / (int)sizeof(typename TT::elem);
+  uint32_t xw[GP][4], ow[4 * GP];
+#pragma unroll
+  for (int g = 0; g < GP; ++g) {
+    xw[g][0] = x[g].x;
+    xw[g][1] = x[g].y;
+    xw[g][2] = x[g].z;
+    xw[g][3] = x[g].w;
+  }
+  if (sizeof(typename TT::elem) == 4) {
+#pragma unroll
+    for (int e = 0; e < EPV; ++e)
+#pragma unroll
+      for (int g = 0; g < GP; ++g) ow[e * GP + g] = xw[g][e];
+  } else if (GP == 1) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) ow[k] = xw[0][k];
+  } else {
+#pragma unroll
+    for (int e = 0; e < EPV; ++e)
+#pragma unroll
+      for (int g = 0; g < GP; g += 2) {
+        const uint32_t lo = (xw[g][e >> 1] >> (16 * (e & 1))) & 0xffffu;
+        const uint32_t hi = (xw[g + 1][e >> 1] >> (16 * (e & 1))) & 0xffffu;
+        ow[(e * GP + g) >> 1] = lo | (hi << 16);
+      }
+  }
+#pragma unroll
+  for (int v = 0; v < GP; ++v) out[v] = make_uint4(ow[4 * v], ow[4 * v + 1], ow[4 * v + 2], ow[4 * v + 3]);
+}
 
 // PT: P known at compile time (0 = use the runtime value).
-template <int GP, int KT4, int THREADS, int PT>
+// The table slice of the tables held by `chunk_words` packed words sits in LDS;
+// with two LDS buffers the next slice is fetched into registers while the
+// current one is being gathered from, and there is one barrier per slice.
+template <int GP, class TT, int KT4, int THREADS, int PT>
 __global__ __launch_bounds__(THREADS) void score_packed_kernel(
-    const float* __restrict__ q_probs, const uint32_t* __restrict__ codes,
+    const typename TT::elem* __restrict__ q_probs, const uint32_t* __restrict__ codes,
     const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens,
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
-    int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int n_pairs, int n_tiles,
-    int xcd_remap) {
+    int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
+    int n_tiles, int xcd_remap, uint32_t bf16_one) {
+  typedef typename TT::elem TE;
+  const Bf16Select sel{bf16_one, bf16_one << 16};
+  constexpr int EPV = 16 / (int)sizeof(TE);   // table elements per 16-byte vector
+  constexpr int SL = 1024 / THREADS;           // staging slots (one 16-byte vector per head) per lane
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  LdsEntry<GP>* table = reinterpret_cast<LdsEntry<GP>*>(lds_raw);
 
   const int P = PT ? PT : P_rt;
   const int cpw = 32 / P;
@@ -70,7 +184,9 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   const int len = lens ? min(lens[b], T) : T;
 
   const uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
-  const float* qp_pair = q_probs + ((int64_t)(b * Hq + kvh * G)) * L * R;
+  const TE* qp_pair = q_probs + ((int64_t)(b * Hq + kvh * G)) * L * R;
+  const int chunk_tables = chunk_words * cpw;
+  const int chunk_elems = chunk_tables * R * GP;  // table elements per LDS buffer
 
   int tbase[KT4];
   bool live[KT4];
@@ -88,69 +204,107 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
 #pragma unroll
       for (int g = 0; g < GP; ++g) acc[j][i][g] = 0.f;
 
-  uint4 nxt[KT4];
+  // packed words of the lane's token groups; each is reloaded with the next word
+  // as soon as it has been consumed
+  uint4 ring[KT4];
 #pragma unroll
   for (int j = 0; j < KT4; ++j)
-    nxt[j] = live[j] ? *reinterpret_cast<const uint4*>(codes_pair + tbase[j]) : make_uint4(0, 0, 0, 0);
+    ring[j] = live[j] ? *reinterpret_cast<const uint4*>(codes_pair + tbase[j]) : make_uint4(0, 0, 0, 0);
 
-  for (int w0 = 0; w0 < NW; w0 += chunk_words) {
-    const int l0 = w0 * cpw;
-    const int nt = min(chunk_words * cpw, L - l0);
-    __syncthreads();  // gathers of the previous slice are done
-    {
-      // Slice fill: for each head g the nt*R floats are contiguous in q_probs.
-      const int n4 = (nt * R) >> 2;
-      const float* src = qp_pair + (int64_t)l0 * R;
-      for (int i4 = tid; i4 < n4; i4 += THREADS) {
-        float4 x[GP];
+  // slice staging: slot s covers table elements [s*EPV, (s+1)*EPV) of every head
+  uint4 stage[SL][GP];
+  auto stage_load = [&](int l0) {
+    const int nt = min(chunk_tables, L - l0);
+    const int nslots = (nt * R) / EPV;
+    const TE* src = qp_pair + (int64_t)l0 * R;
+#pragma unroll
+    for (int k = 0; k < SL; ++k) {
+      const int s = tid + k * THREADS;
+      if (s < nslots) {
 #pragma unroll
         for (int g = 0; g < GP; ++g)
-          x[g] = (g < G) ? *reinterpret_cast<const float4*>(src + (int64_t)g * L * R + 4 * i4)
-                         : make_float4(0.f, 0.f, 0.f, 0.f);
-        LdsEntry<GP> e[4];
-#pragma unroll
-        for (int g = 0; g < GP; ++g) {
-          e[0].v[g] = x[g].x;
-          e[1].v[g] = x[g].y;
-          e[2].v[g] = x[g].z;
-          e[3].v[g] = x[g].w;
-        }
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) table[4 * i4 + rr] = e[rr];
+          stage[k][g] = (g < G) ? *reinterpret_cast<const uint4*>(src + (int64_t)g * L * R + (int64_t)s * EPV)
+                                : make_uint4(0, 0, 0, 0);
       }
     }
-    __syncthreads();
+  };
+  auto stage_store = [&](int l0, int buf) {
+    const int nt = min(chunk_tables, L - l0);
+    const int nslots = (nt * R) / EPV;
+    uint4* dst = reinterpret_cast<uint4*>(lds_raw + (size_t)buf * chunk_elems * sizeof(TE));
+#pragma unroll
+    for (int k = 0; k < SL; ++k) {
+      const int s = tid + k * THREADS;
+      if (s < nslots) {
+        uint4 o[GP];
+        interleave_heads<GP, TT>(stage[k], o);
+#pragma unroll
+        for (int v = 0; v < GP; ++v) dst[(size_t)s * GP + v] = o[v];
+      }
+    }
+  };
 
+  const bool staged = nbuf == 2;
+  if (staged) {
+    stage_load(0);
+    stage_store(0, 0);
+    __syncthreads();
+  }
+
+  int chunk = 0;
+  for (int w0 = 0; w0 < NW; w0 += chunk_words, ++chunk) {
+    const int l0 = w0 * cpw;
+    const int buf = staged ? (chunk & 1) : 0;
+    const bool more = w0 + chunk_words < NW;
+    if (staged) {
+      if (more) stage_load(l0 + chunk_tables);
+    } else {
+      __syncthreads();  // gathers of the previous slice are done
+      const int nt = min(chunk_tables, L - l0);
+      const int nslots = (nt * R) / EPV;
+      const TE* src = qp_pair + (int64_t)l0 * R;
+      uint4* dst = reinterpret_cast<uint4*>(lds_raw);
+      for (int s = tid; s < nslots; s += THREADS) {
+        uint4 x[GP], o[GP];
+#pragma unroll
+        for (int g = 0; g < GP; ++g)
+          x[g] = (g < G) ? *reinterpret_cast<const uint4*>(src + (int64_t)g * L * R + (int64_t)s * EPV)
+                         : make_uint4(0, 0, 0, 0);
+        interleave_heads<GP, TT>(x, o);
+#pragma unroll
+        for (int v = 0; v < GP; ++v) dst[(size_t)s * GP + v] = o[v];
+      }
+      __syncthreads();
+    }
+
+    const TE* table = reinterpret_cast<const TE*>(lds_raw) + (size_t)buf * chunk_elems;
     const int wend = min(w0 + chunk_words, NW);
     for (int w = w0; w < wend; ++w) {
-      uint4 cur[KT4];
-#pragma unroll
-      for (int j = 0; j < KT4; ++j) cur[j] = nxt[j];
-      if (w + 1 < NW) {
-        const uint32_t* row = codes_pair + (int64_t)(w + 1) * Tcap;
-#pragma unroll
-        for (int j = 0; j < KT4; ++j)
-          if (live[j]) nxt[j] = *reinterpret_cast<const uint4*>(row + tbase[j]);
-      }
       const int ntw = min(cpw, L - w * cpw);
-      const int ent0 = (w - w0) * cpw * R;
+      const TE* tw = table + (size_t)(w - w0) * cpw * R * GP;
+      const uint32_t* next_row = codes_pair + (int64_t)(w + 1) * Tcap;
+      const bool has_next = w + 1 < NW;
 #pragma unroll
-      for (int jj = 0; jj < (PT ? 32 / PT : 32); ++jj) {
-        if (jj >= ntw) break;
-        const LdsEntry<GP>* tb = table + ent0 + jj * R;
-        const int sh = jj * P;
+      for (int j = 0; j < KT4; ++j) {
+        const uint32_t wv[4] = {ring[j].x, ring[j].y, ring[j].z, ring[j].w};
+        if (has_next && live[j]) ring[j] = *reinterpret_cast<const uint4*>(next_row + tbase[j]);
 #pragma unroll
-        for (int j = 0; j < KT4; ++j) {
-          const uint32_t wv[4] = {cur[j].x, cur[j].y, cur[j].z, cur[j].w};
+        for (int jj = 0; jj < (PT ? 32 / PT : 32); ++jj) {
+          if (jj >= ntw) break;
+          const TE* tb = tw + (size_t)jj * R * GP;
+          const int sh = jj * P;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const uint32_t code = (wv[i] >> sh) & code_mask;
-            const LdsEntry<GP> e = tb[code];
-#pragma unroll
-            for (int g = 0; g < GP; ++g) acc[j][i][g] += e.v[g];
+            accumulate_entry<GP>(acc[j][i], tb + (size_t)code * GP, sel);
           }
         }
       }
+    }
+
+    if (staged) {
+      if (more) stage_store(l0 + chunk_tables, buf ^ 1);
+      __syncthreads();
     }
   }
 
@@ -182,51 +336,87 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   }
 }
 
-template <int GP, int KT4, int THREADS, int PT>
-int launch_score_packed(const float* q_probs, const uint32_t* codes, const uint16_t* v_norm,
-                        const int32_t* lens, float* scores, int B, int Hq, int Hkv, int L, int P,
-                        int R, int T, int64_t Tcap, int64_t score_stride, hipStream_t stream) {
-  const SocketDeviceLimits& lim = socket_device_limits();
-  const int G = Hq / Hkv;
-  const int cpw = 32 / P;
-  const int NW = (L + cpw - 1) / cpw;
-  const size_t bytes_per_word = (size_t)cpw * R * GP * sizeof(float);
-  // Slice size: as many words as fit a third of the CU's LDS (three resident
-  // workgroups overlap one another's slice fills), at least one word.
-  size_t budget = (size_t)lim.max_lds_per_block / 3;
-  int chunk_words = (int)(budget / bytes_per_word);
-  if (chunk_words < 1) chunk_words = 1;
-  if (chunk_words > NW) chunk_words = NW;
-  const size_t lds_bytes = bytes_per_word * chunk_words;
-  if (lds_bytes > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
+struct ScoreArgs {
+  const void* q_probs;
+  const uint32_t* codes;
+  const uint16_t* v_norm;
+  const int32_t* lens;
+  float* scores;
+  int B, Hq, Hkv, L, P, R, T;
+  int64_t Tcap, score_stride;
+  hipStream_t stream;
+};
 
-  auto kern = score_packed_kernel<GP, KT4, THREADS, PT>;
+template <int GP, class TT, int KT4, int THREADS, int PT>
+int launch_score_packed(const ScoreArgs& a) {
+  typedef typename TT::elem TE;
+  const SocketDeviceLimits& lim = socket_device_limits();
+  const int G = a.Hq / a.Hkv;
+  const int cpw = 32 / a.P;
+  const int NW = (a.L + cpw - 1) / cpw;
+  constexpr int EPV = 16 / (int)sizeof(TE);
+  const size_t bytes_per_word = (size_t)cpw * a.R * GP * sizeof(TE);
+  const size_t slots_per_word = (size_t)cpw * a.R / EPV;
+  // Double-buffered when one word's tables fit twice in LDS and in the staging
+  // registers (1024 vector slots per workgroup); as many words per slice as that
+  // allows.  Otherwise a single buffer filled in place.
+  int nbuf = 2, chunk_words = 1;
+  if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && slots_per_word <= 1024) {
+    while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= (size_t)lim.max_lds_per_block / 2 &&
+           slots_per_word * (chunk_words + 1) <= 1024)
+      ++chunk_words;
+  } else {
+    nbuf = 1;
+    if (bytes_per_word > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
+  }
+  const size_t lds_bytes = bytes_per_word * chunk_words * nbuf;
+
+  auto kern = score_packed_kernel<GP, TT, KT4, THREADS, PT>;
   if (lds_bytes > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
       return SOCKET_ERR_LAUNCH;
   }
   constexpr int TW = THREADS * 4 * KT4;
-  const int n_tiles = (T + TW - 1) / TW;
-  const int n_pairs = B * Hkv;
+  const int n_tiles = (a.T + TW - 1) / TW;
+  const int n_pairs = a.B * a.Hkv;
   const int xcd_remap = (n_pairs % 8 == 0) ? 1 : 0;
   const int n_wg = n_pairs * n_tiles;
-  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, stream, q_probs, codes, v_norm,
-                     lens, scores, Hq, Hkv, G, L, P, R, T, Tcap, score_stride, NW, chunk_words,
-                     n_pairs, n_tiles, xcd_remap);
+  hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
+                     a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
+                     a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, xcd_remap, 0x3f80u);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }
 
-template <int GP, int KT4>
-int dispatch_p(const float* q_probs, const uint32_t* codes, const uint16_t* v_norm,
-               const int32_t* lens, float* scores, int B, int Hq, int Hkv, int L, int P, int R,
-               int T, int64_t Tcap, int64_t score_stride, hipStream_t stream) {
-#define SOCKET_SCORE_ARGS q_probs, codes, v_norm, lens, scores, B, Hq, Hkv, L, P, R, T, Tcap, score_stride, stream
-  if (P == 10) return launch_score_packed<GP, KT4, 512, 10>(SOCKET_SCORE_ARGS);
-  if (P == 8) return launch_score_packed<GP, KT4, 512, 8>(SOCKET_SCORE_ARGS);
-  return launch_score_packed<GP, KT4, 512, 0>(SOCKET_SCORE_ARGS);
-#undef SOCKET_SCORE_ARGS
+template <int GP, class TT, int KT4, int THREADS>
+int dispatch_p(const ScoreArgs& a) {
+  if (a.P == 10) return launch_score_packed<GP, TT, KT4, THREADS, 10>(a);
+  if (a.P == 8) return launch_score_packed<GP, TT, KT4, THREADS, 8>(a);
+  return launch_score_packed<GP, TT, KT4, THREADS, 0>(a);
+}
+
+// Tile size: the largest of 16384 / 4096 / 1024 tokens per workgroup that still
+// gives every CU a workgroup (the 16384-token tile keeps 16 tokens x G partial
+// sums per lane, which only fits the register file for G <= 4).
+template <int GP, class TT>
+int dispatch_tile(const ScoreArgs& a) {
+  const SocketDeviceLimits& lim = socket_device_limits();
+  const int64_t pairs = (int64_t)a.B * a.Hkv;
+  if constexpr (GP <= 4) {
+    if (pairs * ((a.T + 16383) / 16384) >= lim.cu_count) return dispatch_p<GP, TT, 4, 1024>(a);
+  }
+  if (pairs * ((a.T + 4095) / 4096) >= lim.cu_count) return dispatch_p<GP, TT, 2, 512>(a);
+  return dispatch_p<GP, TT, 1, 256>(a);
+}
+
+template <class TT>
+int dispatch_g(const ScoreArgs& a) {
+  const int G = a.Hq / a.Hkv;
+  if (G == 1) return dispatch_tile<1, TT>(a);
+  if (G == 2) return dispatch_tile<2, TT>(a);
+  if (G <= 4) return dispatch_tile<4, TT>(a);
+  return dispatch_tile<8, TT>(a);
 }
 
 // ---------------------------------------------------------------------------
@@ -300,30 +490,21 @@ extern "C" int socket_score_packed(const void* q_probs, int q_dtype, const uint3
                                    int B, int Hq, int Hkv, int L, int P, int R, int T,
                                    int64_t Tcap, int64_t score_stride, void* stream) {
   SOCKET_REQUIRE(q_probs && codes && v_norm && scores, SOCKET_ERR_NULL);
-  SOCKET_REQUIRE(q_dtype == SOCKET_F32, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(q_dtype == SOCKET_F32 || q_dtype == SOCKET_BF16, SOCKET_ERR_UNSUPPORTED);
   SOCKET_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0 && T > 0, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(Hq % Hkv == 0, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(P >= 1 && P <= 16, SOCKET_ERR_SHAPE);
-  SOCKET_REQUIRE(R >= (1 << P) && (R & (R - 1)) == 0 && R >= 4, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(R >= (1 << P) && (R & (R - 1)) == 0 && R >= 8, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(T <= Tcap && score_stride >= T, SOCKET_ERR_SHAPE);
-  SOCKET_REQUIRE((int64_t)B * Hkv * ((T + 2047) / 2048) < (1LL << 31), SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE((int64_t)B * Hkv * ((T + 1023) / 1024) < (1LL << 31), SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(Tcap % 4 == 0 && score_stride % 4 == 0, SOCKET_ERR_ALIGN);
   SOCKET_REQUIRE(socket_aligned16(q_probs) && socket_aligned16(codes) && socket_aligned16(v_norm) &&
                      socket_aligned16(scores),
                  SOCKET_ERR_ALIGN);
-  const int G = Hq / Hkv;
-  SOCKET_REQUIRE(G <= 8, SOCKET_ERR_UNSUPPORTED);
-  hipStream_t s = (hipStream_t)stream;
-  const float* qp = (const float*)q_probs;
-#define SOCKET_SCORE_ARGS qp, codes, v_norm, lens, scores, B, Hq, Hkv, L, P, R, T, Tcap, score_stride, s
-  // 8 tokens per thread once the context is long enough to fill the chip with
-  // 4096-token tiles, 4 per thread below that.
-  const bool big = (int64_t)B * Hkv * ((T + 4095) / 4096) >= 512;
-  if (G == 1) return big ? dispatch_p<1, 2>(SOCKET_SCORE_ARGS) : dispatch_p<1, 1>(SOCKET_SCORE_ARGS);
-  if (G == 2) return big ? dispatch_p<2, 2>(SOCKET_SCORE_ARGS) : dispatch_p<2, 1>(SOCKET_SCORE_ARGS);
-  if (G <= 4) return big ? dispatch_p<4, 2>(SOCKET_SCORE_ARGS) : dispatch_p<4, 1>(SOCKET_SCORE_ARGS);
-  return big ? dispatch_p<8, 2>(SOCKET_SCORE_ARGS) : dispatch_p<8, 1>(SOCKET_SCORE_ARGS);
-#undef SOCKET_SCORE_ARGS
+  SOCKET_REQUIRE(Hq / Hkv <= 8, SOCKET_ERR_UNSUPPORTED);
+  const ScoreArgs a{q_probs, codes, v_norm, lens, scores, B, Hq, Hkv, L, P, R, T, Tcap, score_stride,
+                    (hipStream_t)stream};
+  return q_dtype == SOCKET_F32 ? dispatch_g<TabF32>(a) : dispatch_g<TabBF16>(a);
 }
 
 extern "C" int socket_soft_hash_collision(const float* q_probs, const int16_t* key_buckets,

@@ -73,20 +73,44 @@ __device__ __forceinline__ void find_bin(const uint32_t* hist, int need, int des
   }
 }
 
+// Visit scores[0:n] once, 16 bytes per lane per load and four loads in flight
+// per lane (a lone workgroup per row has to cover the memory latency itself).
 template <bool VEC, class F>
 __device__ __forceinline__ void for_each_score(const float* row, int n, int tid, F&& f) {
   if (VEC) {
     const int n4 = n & ~3;
-    for (int i = tid * 4; i < n4; i += kThreads * 4) {
+    constexpr int kStride = kThreads * 4;
+    int i = tid * 4;
+    for (; i + 3 * kStride < n4; i += 4 * kStride) {
+      float4 x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) x[u] = *reinterpret_cast<const float4*>(row + i + u * kStride);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        f(i + u * kStride, x[u].x);
+        f(i + u * kStride + 1, x[u].y);
+        f(i + u * kStride + 2, x[u].z);
+        f(i + u * kStride + 3, x[u].w);
+      }
+    }
+    for (; i < n4; i += kStride) {
       const float4 x = *reinterpret_cast<const float4*>(row + i);
       f(i, x.x);
       f(i + 1, x.y);
       f(i + 2, x.z);
       f(i + 3, x.w);
     }
-    for (int i = n4 + tid; i < n; i += kThreads) f(i, row[i]);
+    for (int t = n4 + tid; t < n; t += kThreads) f(t, row[t]);
   } else {
-    for (int i = tid; i < n; i += kThreads) f(i, row[i]);
+    int i = tid;
+    for (; i + 3 * kThreads < n; i += 4 * kThreads) {
+      float x[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) x[u] = row[i + u * kThreads];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) f(i + u * kThreads, x[u]);
+    }
+    for (; i < n; i += kThreads) f(i, row[i]);
   }
 }
 

@@ -113,9 +113,12 @@ def pack_codes_into(codes_i16_bhlt: torch.Tensor, codes: torch.Tensor, P: int, t
 def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
                  lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Soft-collision scores [B,Hq,T] fp32 (row pitch padded to a multiple of 4)
-    from q_probs fp32 [B,Hq,L,R] and the packed cache."""
+    from q_probs [B,Hq,L,R] and the packed cache.  q_probs may be float32 or
+    bfloat16; a bfloat16 table is read as is (the reference widens it with
+    `.float()`, GPT-FAST/kernels/sparse.py:42, which changes no value) and halves
+    the LDS bytes per gather.  float16 is widened to float32 first."""
     assert q_probs.is_cuda and q_probs.dim() == 4
-    if q_probs.dtype != torch.float32:
+    if q_probs.dtype not in (torch.float32, torch.bfloat16):
         q_probs = q_probs.float()
     q_probs = q_probs.contiguous()
     B, Hq, L, R = q_probs.shape
@@ -131,7 +134,7 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
     if lens is not None:
         assert lens.dtype == torch.int32 and lens.is_cuda and lens.numel() == B
     check("socket_score_packed", lib().socket_score_packed(
-        ptr(q_probs), 0, ptr(codes), ptr(v_norm), ptr(lens), ptr(out), B, Hq, Hkv, L, int(P), R, int(T),
+        ptr(q_probs), dtype_enum(q_probs.dtype), ptr(codes), ptr(v_norm), ptr(lens), ptr(out), B, Hq, Hkv, L, int(P), R, int(T),
         Tcap, pitch, stream_ptr(q_probs.device)))
     return out[:, :, :T]
 
