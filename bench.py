@@ -60,6 +60,7 @@ def algorithmic_bytes(w, lens=None, budgets=None):
         "score_f32": w.Hkv * tok * (wc + 2 + 4 * G),
         "score_f32_table": w.Hkv * tok * (wc + 2 + 4 * G),
         "select": sel,
+        "select_own_range": sel,
         "attend": w.Hq * kt * (4 * w.D + 4) + w.B * w.Hq * 4 * w.D,
         "dense": w.Hkv * tok * 4 * w.D,
     }
@@ -230,13 +231,13 @@ def main():
     q_table_f32 = q_table.float()
 
     def k_score():
-        return hash_cache.score_packed(q_table, codes, v_norm, T, w.P, lens=lens, out=scores_buf)
+        return hash_cache.score_packed(q_table, codes, v_norm, T, w.P, lens=lens, out=scores_buf, with_range=True)
 
     def k_score_f32():
         return hash_cache.score_packed(q_table_f32, codes, v_norm, T, w.P, lens=lens, out=scores_buf)
 
-    def k_select(scores):
-        return sparse.select_list(scores, w.sink, w.window, w.M, lens=lens, budgets=budgets)
+    def k_select(scores, rng=None):
+        return sparse.select_list(scores, w.sink, w.window, w.M, lens=lens, budgets=budgets, row_range=rng)
 
     def k_attend(sl, ln):
         return socket_kernels.sparse_attention_fwd(inp.q, inp.k, inp.v, sl, ln)
@@ -248,18 +249,18 @@ def main():
 
     def step():
         k_hash()
-        s = k_score()
-        sl, ln = k_select(s)
+        s, r = k_score()
+        sl, ln = k_select(s, r)
         return k_attend(sl, ln)
 
-    scores = k_score()
-    sl, ln = k_select(scores)
+    scores, rng = k_score()
+    sl, ln = k_select(scores, rng)
     out = k_attend(sl, ln)
     torch.cuda.synchronize()
 
     iters = max(args.steps, 1)
     if args.only:
-        fn = {"score": k_score, "score_f32": k_score_f32, "select": lambda: k_select(scores), "attend": lambda: k_attend(sl, ln),
+        fn = {"score": k_score, "score_f32": k_score_f32, "select": lambda: k_select(scores, rng), "attend": lambda: k_attend(sl, ln),
               "hash": k_hash, "dense": k_dense}[args.only]
         us = time_launches(fn, iters, warmup=args.warmup)
         print(json.dumps({"only": args.only, "workload": w.name, "us": round(us, 2),
@@ -299,7 +300,8 @@ def main():
         "hash": time_launches(k_hash, iters),
         "score": time_launches(k_score, iters),
         "score_f32_table": time_launches(k_score_f32, iters),
-        "select": time_launches(lambda: k_select(scores), iters),
+        "select": time_launches(lambda: k_select(scores, rng), iters),
+        "select_own_range": time_launches(lambda: k_select(scores), iters),
         "attend": time_launches(lambda: k_attend(sl, ln), iters),
         "dense": time_launches(k_dense, max(iters // 2, 5)),
     }

@@ -117,9 +117,17 @@ int socket_pack_codes(const int16_t* in, int64_t in_stride_b, int64_t in_stride_
  * GPT-FAST/kernels/sparse.py:42-55.
  * Requires Tcap % 4 == 0, score_stride % 4 == 0, 16-byte aligned pointers,
  * R a power of two >= 8, 2^P <= R, G <= 8, and the tables of one packed word
- * (32/P tables x R entries x G values) must fit in LDS. */
+ * (32/P tables x R entries x G values) must fit in LDS.
+ *
+ * row_range (optional, may be NULL): uint32 [B*Hq, range_parts, 2]; for every row
+ * and token tile the minimum and maximum order-preserving key of the tile's
+ * scores at t < len(b) (0xffffffff / 0 for a tile without such a token).
+ * range_parts must equal socket_score_range_parts(B, Hq, Hkv, T).  Passing the
+ * array on to socket_select_list saves that kernel its first pass over the scores. */
+int socket_score_range_parts(int B, int Hq, int Hkv, int T);
 int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
                         const uint16_t* v_norm, const int32_t* lens, float* scores,
+                        uint32_t* row_range, int range_parts,
                         int B, int Hq, int Hkv, int L, int P, int R, int T, int64_t Tcap,
                         int64_t score_stride, void* stream);
 
@@ -155,12 +163,15 @@ int socket_soft_hash_score_f16(const uint16_t* q_probs, const int16_t* key_bucke
  * part is written, starting at column 0.
  * Replaces torch.topk + the list assembly of build_sparse_list_decode,
  * GPT-FAST/kernels/sparse.py:57-95.  NaN scores rank above +inf, -0.0 equals +0.0.
+ * row_range / range_parts: the key ranges written by socket_score_packed for
+ * these scores, or NULL / 0 (then the kernel finds each row's range itself).
  * Requires M <= SOCKET_TOPK_MAX_M. */
 #define SOCKET_TOPK_MAX_M 16384
 int socket_select_list(const float* scores, int64_t score_stride, const int32_t* lens,
-                       const int32_t* budgets, int B, int Hq, int T, int M, int sink,
-                       int window, int write_base, int32_t* sparse_list, int64_t list_stride,
-                       int list_width, int32_t* sparse_len, void* stream);
+                       const int32_t* budgets, const uint32_t* row_range, int range_parts,
+                       int B, int Hq, int T, int M, int sink, int window, int write_base,
+                       int32_t* sparse_list, int64_t list_stride, int list_width,
+                       int32_t* sparse_len, void* stream);
 
 /* ------------------------------------------------------------------------
  * K4  sparse flash-decode

@@ -151,7 +151,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens,
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
     int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
-    int n_tiles, int xcd_remap, uint32_t bf16_one) {
+    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range) {
   typedef typename TT::elem TE;
   const Bf16Select sel{bf16_one, bf16_one << 16};
   constexpr int EPV = 16 / (int)sizeof(TE);   // table elements per 16-byte vector
@@ -308,8 +308,15 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     }
   }
 
-  // epilogue: multiply by the value norm, mask, store one float4 per head
+  // epilogue: multiply by the value norm, mask, store one float4 per head; on
+  // request also the tile's range of score keys per head, for the select kernel
   const uint16_t* vn_pair = v_norm + (int64_t)pair * Tcap;
+  uint32_t kmin[GP], kmax[GP];
+#pragma unroll
+  for (int g = 0; g < GP; ++g) {
+    kmin[g] = 0xffffffffu;
+    kmax[g] = 0u;
+  }
 #pragma unroll
   for (int j = 0; j < KT4; ++j) {
     if (!live[j]) continue;
@@ -324,14 +331,52 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
       if (g >= G) break;
       float o[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        o[i] = (tbase[j] + i < len) ? acc[j][i][g] * vn[i] : -INFINITY;
+      for (int i = 0; i < 4; ++i) {
+        const bool valid = tbase[j] + i < len;
+        o[i] = valid ? acc[j][i][g] * vn[i] : -INFINITY;
+        if (valid) {
+          const uint32_t key = score_to_key(o[i]);
+          kmin[g] = min(kmin[g], key);
+          kmax[g] = max(kmax[g], key);
+        }
+      }
       float* dst = scores + ((int64_t)(b * Hq + kvh * G + g)) * score_stride + tbase[j];
       if (tbase[j] + 4 <= T) {
         *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
       } else {
         for (int i = 0; i < 4 && tbase[j] + i < T; ++i) dst[i] = o[i];
       }
+    }
+  }
+  if (row_range) {
+    const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+    for (int g = 0; g < GP; ++g) {
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) {
+        kmin[g] = min(kmin[g], (uint32_t)__shfl_xor((int)kmin[g], d, SOCKET_WAVE));
+        kmax[g] = max(kmax[g], (uint32_t)__shfl_xor((int)kmax[g], d, SOCKET_WAVE));
+      }
+    }
+    __syncthreads();  // every wave is done with the table slices
+    uint32_t* red = reinterpret_cast<uint32_t*>(lds_raw);
+    if (lane == 0) {
+#pragma unroll
+      for (int g = 0; g < GP; ++g) {
+        red[(wave * GP + g) * 2] = kmin[g];
+        red[(wave * GP + g) * 2 + 1] = kmax[g];
+      }
+    }
+    __syncthreads();
+    if (tid < G) {
+      uint32_t lo = 0xffffffffu, hi = 0u;
+      for (int w = 0; w < THREADS / 64; ++w) {
+        lo = min(lo, red[(w * GP + tid) * 2]);
+        hi = max(hi, red[(w * GP + tid) * 2 + 1]);
+      }
+      uint32_t* dst = row_range + (((int64_t)(b * Hq + kvh * G + tid)) * n_tiles + tile) * 2;
+      dst[0] = lo;
+      dst[1] = hi;
     }
   }
 }
@@ -344,6 +389,8 @@ struct ScoreArgs {
   float* scores;
   int B, Hq, Hkv, L, P, R, T;
   int64_t Tcap, score_stride;
+  uint32_t* row_range;
+  int range_parts;
   hipStream_t stream;
 };
 
@@ -379,12 +426,14 @@ int launch_score_packed(const ScoreArgs& a) {
   }
   constexpr int TW = THREADS * 4 * KT4;
   const int n_tiles = (a.T + TW - 1) / TW;
+  if (a.row_range && a.range_parts != n_tiles) return SOCKET_ERR_SHAPE;
   const int n_pairs = a.B * a.Hkv;
   const int xcd_remap = (n_pairs % 8 == 0) ? 1 : 0;
   const int n_wg = n_pairs * n_tiles;
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
                      a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
-                     a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, xcd_remap, 0x3f80u);
+                     a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, xcd_remap, 0x3f80u,
+                     a.row_range);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }
@@ -399,14 +448,21 @@ int dispatch_p(const ScoreArgs& a) {
 // Tile size: the largest of 16384 / 4096 / 1024 tokens per workgroup that still
 // gives every CU a workgroup (the 16384-token tile keeps 16 tokens x G partial
 // sums per lane, which only fits the register file for G <= 4).
+int tile_tokens(int B, int Hkv, int G, int T) {
+  const SocketDeviceLimits& lim = socket_device_limits();
+  const int64_t pairs = (int64_t)B * Hkv;
+  if (G <= 4 && pairs * ((T + 16383) / 16384) >= lim.cu_count) return 16384;
+  if (pairs * ((T + 4095) / 4096) >= lim.cu_count) return 4096;
+  return 1024;
+}
+
 template <int GP, class TT>
 int dispatch_tile(const ScoreArgs& a) {
-  const SocketDeviceLimits& lim = socket_device_limits();
-  const int64_t pairs = (int64_t)a.B * a.Hkv;
+  const int tw = tile_tokens(a.B, a.Hkv, a.Hq / a.Hkv, a.T);
   if constexpr (GP <= 4) {
-    if (pairs * ((a.T + 16383) / 16384) >= lim.cu_count) return dispatch_p<GP, TT, 4, 1024>(a);
+    if (tw == 16384) return dispatch_p<GP, TT, 4, 1024>(a);
   }
-  if (pairs * ((a.T + 4095) / 4096) >= lim.cu_count) return dispatch_p<GP, TT, 2, 512>(a);
+  if (tw == 4096) return dispatch_p<GP, TT, 2, 512>(a);
   return dispatch_p<GP, TT, 1, 256>(a);
 }
 
@@ -485,8 +541,15 @@ int launch_collision_i16(const QT* q_probs, const int16_t* key_buckets, const ui
 
 }  // namespace
 
+extern "C" int socket_score_range_parts(int B, int Hq, int Hkv, int T) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv != 0) return 0;
+  const int tw = tile_tokens(B, Hkv, Hq / Hkv, T);
+  return (T + tw - 1) / tw;
+}
+
 extern "C" int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
                                    const uint16_t* v_norm, const int32_t* lens, float* scores,
+                                   uint32_t* row_range, int range_parts,
                                    int B, int Hq, int Hkv, int L, int P, int R, int T,
                                    int64_t Tcap, int64_t score_stride, void* stream) {
   SOCKET_REQUIRE(q_probs && codes && v_norm && scores, SOCKET_ERR_NULL);
@@ -503,7 +566,7 @@ extern "C" int socket_score_packed(const void* q_probs, int q_dtype, const uint3
                  SOCKET_ERR_ALIGN);
   SOCKET_REQUIRE(Hq / Hkv <= 8, SOCKET_ERR_UNSUPPORTED);
   const ScoreArgs a{q_probs, codes, v_norm, lens, scores, B, Hq, Hkv, L, P, R, T, Tcap, score_stride,
-                    (hipStream_t)stream};
+                    row_range, range_parts, (hipStream_t)stream};
   return q_dtype == SOCKET_F32 ? dispatch_g<TabF32>(a) : dispatch_g<TabBF16>(a);
 }
 

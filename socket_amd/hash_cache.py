@@ -111,12 +111,15 @@ def pack_codes_into(codes_i16_bhlt: torch.Tensor, codes: torch.Tensor, P: int, t
 
 @torch.no_grad()
 def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
-                 lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                 with_range: bool = False):
     """Soft-collision scores [B,Hq,T] fp32 (row pitch padded to a multiple of 4)
     from q_probs [B,Hq,L,R] and the packed cache.  q_probs may be float32 or
     bfloat16; a bfloat16 table is read as is (the reference widens it with
     `.float()`, GPT-FAST/kernels/sparse.py:42, which changes no value) and halves
-    the LDS bytes per gather.  float16 is widened to float32 first."""
+    the LDS bytes per gather.  float16 is widened to float32 first.
+    with_range=True also returns the per-tile key ranges of every row (int32
+    [B,Hq,parts,2]) for `select_list(..., row_range=...)`."""
     assert q_probs.is_cuda and q_probs.dim() == 4
     if q_probs.dtype not in (torch.float32, torch.bfloat16):
         q_probs = q_probs.float()
@@ -133,9 +136,15 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
         assert out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (B, Hq, pitch)
     if lens is not None:
         assert lens.dtype == torch.int32 and lens.is_cuda and lens.numel() == B
+    rng, parts = None, 0
+    if with_range:
+        parts = lib().socket_score_range_parts(B, Hq, Hkv, int(T))
+        rng = torch.empty((B, Hq, parts, 2), dtype=torch.int32, device=q_probs.device)
     check("socket_score_packed", lib().socket_score_packed(
-        ptr(q_probs), dtype_enum(q_probs.dtype), ptr(codes), ptr(v_norm), ptr(lens), ptr(out), B, Hq, Hkv, L, int(P), R, int(T),
-        Tcap, pitch, stream_ptr(q_probs.device)))
+        ptr(q_probs), dtype_enum(q_probs.dtype), ptr(codes), ptr(v_norm), ptr(lens), ptr(out),
+        ptr(rng), parts, B, Hq, Hkv, L, int(P), R, int(T), Tcap, pitch, stream_ptr(q_probs.device)))
+    if with_range:
+        return out[:, :, :T], rng
     return out[:, :, :T]
 
 
@@ -151,8 +160,8 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     q [B,Hq,D]; q_probs [B,Hq,L,R]; T = number of cached tokens to consider (an
     upper bound when `lens` gives per-sequence lengths).  Returns out [B,Hq,D].
     """
-    scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens)
-    sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets)
+    scores, rng = score_packed(q_probs, codes, v_norm, T, P, lens=lens, with_range=True)
+    sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets, row_range=rng)
     out = sparse_attention_fwd(q, k_cache, v_cache, sparse_list, sparse_len)
     if return_details:
         return out, scores, sparse_list, sparse_len

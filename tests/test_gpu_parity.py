@@ -21,6 +21,14 @@ pytestmark = pytest.mark.gpu
 ATOL = {torch.float32: 2e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
 
 
+def _score_keys(scores: torch.Tensor) -> np.ndarray:
+    """The select kernel's order-preserving float -> uint32 map (finite inputs)."""
+    u = scores.contiguous().numpy().view(np.uint32).copy()
+    u[u == 0x80000000] = 0
+    neg = (u & 0x80000000) != 0
+    return np.where(neg, ~u, u | np.uint32(0x80000000))
+
+
 def _rand_codes(g, B, H, L, T, P):
     return torch.randint(0, 1 << P, (B, H, L, T), generator=g, dtype=torch.int32).to(torch.int16)
 
@@ -58,9 +66,16 @@ def test_score_packed_matches_oracle(dev, B, Hq, Hkv, L, P, T, table_dtype):
     Tcap = (T + 64 + 7) // 8 * 8
     vn_full = torch.zeros(B, Hkv, Tcap, dtype=torch.float16)
     vn_full[..., :T] = v_norm
-    got = hash_cache.score_packed(q_probs.to(dev), _packed_cache(codes, P, Tcap, dev), vn_full.to(dev),
-                                  T, P, lens=lens.to(dev)).cpu()
+    got, rng = hash_cache.score_packed(q_probs.to(dev), _packed_cache(codes, P, Tcap, dev), vn_full.to(dev),
+                                       T, P, lens=lens.to(dev), with_range=True)
+    got, rng = got.cpu(), rng.cpu()
     allowed = (torch.arange(T)[None, None, :] < lens[:, None, None]).expand(B, Hq, T)
+    # per-tile key ranges handed to the select kernel: their union is the row's range
+    keys = _score_keys(got)
+    for b in range(B):
+        kk = keys[b, :, :int(lens[b])]
+        r = rng[b].numpy().view(np.uint32)
+        assert np.array_equal(r[..., 0].min(-1), kk.min(-1)) and np.array_equal(r[..., 1].max(-1), kk.max(-1))
     want = orc.collision_score(q_probs.float(), codes.repeat_interleave(G, dim=1), allowed,
                                v_norm.float().repeat_interleave(G, dim=1))
     rel = ((got - want).abs() / want.abs().clamp_min(1e-30)).nan_to_num(0).max()
