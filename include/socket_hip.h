@@ -165,13 +165,18 @@ int socket_soft_hash_score_f16(const uint16_t* q_probs, const int16_t* key_bucke
  * GPT-FAST/kernels/sparse.py:57-95.  NaN scores rank above +inf, -0.0 equals +0.0.
  * row_range / range_parts: the key ranges written by socket_score_packed for
  * these scores, or NULL / 0 (then the kernel finds each row's range itself).
- * Requires M <= SOCKET_TOPK_MAX_M. */
+ * workspace: optional scratch of socket_select_workspace_bytes(B, Hq, T, M) bytes
+ * (0 for short rows).  With it, long rows are cut into slices handled by many
+ * workgroups; without it (NULL) one workgroup handles a whole row.  Same result.
+ * Requires M <= SOCKET_TOPK_MAX_M, B*Hq <= 65535. */
 #define SOCKET_TOPK_MAX_M 16384
+size_t socket_select_workspace_bytes(int B, int Hq, int T, int M);
 int socket_select_list(const float* scores, int64_t score_stride, const int32_t* lens,
                        const int32_t* budgets, const uint32_t* row_range, int range_parts,
                        int B, int Hq, int T, int M, int sink, int window, int write_base,
                        int32_t* sparse_list, int64_t list_stride, int list_width,
-                       int32_t* sparse_len, void* stream);
+                       int32_t* sparse_len, void* workspace, size_t workspace_bytes,
+                       void* stream);
 
 /* ------------------------------------------------------------------------
  * K4  sparse flash-decode

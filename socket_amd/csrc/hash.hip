@@ -14,9 +14,11 @@
 // consecutive keys are gathered into lanes 0..31 and stored as one 128-byte
 // run of the table-major code cache.
 //
-// A wave owns 64 consecutive keys of one (b, kv head) (two 32-row M tiles) and
-// keeps their A fragments in registers for the whole column sweep; the planes
-// are staged in LDS, `wc` words (wc*32 columns, wc*8 KB) at a time.
+// A wave owns 64 consecutive keys of one (b, kv head) (two 32-row M tiles) at a
+// time and keeps their A fragments in registers for the whole column sweep; the
+// planes sit in LDS (all NW words when NW*8 KB fits, which L=60 x P=10 exactly
+// does at 160 KB) and workgroups are persistent, so the planes are fetched once
+// per CU, not once per tile.
 #include "socket_common.h"
 
 namespace {
@@ -24,7 +26,7 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 
-constexpr int kHashThreads = 256;
+constexpr int kHashThreads = 512;
 constexpr int kHashWaves = kHashThreads / SOCKET_WAVE;
 constexpr int kKeysPerWave = 64;
 constexpr int kD = 128;
@@ -87,14 +89,17 @@ __device__ __forceinline__ float sumsq8(const typename DT::storage* p) {
   return s;
 }
 
+// Persistent: the grid is sized to the CU count and every wave walks the 64-key
+// tiles tile = first, first + stride, ...; the plane slice is loaded into LDS once
+// per workgroup (all of it when NW*8 KB fits) and amortised over all of them.
 template <class DT>
-__global__ __launch_bounds__(kHashThreads) void hash_keys_kernel(
+__global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void hash_keys_kernel(
     const void* __restrict__ k_, const void* __restrict__ v_, int64_t k_sb, int64_t k_sh,
     int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss,
     const uint16_t* __restrict__ planes_words,  // bf16 [NW*32, 128]
     uint32_t* __restrict__ codes, uint16_t* __restrict__ v_norm,
     const int32_t* __restrict__ pos_b, int t0, int Hkv, int S, int L, int P, int NW, int64_t Tcap,
-    int tiles_per_row, int n_tiles, int wc) {
+    int tiles_per_row, int n_tiles, int wc, int words_per_wg) {
   typedef typename DT::storage ST;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   // planes slice in LDS: [wc*32 columns][128] bf16, 16-byte groups XOR-swizzled
@@ -102,90 +107,115 @@ __global__ __launch_bounds__(kHashThreads) void hash_keys_kernel(
   uint4* plds = reinterpret_cast<uint4*>(lds_raw);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int tile = blockIdx.x * kHashWaves + wave;  // 64-key tile of one (b, kv head)
-  const bool tile_ok = tile < n_tiles;
-  const int pair = tile_ok ? tile / tiles_per_row : 0;
-  const int s0 = tile_ok ? (tile % tiles_per_row) * kKeysPerWave : 0;
-  const int b = pair / Hkv, h = pair % Hkv;
-  const int pos0 = pos_b ? pos_b[b] : t0;
+  const int first_tile = blockIdx.x * kHashWaves + wave;
+  const int tile_stride = gridDim.x * kHashWaves;
   const int cpw = 32 / P;
 
-  // ---- A fragments: lane x holds row x%32, elements 8*(x/32) + 16*kk .. +7 ----
-  Frag afrag[2][kKSteps];
-  const ST* kbase = (const ST*)k_ + b * k_sb + h * k_sh;
-#pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
-    const int srow = s0 + mt * 32 + (lane & 31);
-    const bool ok = tile_ok && srow < S;
-#pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk) {
-      afrag[mt][kk].u = ok ? load_frag8<DT>(kbase + (int64_t)srow * k_ss + kk * 16 + (lane >> 5) * 8)
-                           : make_uint4(0, 0, 0, 0);
-    }
-  }
+  // gridDim.y splits the packed words between workgroups when there are too
+  // few key tiles to occupy the chip (the per-step append of a handful of keys)
+  const int word_begin = blockIdx.y * words_per_wg;
+  const int word_end = min(NW, word_begin + words_per_wg);
 
-  uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
-
-  for (int w0 = 0; w0 < NW; w0 += wc) {
-    const int nw = min(wc, NW - w0);
+  for (int w0 = word_begin; w0 < word_end; w0 += wc) {
+    const int nw = min(wc, word_end - w0);
     __syncthreads();
     {
-      // fill: nw*32 columns x 16 groups of 16 bytes
+      // fill: nw*32 columns x 16 groups of 16 bytes, eight loads in flight per lane
       const uint4* src = reinterpret_cast<const uint4*>(planes_words) + (int64_t)w0 * 32 * 16;
-      for (int i = tid; i < nw * 32 * 16; i += kHashThreads) {
-        const int col = i >> 4, grp = i & 15;
-        plds[col * 16 + (grp ^ (col & 15))] = src[i];
+      const int total = nw * 32 * 16;
+      constexpr int U = 8;
+      int i0 = tid;
+      for (; i0 + (U - 1) * kHashThreads < total; i0 += U * kHashThreads) {
+        uint4 x[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) x[u] = src[i0 + u * kHashThreads];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = i0 + u * kHashThreads;
+          const int col = i >> 4, grp = i & 15;
+          plds[col * 16 + (grp ^ (col & 15))] = x[u];
+        }
+      }
+      for (; i0 < total; i0 += kHashThreads) {
+        const int col = i0 >> 4, grp = i0 & 15;
+        plds[col * 16 + (grp ^ (col & 15))] = src[i0];
       }
     }
     __syncthreads();
-    if (!tile_ok) continue;
-    for (int ww = 0; ww < nw; ++ww) {
-      f32x16 acc0 = {0}, acc1 = {0};
-      const int col = ww * 32 + (lane & 31);
+
+    for (int tile = first_tile; tile < n_tiles; tile += tile_stride) {
+      const int pair = tile / tiles_per_row;
+      const int s0 = (tile % tiles_per_row) * kKeysPerWave;
+      const int b = pair / Hkv, h = pair % Hkv;
+      const int pos0 = pos_b ? pos_b[b] : t0;
+
+      // A fragments: lane x holds row x%32, elements 64*(x/32) + 8*kk .. +7, so a
+      // lane reads one contiguous half row over the 8 k-steps.  (The contraction
+      // only needs A and B to agree on which k each slot holds.)
+      Frag afrag[2][kKSteps];
+      const ST* kbase = (const ST*)k_ + b * k_sb + h * k_sh;
 #pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) {
-        Frag bf;
-        const int grp = kk * 2 + (lane >> 5);
-        bf.u = plds[col * 16 + (grp ^ (col & 15))];
-        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[0][kk].v, bf.v, acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[1][kk].v, bf.v, acc1, 0, 0, 0);
-      }
-      const int w = w0 + ww;
-      const int nbits = min(cpw, L - w * cpw) * P;
-      const uint32_t valid = nbits >= 32 ? 0xffffffffu : ((1u << nbits) - 1u);
-      uint32_t word0 = 0, word1 = 0;  // lane x < 32: packed word of key row x in M tile 0 / 1
+      for (int mt = 0; mt < 2; ++mt) {
+        const int srow = s0 + mt * 32 + (lane & 31);
+        const bool ok = srow < S;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row_lo = 8 * (r / 4) + (r % 4);  // lanes 0..31 of the ballot
-        const unsigned long long b0 = __ballot(acc0[r] >= 0.f);
-        const unsigned long long b1 = __ballot(acc1[r] >= 0.f);
-        if (lane == row_lo) {
-          word0 = (uint32_t)b0;
-          word1 = (uint32_t)b1;
-        } else if (lane == row_lo + 4) {
-          word0 = (uint32_t)(b0 >> 32);
-          word1 = (uint32_t)(b1 >> 32);
+        for (int kk = 0; kk < kKSteps; ++kk) {
+          afrag[mt][kk].u = ok ? load_frag8<DT>(kbase + (int64_t)srow * k_ss + (lane >> 5) * 64 + kk * 8)
+                               : make_uint4(0, 0, 0, 0);
         }
       }
-      if (lane < 32) {
-        uint32_t* dst = codes_pair + (int64_t)w * Tcap + pos0 + s0;
-        if (s0 + lane < S) dst[lane] = word0 & valid;
-        if (s0 + 32 + lane < S) dst[32 + lane] = word1 & valid;
-      }
-    }
-  }
+      const bool second = s0 + 32 < S;  // the tile's second 32 rows hold keys at all
 
-  // ---- fused value norm: 16 lanes per row, 4 rows per pass -----------------------
-  if (v_ != nullptr && tile_ok) {
-    const ST* vbase = (const ST*)v_ + b * v_sb + h * v_sh;
-    uint16_t* vn = v_norm + (int64_t)pair * Tcap + pos0;
-    const int sub = lane >> 4, part = lane & 15;
-    for (int r0 = 0; r0 < kKeysPerWave; r0 += 4) {
-      const int srow = s0 + r0 + sub;
-      float ss = (srow < S) ? sumsq8<DT>(vbase + (int64_t)srow * v_ss + part * 8) : 0.f;
+      uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
+      for (int ww = 0; ww < nw; ++ww) {
+        f32x16 acc0 = {0}, acc1 = {0};
+        const int col = ww * 32 + (lane & 31);
 #pragma unroll
-      for (int x = 1; x < 16; x <<= 1) ss += __shfl_xor(ss, x, SOCKET_WAVE);
-      if (part == 0 && srow < S) vn[srow] = f32_to_f16_bits(sqrtf(ss));
+        for (int kk = 0; kk < kKSteps; ++kk) {
+          Frag bf;
+          const int grp = (lane >> 5) * 8 + kk;
+          bf.u = plds[col * 16 + (grp ^ (col & 15))];
+          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[0][kk].v, bf.v, acc0, 0, 0, 0);
+          if (second) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[1][kk].v, bf.v, acc1, 0, 0, 0);
+        }
+        const int w = w0 + ww;
+        const int nbits = min(cpw, L - w * cpw) * P;
+        const uint32_t valid = nbits >= 32 ? 0xffffffffu : ((1u << nbits) - 1u);
+        uint32_t word0 = 0, word1 = 0;  // lane x < 32: packed word of key row x in M tile 0 / 1
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row_lo = 8 * (r / 4) + (r % 4);  // lanes 0..31 of the ballot
+          const unsigned long long b0 = __ballot(acc0[r] >= 0.f);
+          const unsigned long long b1 = __ballot(acc1[r] >= 0.f);
+          if (lane == row_lo) {
+            word0 = (uint32_t)b0;
+            word1 = (uint32_t)b1;
+          } else if (lane == row_lo + 4) {
+            word0 = (uint32_t)(b0 >> 32);
+            word1 = (uint32_t)(b1 >> 32);
+          }
+        }
+        if (lane < 32) {
+          uint32_t* dst = codes_pair + (int64_t)w * Tcap + pos0 + s0;
+          if (s0 + lane < S) dst[lane] = word0 & valid;
+          if (s0 + 32 + lane < S) dst[32 + lane] = word1 & valid;
+        }
+      }
+
+      // fused value norm: 16 lanes per row, 4 rows per pass (once per tile)
+      if (v_ != nullptr && w0 == 0) {  // only the workgroups that own word 0
+        const ST* vbase = (const ST*)v_ + b * v_sb + h * v_sh;
+        uint16_t* vn = v_norm + (int64_t)pair * Tcap + pos0;
+        const int sub = lane >> 4, part = lane & 15;
+        const int rows_here = min(kKeysPerWave, S - s0);
+        for (int r0 = 0; r0 < rows_here; r0 += 4) {
+          const int srow = s0 + r0 + sub;
+          float ss = (srow < S) ? sumsq8<DT>(vbase + (int64_t)srow * v_ss + part * 8) : 0.f;
+#pragma unroll
+          for (int x = 1; x < 16; x <<= 1) ss += __shfl_xor(ss, x, SOCKET_WAVE);
+          if (part == 0 && srow < S) vn[srow] = f32_to_f16_bits(sqrtf(ss));
+        }
+      }
     }
   }
 }
@@ -311,12 +341,21 @@ extern "C" int socket_hash_keys(const void* k, const void* v, int dtype, int64_t
   SOCKET_REQUIRE(n_tiles64 < (1LL << 31), SOCKET_ERR_SHAPE);
   const int n_tiles = (int)n_tiles64;
   const SocketDeviceLimits& lim = socket_device_limits();
-  // plane slice: as many words as fit half the LDS of a CU (two workgroups per CU)
-  int wc = (lim.max_lds_per_block / 2) / (32 * kD * 2);
+  // plane slice: every word when they all fit in LDS (one slice, loaded once per
+  // workgroup), else as many as fit; one persistent workgroup per CU
+  int wc = lim.max_lds_per_block / (32 * kD * 2);
   if (wc < 1) wc = 1;
   if (wc > NW) wc = NW;
+  int n_wg = (n_tiles + kHashWaves - 1) / kHashWaves;
+  if (n_wg > lim.cu_count) n_wg = lim.cu_count;
+  int wsplit = lim.cu_count / n_wg;  // > 1 only when the tiles leave CUs idle
+  if (wsplit > NW) wsplit = NW;
+  if (wsplit < 1) wsplit = 1;
+  const int words_per_wg = (NW + wsplit - 1) / wsplit;
+  wsplit = (NW + words_per_wg - 1) / words_per_wg;
+  if (wc > words_per_wg) wc = words_per_wg;
   const size_t lds = (size_t)wc * 32 * kD * 2;
-  const dim3 grid((n_tiles + kHashWaves - 1) / kHashWaves);
+  const dim3 grid(n_wg, wsplit);
   hipStream_t s = (hipStream_t)stream;
 #define SOCKET_HASH_LAUNCH(DT)                                                                     \
   do {                                                                                             \
@@ -328,7 +367,7 @@ extern "C" int socket_hash_keys(const void* k, const void* v, int dtype, int64_t
     hipLaunchKernelGGL(kern, grid, dim3(kHashThreads), lds, s, k, v, k_stride_b, k_stride_h,       \
                        k_stride_s, v_stride_b, v_stride_h, v_stride_s,                             \
                        (const uint16_t*)planes_words, codes, v_norm, pos_b, t0, Hkv, S, L, P, NW,  \
-                       Tcap, tiles_per_row, n_tiles, wc);                                          \
+                       Tcap, tiles_per_row, n_tiles, wc, words_per_wg);                            \
   } while (0)
   if (dtype == SOCKET_BF16) SOCKET_HASH_LAUNCH(DType_bf16);
   else if (dtype == SOCKET_F16) SOCKET_HASH_LAUNCH(DType_f16);

@@ -34,13 +34,14 @@ def _get_soft_hash_ext():
 
 
 def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=None, budgets=None,
-                write_base: bool = True, list_width=None, row_range=None):
+                write_base: bool = True, list_width=None, row_range=None, split: bool = True):
     """Top-M + [sink | window | heavy] assembly on fp32 score rows [B,H,T]
     (row pitch = scores.stride(1)).  Returns (sparse_list int32 [B,H,width],
     sparse_len int32 [B,H]).  `lens`/`budgets`: optional int32 [B] device tensors
     (per-sequence context length and top-k budget).  `row_range`: the int32
     [B,H,parts,2] key ranges `hash_cache.score_packed(..., with_range=True)`
-    returns for these scores (saves the kernel's first pass)."""
+    returns for these scores (saves the kernel's first pass).  `split=False`
+    forces the one-workgroup-per-row kernel (the result is the same)."""
     assert scores.is_cuda and scores.dtype == torch.float32 and scores.dim() == 3
     assert scores.stride(2) == 1 and scores.stride(0) == scores.shape[1] * scores.stride(1)
     B, H, T = scores.shape
@@ -58,11 +59,15 @@ def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=No
     sparse_len = torch.empty((B, H), dtype=torch.int32, device=scores.device)
     if list_width == 0:
         return sparse_list, sparse_len.zero_()
-    check("socket_select_list", lib().socket_select_list(
+    L = lib()
+    ws, ws_bytes = None, L.socket_select_workspace_bytes(B, H, T, M) if split else 0
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=scores.device)
+    check("socket_select_list", L.socket_select_list(
         ptr(scores), scores.stride(1), ptr(lens), ptr(budgets), ptr(row_range),
         0 if row_range is None else row_range.shape[2], B, H, T, M, int(sink), int(window),
         1 if write_base else 0, ptr(sparse_list), list_width, list_width, ptr(sparse_len),
-        stream_ptr(scores.device)))
+        ptr(ws), ws_bytes, stream_ptr(scores.device)))
     return sparse_list, sparse_len
 
 

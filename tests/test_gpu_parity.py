@@ -146,13 +146,20 @@ def test_loader_errors(dev):
 
 # ---------------------------------------------------------------- K3 select
 def _check_select(scores, sink, window, M, dev, lens=None, budgets=None):
+    """Both kernels paths (rows split over many workgroups / one workgroup per
+    row; they coincide for short rows) against the stable-sort oracle."""
+    for split in (True, False):
+        _check_select_path(scores, sink, window, M, dev, lens, budgets, split)
+
+
+def _check_select_path(scores, sink, window, M, dev, lens, budgets, split):
     B, H, T = scores.shape
     pitch = (T + 3) // 4 * 4
     buf = torch.full((B, H, pitch), float("nan"))
     buf[..., :T] = scores
     sl, ln = sparse.select_list(buf.to(dev)[..., :T], sink, window, M,
                                 lens=None if lens is None else lens.to(dev),
-                                budgets=None if budgets is None else budgets.to(dev))
+                                budgets=None if budgets is None else budgets.to(dev), split=split)
     sl, ln = sl.cpu(), ln.cpu()
     for b in range(B):
         n = T if lens is None else int(lens[b])
@@ -173,9 +180,9 @@ def test_select_random_scores(dev, T, M):
     _check_select(scores, 4, 64, M, dev)
 
 
-def test_select_ties_and_special_values(dev):
+@pytest.mark.parametrize("T", [20000, 70001])
+def test_select_ties_and_special_values(dev, T):
     g = torch.Generator().manual_seed(3)
-    T = 20000
     s = torch.randint(0, 50, (1, 6, T), generator=g).float()     # heavy ties, few distinct values
     s[0, 1] = 1.0                                                 # all equal -> indices 0..M-1
     s[0, 2, ::3] = float("-inf")                                  # masked keys
@@ -187,11 +194,12 @@ def test_select_ties_and_special_values(dev):
         _check_select(s, 4, 16, M, dev)
 
 
-def test_select_ragged_lengths_and_budgets(dev):
+@pytest.mark.parametrize("T", [9000, 66000])
+def test_select_ragged_lengths_and_budgets(dev, T):
     g = torch.Generator().manual_seed(11)
-    B, H, T = 4, 2, 9000
+    B, H = 4, 2
     scores = torch.rand(B, H, T, generator=g)
-    lens = torch.tensor([9000, 130, 4097, 1], dtype=torch.int32)
+    lens = torch.tensor([T, 130, T // 2 + 1, 1], dtype=torch.int32)
     budgets = torch.tensor([180, 500, 81, 3], dtype=torch.int32)
     _check_select(scores, 4, 128, 500, dev, lens=lens, budgets=budgets)
 
