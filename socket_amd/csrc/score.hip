@@ -12,9 +12,9 @@
 //    interleaved ([table][bucket][g]), so one LDS gather returns the terms of
 //    all G heads.  Partial sums stay in registers across slices, which keeps the
 //    reference's summation order.  Codes are read once per kv head, 16 bytes per
-//    lane, fully coalesced, one word ahead of their use.  The table may be fp32
-//    or bf16 (a bf16 soft-hash producer loses nothing and halves the LDS bytes
-//    per gather, which is what bounds this kernel).
+//    lane, fully coalesced, three words ahead of their use.  The table may be
+//    fp32 or bf16 (a bf16 soft-hash producer loses nothing, halves the LDS bytes
+//    per gather and lets the matrix core do the four head adds of a lookup).
 //  * collision_i16_kernel: the reference's own operand layout (int16 codes per
 //    query head), for drop-in callers.
 #include "socket_common.h"
@@ -35,74 +35,109 @@ struct TabBF16 {
   static constexpr int kEnum = SOCKET_BF16;
 };
 
-// acc[g] += entry[g] for one LDS entry of GP table elements.
+// One LDS entry (the GP heads' values for one bucket of one table) as raw words,
+// so that the gather (load) and the accumulation can be scheduled apart.
+template <int BYTES>
+struct RawEntry;
+template <>
+struct RawEntry<2> { uint16_t w; };
+template <>
+struct RawEntry<4> { uint32_t w; };
+template <>
+struct RawEntry<8> { uint2 w; };
+template <>
+struct RawEntry<16> { uint4 w; };
+template <>
+struct RawEntry<32> { uint4 w[2]; };
+
+template <int BYTES>
+__device__ __forceinline__ RawEntry<BYTES> load_entry(const void* lds) {
+  return *reinterpret_cast<const RawEntry<BYTES>*>(lds);
+}
+
+// bf16 entries are widened and added by the matrix core used as a four-wide
+// adder: v_mfma_f32_4x4x4_16B_bf16 computes, in each of its 16 independent 4x4
+// blocks (4 lanes each), D[i][j] = C[i][j] + sum_k A[i][k] * B[k][j], where lane
+// j of a block supplies column B[:,j] (4 bf16 = one 8-byte LDS entry: the four
+// heads' values) and holds column D[:,j] (4 fp32 = that lane's four head sums),
+// and lane i supplies row A[i,:].  With A the identity (lane i holds e_i) this is
+// acc[h] += entry[h] for h = 0..3 in one instruction, on a pipe that is
+// otherwise idle, instead of four VALU operations.  The products are exact; the
+// matrix core's accumulate may round differently from the fp32 adder in the last
+// place (and flushes denormals), hence the 2e-6 relative bound stated for bf16
+// tables; the fp32-table path uses plain adds and reproduces the reference sum
+// exactly.
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+struct Bf16Select {
+  short4_t identity_row;  // e_{lane % 4} as four bf16
+};
+
+__device__ __forceinline__ Bf16Select make_bf16_select(uint32_t bf16_one) {
+  const int r = threadIdx.x & 3;
+  uint2 w = make_uint2(0u, 0u);
+  if (r == 0) w.x = bf16_one;
+  else if (r == 1) w.x = bf16_one << 16;
+  else if (r == 2) w.y = bf16_one;
+  else w.y = bf16_one << 16;
+  Bf16Select s;
+  __builtin_memcpy(&s.identity_row, &w, 8);
+  return s;
+}
+
+__device__ __forceinline__ void add4_bf16(float* acc, uint2 four, const Bf16Select& sel) {
+  short4_t b;
+  __builtin_memcpy(&b, &four, 8);
+  float4_t c = {acc[0], acc[1], acc[2], acc[3]};
+  c = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(sel.identity_row, b, c, 0, 0, 0);
+  acc[0] = c[0];
+  acc[1] = c[1];
+  acc[2] = c[2];
+  acc[3] = c[3];
+}
+
+// acc[g] += entry[g], fp32 table
 template <int GP>
-__device__ __forceinline__ void accumulate_entry(float* acc, const float* entry_lds) {
-  if (GP == 1) {
-    acc[0] += entry_lds[0];
-  } else if (GP == 2) {
-    const float2 e = *reinterpret_cast<const float2*>(entry_lds);
-    acc[0] += e.x;
-    acc[1] += e.y;
+__device__ __forceinline__ void accumulate(float* acc, const RawEntry<GP * 4>& e, const TabF32*,
+                                           const Bf16Select&) {
+  if constexpr (GP == 1) {
+    acc[0] += __uint_as_float(e.w);
+  } else if constexpr (GP == 2) {
+    acc[0] += __uint_as_float(e.w.x);
+    acc[1] += __uint_as_float(e.w.y);
+  } else if constexpr (GP == 4) {
+    acc[0] += __uint_as_float(e.w.x);
+    acc[1] += __uint_as_float(e.w.y);
+    acc[2] += __uint_as_float(e.w.z);
+    acc[3] += __uint_as_float(e.w.w);
   } else {
 #pragma unroll
-    for (int v = 0; v < GP / 4; ++v) {
-      const float4 e = reinterpret_cast<const float4*>(entry_lds)[v];
-      acc[4 * v + 0] += e.x;
-      acc[4 * v + 1] += e.y;
-      acc[4 * v + 2] += e.z;
-      acc[4 * v + 3] += e.w;
+    for (int v = 0; v < 2; ++v) {
+      acc[4 * v + 0] += __uint_as_float(e.w[v].x);
+      acc[4 * v + 1] += __uint_as_float(e.w[v].y);
+      acc[4 * v + 2] += __uint_as_float(e.w[v].z);
+      acc[4 * v + 3] += __uint_as_float(e.w[v].w);
     }
   }
 }
 
-// bf16 entries: widening to fp32 and the add are one v_dot2_f32_bf16 per head,
-// acc += lo * 1 + hi * 0 (or the other way round).  The dot unit's final rounding
-// is not always that of the fp32 adder, so a sum of L terms can differ from the
-// sequential fp32 sum in the last few ulp (measured below 2e-6 relative; the
-// fp32-table path uses plain adds and reproduces the reference sum exactly).  The
-// (1,0) / (0,1) selectors are passed in as run-time values held in scalar
-// registers: written as literals the compiler folds them into an inline operand
-// constant, and with that encoding the instruction picked the wrong half.
-struct Bf16Select {
-  uint32_t lo, hi;  // bf16 pairs (1.0, 0.0) and (0.0, 1.0)
-};
-__device__ __forceinline__ float add_bf16(float acc, uint32_t pair, uint32_t selector) {
-  bf16x2_t a, one;
-  __builtin_memcpy(&a, &pair, 4);
-  __builtin_memcpy(&one, &selector, 4);
-  return __builtin_amdgcn_fdot2_f32_bf16(a, one, acc, false);
-}
-
+// acc[g] += entry[g], bf16 table
 template <int GP>
-__device__ __forceinline__ void accumulate_entry(float* acc, const float* entry_lds, const Bf16Select&) {
-  accumulate_entry<GP>(acc, entry_lds);
-}
-
-template <int GP>
-__device__ __forceinline__ void accumulate_entry(float* acc, const uint16_t* entry_lds, const Bf16Select& sel) {
-  if (GP == 1) {
-    acc[0] += bf16_bits_to_f32(entry_lds[0]);
-  } else if (GP == 2) {
-    const uint32_t e = *reinterpret_cast<const uint32_t*>(entry_lds);
-    acc[0] = add_bf16(acc[0], e, sel.lo);
-    acc[1] = add_bf16(acc[1], e, sel.hi);
-  } else if (GP == 4) {
-    const uint2 e = *reinterpret_cast<const uint2*>(entry_lds);
-    acc[0] = add_bf16(acc[0], e.x, sel.lo);
-    acc[1] = add_bf16(acc[1], e.x, sel.hi);
-    acc[2] = add_bf16(acc[2], e.y, sel.lo);
-    acc[3] = add_bf16(acc[3], e.y, sel.hi);
+__device__ __forceinline__ void accumulate(float* acc, const RawEntry<GP * 2>& e, const TabBF16*,
+                                           const Bf16Select& sel) {
+  if constexpr (GP == 1) {
+    acc[0] += bf16_bits_to_f32(e.w);
+  } else if constexpr (GP == 2) {
+    float a4[4] = {acc[0], acc[1], 0.f, 0.f};
+    add4_bf16(a4, make_uint2(e.w, 0u), sel);
+    acc[0] = a4[0];
+    acc[1] = a4[1];
+  } else if constexpr (GP == 4) {
+    add4_bf16(acc, e.w, sel);
   } else {
-    const uint4 e = *reinterpret_cast<const uint4*>(entry_lds);
-    acc[0] = add_bf16(acc[0], e.x, sel.lo);
-    acc[1] = add_bf16(acc[1], e.x, sel.hi);
-    acc[2] = add_bf16(acc[2], e.y, sel.lo);
-    acc[3] = add_bf16(acc[3], e.y, sel.hi);
-    acc[4] = add_bf16(acc[4], e.z, sel.lo);
-    acc[5] = add_bf16(acc[5], e.z, sel.hi);
-    acc[6] = add_bf16(acc[6], e.w, sel.lo);
-    acc[7] = add_bf16(acc[7], e.w, sel.hi);
+    add4_bf16(acc, make_uint2(e.w.x, e.w.y), sel);
+    add4_bf16(acc + 4, make_uint2(e.w.z, e.w.w), sel);
   }
 }
 
@@ -153,7 +188,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
     int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range) {
   typedef typename TT::elem TE;
-  const Bf16Select sel{bf16_one, bf16_one << 16};
+  const Bf16Select sel = make_bf16_select(bf16_one);
   constexpr int EPV = 16 / (int)sizeof(TE);   // table elements per 16-byte vector
   constexpr int SL = 1024 / THREADS;           // staging slots (one 16-byte vector per head) per lane
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -188,12 +223,15 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   const int chunk_tables = chunk_words * cpw;
   const int chunk_elems = chunk_tables * R * GP;  // table elements per LDS buffer
 
-  int tbase[KT4];
+  // tsafe: where a lane group without tokens (tile tail) reads instead, so that
+  // code loads need no predicate; its results are never stored
+  int tbase[KT4], tsafe[KT4];
   bool live[KT4];
 #pragma unroll
   for (int j = 0; j < KT4; ++j) {
     tbase[j] = tile * TW + j * (THREADS * 4) + tid * 4;
     live[j] = tbase[j] < T;
+    tsafe[j] = live[j] ? tbase[j] : tile * TW;
   }
 
   float acc[KT4][4][GP];
@@ -204,12 +242,25 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
 #pragma unroll
       for (int g = 0; g < GP; ++g) acc[j][i][g] = 0.f;
 
-  // packed words of the lane's token groups; each is reloaded with the next word
-  // as soon as it has been consumed
-  uint4 ring[KT4];
+  // Packed words of the lane's token groups, kPrefetch words deep: ring[0] is the
+  // word being consumed, ring[d] the word d steps ahead.  The code stream is the
+  // HBM traffic of this kernel and a CU needs tens of KB of it in flight to cover
+  // the memory latency; one word ahead (16 B x tokens/4 per lane) is not enough.
+  constexpr int kPrefetch = 3;
+  uint4 ring[kPrefetch][KT4];
 #pragma unroll
-  for (int j = 0; j < KT4; ++j)
-    ring[j] = live[j] ? *reinterpret_cast<const uint4*>(codes_pair + tbase[j]) : make_uint4(0, 0, 0, 0);
+  for (int d = 0; d < kPrefetch; ++d)
+#pragma unroll
+    for (int j = 0; j < KT4; ++j)
+      ring[d][j] = *reinterpret_cast<const uint4*>(codes_pair + (int64_t)min(d, NW - 1) * Tcap + tsafe[j]);
+  // group j has consumed its current word: shift the ring and fetch the word
+  // kPrefetch steps ahead (past the end it refetches the last word, unused)
+  auto advance = [&](int j, int w) {
+#pragma unroll
+    for (int d = 0; d + 1 < kPrefetch; ++d) ring[d][j] = ring[d + 1][j];
+    ring[kPrefetch - 1][j] = *reinterpret_cast<const uint4*>(
+        codes_pair + (int64_t)min(w + kPrefetch, NW - 1) * Tcap + tsafe[j]);
+  };
 
   // slice staging: slot s covers table elements [s*EPV, (s+1)*EPV) of every head
   uint4 stage[SL][GP];
@@ -282,22 +333,47 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     for (int w = w0; w < wend; ++w) {
       const int ntw = min(cpw, L - w * cpw);
       const TE* tw = table + (size_t)(w - w0) * cpw * R * GP;
-      const uint32_t* next_row = codes_pair + (int64_t)(w + 1) * Tcap;
-      const bool has_next = w + 1 < NW;
-#pragma unroll
-      for (int j = 0; j < KT4; ++j) {
-        const uint32_t wv[4] = {ring[j].x, ring[j].y, ring[j].z, ring[j].w};
-        if (has_next && live[j]) ring[j] = *reinterpret_cast<const uint4*>(next_row + tbase[j]);
-#pragma unroll
-        for (int jj = 0; jj < (PT ? 32 / PT : 32); ++jj) {
-          if (jj >= ntw) break;
-          const TE* tb = tw + (size_t)jj * R * GP;
-          const int sh = jj * P;
+      constexpr int EB = GP * (int)sizeof(TE);
+      if (PT != 0 && ntw == 32 / (PT ? PT : 1)) {
+        // Every table of the word is real: straight-line code.  The lookups are
+        // cut into batches of four (one table, one group of four tokens) and the
+        // LDS reads of batch k+1 are issued before batch k is accumulated, so the
+        // gather latency overlaps the adds instead of preceding them.
+        constexpr int CPW = PT ? 32 / PT : 1;
+        constexpr int NB = KT4 * CPW;
+        RawEntry<EB> ent[2][4];
+        auto issue = [&](int bi, RawEntry<EB>(&dst)[4]) {
+          const int j = bi / CPW, jj = bi % CPW;
+          const uint32_t wv[4] = {ring[0][j].x, ring[0][j].y, ring[0][j].z, ring[0][j].w};
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const uint32_t code = (wv[i] >> sh) & code_mask;
-            accumulate_entry<GP>(acc[j][i], tb + (size_t)code * GP, sel);
+            const uint32_t code = __builtin_amdgcn_ubfe(wv[i], jj * (PT ? PT : 1), PT ? PT : 1);
+            dst[i] = load_entry<EB>(tw + (size_t)jj * R * GP + (size_t)code * GP);
           }
+          if (jj == CPW - 1) advance(j, w);  // last use of this group's word
+        };
+        issue(0, ent[0]);
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi) {
+          if (bi + 1 < NB) issue(bi + 1, ent[(bi + 1) & 1]);
+          const int j = bi / CPW;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) accumulate<GP>(acc[j][i], ent[bi & 1][i], (const TT*)nullptr, sel);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < KT4; ++j) {
+          const uint32_t wv[4] = {ring[0][j].x, ring[0][j].y, ring[0][j].z, ring[0][j].w};
+          for (int jj = 0; jj < ntw; ++jj) {
+            const TE* tb = tw + (size_t)jj * R * GP;
+            const int sh = jj * P;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const uint32_t code = (wv[i] >> sh) & code_mask;
+              accumulate<GP>(acc[j][i], load_entry<EB>(tb + (size_t)code * GP), (const TT*)nullptr, sel);
+            }
+          }
+          advance(j, w);
         }
       }
     }
@@ -445,13 +521,13 @@ int dispatch_p(const ScoreArgs& a) {
   return launch_score_packed<GP, TT, KT4, THREADS, 0>(a);
 }
 
-// Tile size: the largest of 16384 / 4096 / 1024 tokens per workgroup that still
-// gives every CU a workgroup (the 16384-token tile keeps 16 tokens x G partial
-// sums per lane, which only fits the register file for G <= 4).
+// Tile size: the largest of 8192 / 4096 / 1024 tokens per workgroup that still
+// gives every CU a workgroup.  (16 tokens per lane would halve the table
+// refills again but does not fit 128 registers next to the prefetched codes.)
 int tile_tokens(int B, int Hkv, int G, int T) {
   const SocketDeviceLimits& lim = socket_device_limits();
   const int64_t pairs = (int64_t)B * Hkv;
-  if (G <= 4 && pairs * ((T + 16383) / 16384) >= lim.cu_count) return 16384;
+  if (G <= 4 && pairs * ((T + 8191) / 8192) >= lim.cu_count) return 8192;
   if (pairs * ((T + 4095) / 4096) >= lim.cu_count) return 4096;
   return 1024;
 }
@@ -460,7 +536,7 @@ template <int GP, class TT>
 int dispatch_tile(const ScoreArgs& a) {
   const int tw = tile_tokens(a.B, a.Hkv, a.Hq / a.Hkv, a.T);
   if constexpr (GP <= 4) {
-    if (tw == 16384) return dispatch_p<GP, TT, 4, 1024>(a);
+    if (tw == 8192) return dispatch_p<GP, TT, 2, 1024>(a);
   }
   if (tw == 4096) return dispatch_p<GP, TT, 2, 512>(a);
   return dispatch_p<GP, TT, 1, 256>(a);
