@@ -6,6 +6,7 @@ so it is in fact compared for equality as well where stated); attention within
 2e-2 absolute for bf16/fp16 inputs and 2e-5 for fp32 inputs.
 """
 import math
+import os
 
 import numpy as np
 import pytest
@@ -124,6 +125,62 @@ def test_reference_layout_scorer(dev, L, R, T):
     assert torch.equal(got, orc.collision_score(q_probs, codes, allowed, v_hist))
     got16 = soft_hash_score(q_probs.half().to(dev), codes.to(dev), v_hist.half().to(dev), allowed.to(dev)).cpu()
     assert torch.equal(got16, orc.collision_score_vnorm16(q_probs.half(), codes, v_hist.half(), allowed))
+
+
+REF_SO = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref", "libref_scorer.so")
+
+
+@pytest.mark.skipif(not os.path.exists(REF_SO), reason="oracle/_ref not built (needs the reference checkout at build time)")
+def test_scorers_vs_the_reference_kernel_at_config2_size(dev):
+    """The reference's own soft_hash_collision_kernel_3, compiled unmodified for
+    gfx950 (oracle/Makefile `ref`), as the checker at the full configuration-2
+    shape: B1, 32/8 heads, T=32768, L=60, P=10."""
+    import ctypes
+    ref = ctypes.CDLL(REF_SO)
+    g = torch.Generator().manual_seed(2000)
+    B, Hq, Hkv, L, P, T = 1, 32, 8, 60, 10, 32768
+    R, G = 1 << P, Hq // Hkv
+    q_probs = torch.softmax(torch.randn(B, Hq, L, R, generator=g) * 3, -1).to(dev)
+    codes = _rand_codes(g, B, Hkv, L, T, P).to(dev)
+    v_norm = (torch.rand(B, Hkv, T, generator=g) * 12).to(torch.float16).to(dev)
+    lens = torch.tensor([T - 77], dtype=torch.int32, device=dev)
+    # reference operands: codes and norms repeated per query head, bool mask
+    kb = codes.repeat_interleave(G, 1).contiguous()
+    allowed = (torch.arange(T, device=dev) < lens[0]).view(1, 1, T).expand(B, Hq, T).contiguous()
+    v_hist = v_norm.float().repeat_interleave(G, 1).contiguous()
+    want = torch.empty(B, Hq, T, dtype=torch.float32, device=dev)
+    rc = ref.ref_soft_hash_collision(
+        ctypes.c_void_p(q_probs.data_ptr()), ctypes.c_void_p(kb.data_ptr()), ctypes.c_void_p(allowed.data_ptr()),
+        ctypes.c_void_p(v_hist.data_ptr()), ctypes.c_void_p(want.data_ptr()), B, Hq, L, R, T,
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    # packed scorer, fp32 table: bit-identical
+    words = torch.zeros((B, Hkv, orc.words_per_key(L, P), T), dtype=torch.int32, device=dev)
+    hash_cache.pack_codes_into(codes, words, P)
+    got = hash_cache.score_packed(q_probs, words, v_norm, T, P, lens=lens)
+    assert torch.equal(got, want)
+    # packed scorer, bf16 table against the reference fed the same bf16 values widened
+    qb = q_probs.to(torch.bfloat16)
+    rc = ref.ref_soft_hash_collision(
+        ctypes.c_void_p(qb.float().contiguous().data_ptr()), ctypes.c_void_p(kb.data_ptr()),
+        ctypes.c_void_p(allowed.data_ptr()), ctypes.c_void_p(v_hist.data_ptr()), ctypes.c_void_p(want.data_ptr()),
+        B, Hq, L, R, T, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    gotb = hash_cache.score_packed(qb, words, v_norm, T, P, lens=lens)
+    ok = allowed
+    rel = ((gotb[ok] - want[ok]).abs() / want[ok].abs().clamp_min(1e-30)).max()
+    assert rel <= 1e-5 and torch.equal(gotb[~ok], want[~ok])
+    # the drop-in scorer on the reference's own operand layout: bit-identical
+    ext = load_soft_hash_collision(3)
+    qf = q_probs
+    rc = ref.ref_soft_hash_collision(
+        ctypes.c_void_p(qf.data_ptr()), ctypes.c_void_p(kb.data_ptr()), ctypes.c_void_p(allowed.data_ptr()),
+        ctypes.c_void_p(v_hist.data_ptr()), ctypes.c_void_p(want.data_ptr()), B, Hq, L, R, T,
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    got2 = ext.soft_hash_collision(qf.unsqueeze(2).contiguous(), kb, allowed.unsqueeze(2).contiguous(),
+                                   v_hist.unsqueeze(2).contiguous()).squeeze(2)
+    assert torch.equal(got2, want)
 
 
 def test_loader_errors(dev):

@@ -1,0 +1,170 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports every
+symbol include/socket_hip.h declares, entry points reject bad arguments before
+touching a device, the Python shims keep the reference's signatures, and the
+synthetic workloads are deterministic."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from socket_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "socket_hip.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        from socket_amd import build
+        build.build()
+    return _lib.lib()
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(socket_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = _declared()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in socket_hip.h but not exported"
+    # and the binding table covers exactly the header
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_status_strings_and_version(lib):
+    assert lib.socket_abi_version() == 1
+    seen = set()
+    for st in range(0, -7, -1):
+        s = lib.socket_status_string(st).decode()
+        assert s and s != "unknown status"
+        seen.add(s)
+    assert len(seen) == 7
+    assert lib.socket_status_string(-99).decode() == "unknown status"
+
+
+def test_words_per_key(lib):
+    assert lib.socket_words_per_key(60, 10) == 20      # 80 B per key
+    assert lib.socket_words_per_key(48, 10) == 16      # 64 B
+    assert lib.socket_words_per_key(32, 8) == 8        # 32 B
+    assert lib.socket_words_per_key(5, 16) == 3
+    assert lib.socket_words_per_key(0, 10) == 0 and lib.socket_words_per_key(4, 17) == 0 and lib.socket_words_per_key(4, 0) == 0
+
+
+def test_entry_points_reject_bad_arguments_without_a_device(lib):
+    nul = ctypes.c_void_p(0)
+    one = ctypes.c_void_p(16)          # non-NULL, 16-byte aligned, never dereferenced: validation fails first
+    # NULL pointers
+    assert lib.socket_score_packed(nul, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_NULL
+    assert lib.socket_select_list(nul, 64, nul, nul, nul, 0, 1, 1, 64, 4, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_NULL
+    assert lib.socket_hash_keys(nul, nul, 1, 0, 0, 128, 0, 0, 128, one, one, nul, nul, 0, 1, 1, 1, 128, 60, 10, 8, nul) == _lib.SOCKET_ERR_NULL
+    # shapes
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 5, 2, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_SHAPE    # Hq % Hkv
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 512, 64, 64, 64, nul) == _lib.SOCKET_ERR_SHAPE     # R < 2^P
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 65, 64, 68, nul) == _lib.SOCKET_ERR_SHAPE    # T > Tcap
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 66, 64, nul) == _lib.SOCKET_ERR_ALIGN    # Tcap % 4
+    assert lib.socket_score_packed(one, 2, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # fp16 table
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 16, 1, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # G = 16
+    assert lib.socket_hash_keys(one, nul, 1, 0, 0, 64, 0, 0, 64, one, one, nul, nul, 0, 1, 1, 1, 64, 60, 10, 8, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # D != 128
+    assert lib.socket_hash_keys(one, nul, 1, 0, 0, 128, 0, 0, 128, one, one, nul, nul, 4, 1, 1, 8, 128, 60, 10, 8, nul) == _lib.SOCKET_ERR_SHAPE  # t0 + S > Tcap
+    assert lib.socket_select_list(one, 64, nul, nul, nul, 0, 1, 1, 64, 20000, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # M too large
+    assert lib.socket_select_list(one, 32, nul, nul, nul, 0, 1, 1, 64, 4, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_SHAPE  # pitch < T
+    a = [one, one, one, 1, 128, 128, 0, 0, 128, 0, 0, 128, one, 8, 8, one, 1, 1, one, one]
+    assert lib.socket_attend_stage1(*a, 1, 4, 1, 48, 16, 1, 256, nul) == _lib.SOCKET_ERR_UNSUPPORTED       # D = 48
+    assert lib.socket_attend_stage1(*a, 1, 5, 2, 128, 16, 1, 256, nul) == _lib.SOCKET_ERR_SHAPE             # Hq % Hkv
+    a[5] = 100                                                                                            # q head stride not 16-byte aligned for bf16
+    assert lib.socket_attend_stage1(*a, 1, 4, 1, 128, 16, 1, 256, nul) == _lib.SOCKET_ERR_ALIGN
+    # workspace too small
+    need = lib.socket_sparse_attention_workspace_bytes(1, 4, 128, 300)
+    assert need > 0
+    r = lib.socket_sparse_attention(one, one, one, 1, 128, 128, 0, 0, 128, 0, 0, 128, one, 300, 300, one, 4, 1, one, 512, 128,
+                                    one, need - 1, 1, 4, 1, 128, 16, 300, nul)
+    assert r == _lib.SOCKET_ERR_WORKSPACE
+    with pytest.raises(_lib.SocketHipError, match="workspace"):
+        _lib.check("socket_sparse_attention", r)
+
+
+def test_sizes_helpers(lib):
+    bs = lib.socket_sparse_attention_block_seq(4, 32, 2308)
+    assert bs % 64 == 0 and bs >= 64
+    ns = (2308 + bs - 1) // bs
+    assert lib.socket_sparse_attention_workspace_bytes(4, 32, 128, 2308) == 4 * 32 * ns * 129 * 4
+    assert lib.socket_select_workspace_bytes(4, 32, 4096, 128) == 0        # short rows: one workgroup per row
+    assert lib.socket_select_workspace_bytes(4, 32, 131072, 2048) > 0
+    assert lib.socket_score_range_parts(4, 32, 8, 131072) * 8192 >= 131072
+    assert lib.socket_score_range_parts(1, 5, 2, 100) == 0
+
+
+def test_python_api_keeps_reference_signatures():
+    from socket_amd import socket_kernels, sparse
+    from socket_amd.soft_hash_collision_loader import load_soft_hash_collision
+
+    def params(f):
+        return list(inspect.signature(f).parameters)
+
+    # kernels/socket_triton_kernels.py:167-258
+    assert params(socket_kernels.sparse_attention_fwd) == ["query", "key", "value", "sparse_list", "sparse_len", "block_seq"]
+    assert inspect.signature(socket_kernels.sparse_attention_fwd).parameters["block_seq"].default == 256
+    assert params(socket_kernels.sparse_decode_stage1) == ["q", "k", "v", "sparse_list", "sparse_len", "max_len_in_batch",
+                                                           "mid_out", "mid_out_logsumexp", "block_seq"]
+    assert params(socket_kernels.sparse_decode_stage2) == ["mid_out", "mid_out_logsumexp", "sparse_len", "out", "block_seq"]
+    assert params(socket_kernels.attention_mask_to_allowed_prob) == ["attention_mask", "K"]
+    # GPT-FAST/kernels/sparse.py:16-28
+    sig = inspect.signature(sparse.build_sparse_list_decode)
+    assert list(sig.parameters) == ["q_probs", "k_hard_bhlt", "v_norm_bht", "allowed_bht", "sink", "window", "M",
+                                    "KC", "BLOCK_N", "num_warps", "num_stages"]
+    assert [sig.parameters[k].default for k in ("KC", "BLOCK_N", "num_warps", "num_stages")] == [8, 512, 8, 2]
+    assert inspect.signature(load_soft_hash_collision).parameters["version"].default == 3
+
+
+def test_attention_mask_to_allowed_prob():
+    from socket_amd.socket_kernels import attention_mask_to_allowed_prob as f
+
+    m = torch.tensor([[[False, True, False, True]]])                # bool: True = forbidden
+    out = f(m, 3)
+    assert out.shape == (1, 1, 1, 3) and out.dtype == torch.float32 and out.flatten().tolist() == [1.0, 0.0, 1.0]
+    add = torch.tensor([[[[0.0, -1e9, 0.0, 0.0]]]])                  # additive: < 0 = forbidden
+    assert f(add, 4).flatten().tolist() == [1.0, 0.0, 1.0, 1.0]
+
+
+def test_asserts_fire_on_cpu_tensors():
+    from socket_amd import socket_kernels, sparse
+
+    q = torch.zeros(1, 4, 128)
+    kv = torch.zeros(1, 1, 8, 128)
+    sl = torch.zeros(1, 4, 3, dtype=torch.int32)
+    ln = torch.zeros(1, 4, dtype=torch.int32)
+    with pytest.raises(AssertionError):
+        socket_kernels.sparse_attention_fwd(q, kv, kv, sl, ln)
+    with pytest.raises(AssertionError):
+        sparse.build_sparse_list_decode(torch.zeros(1, 4, 2, 16), torch.zeros(1, 4, 2, 8, dtype=torch.int16),
+                                        torch.zeros(1, 4, 8), torch.ones(1, 4, 8, dtype=torch.bool), 1, 1, 2)
+
+
+def test_workloads_are_deterministic_and_shaped():
+    from socket_amd.workloads import WORKLOADS, make_inputs, scaled
+
+    w = scaled(WORKLOADS["c1"], T=256)
+    a, b = make_inputs(w), make_inputs(w)
+    assert torch.equal(a.k, b.k) and torch.equal(a.q_probs, b.q_probs) and torch.equal(a.planes, b.planes)
+    assert a.q.shape == (1, 32, 128) and a.k.shape == (1, 8, 256, 128) and a.q_probs.shape == (1, 32, 32, 256)
+    assert torch.allclose(a.q_probs.sum(-1), torch.ones(1, 32, 32), atol=1e-5)
+    c = make_inputs(w, layer=1)
+    assert not torch.equal(a.k, c.k)
+    r = make_inputs(scaled(WORKLOADS["c5"], T=2048, t_min=512, B=3))
+    assert r.lens.dtype == torch.int32 and int(r.lens.max()) == 2048 and int(r.lens.min()) >= 512
+    assert torch.equal(r.budgets, (r.lens.double() * 0.02).floor().int())
+    # planted keys point along the group's mean query direction: they outscore a typical key
+    w2 = scaled(WORKLOADS["c1"], T=1024)
+    i2 = make_inputs(w2)
+    qdir = i2.q.view(1, 8, 4, 128).mean(2)
+    proj = torch.einsum("bhtd,bhd->bht", i2.k, qdir / qdir.norm(dim=-1, keepdim=True))
+    top16 = proj.topk(16, dim=-1).values.min()
+    assert top16 > 2.0 and proj.median() < 1.0
