@@ -163,7 +163,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c5"])
-    ap.add_argument("--only", default=None, choices=["score", "score_f32", "select", "attend", "hash", "dense"])
+    ap.add_argument("--only", default=None,
+                    choices=["score", "score_f32", "select", "attend", "hash", "dense", "copy"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     args = ap.parse_args()
@@ -259,6 +260,15 @@ def main():
     torch.cuda.synchronize()
 
     iters = max(args.steps, 1)
+    if args.only == "copy":
+        # a plain device copy of known size (256 MiB read + 256 MiB written per launch):
+        # the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters
+        a = torch.empty(1 << 26, dtype=torch.float32, device=dev).normal_()
+        b = torch.empty_like(a)
+        us = time_launches(lambda: b.copy_(a), iters, warmup=args.warmup)
+        print(json.dumps({"only": "copy", "bytes_read": a.numel() * 4, "bytes_written": a.numel() * 4,
+                          "us": round(us, 2), "gbs": round(2 * a.numel() * 4 / us / 1e3, 1), "iters": iters}))
+        return
     if args.only:
         fn = {"score": k_score, "score_f32": k_score_f32, "select": lambda: k_select(scores, rng), "attend": lambda: k_attend(sl, ln),
               "hash": k_hash, "dense": k_dense}[args.only]
