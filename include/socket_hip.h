@@ -123,7 +123,8 @@ int socket_pack_codes(const int16_t* in, int64_t in_stride_b, int64_t in_stride_
  * and token tile the minimum and maximum order-preserving key of the tile's
  * scores at t < len(b) (0xffffffff / 0 for a tile without such a token).
  * range_parts must equal socket_score_range_parts(B, Hq, Hkv, T).  Passing the
- * array on to socket_select_list saves that kernel its first pass over the scores. */
+ * array on to socket_select_list saves that kernel a pass over the scores for the
+ * rows it has to select without its sampled threshold. */
 int socket_score_range_parts(int B, int Hq, int Hkv, int T);
 int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
                         const uint16_t* v_norm, const int32_t* lens, float* scores,
@@ -164,10 +165,11 @@ int socket_soft_hash_score_f16(const uint16_t* q_probs, const int16_t* key_bucke
  * Replaces torch.topk + the list assembly of build_sparse_list_decode,
  * GPT-FAST/kernels/sparse.py:57-95.  NaN scores rank above +inf, -0.0 equals +0.0.
  * row_range / range_parts: the key ranges written by socket_score_packed for
- * these scores, or NULL / 0 (then the kernel finds each row's range itself).
+ * these scores, or NULL / 0 (then the kernel finds a row's range itself when it
+ * needs it).
  * workspace: optional scratch of socket_select_workspace_bytes(B, Hq, T, M) bytes
- * (0 for short rows).  With it, long rows are cut into slices handled by many
- * workgroups; without it (NULL) one workgroup handles a whole row.  Same result.
+ * (0 for short rows).  With it, long rows are first filtered slice by slice by
+ * many workgroups; without it (NULL) one workgroup handles a whole row.  Same result.
  * Requires M <= SOCKET_TOPK_MAX_M, B*Hq <= 65535. */
 #define SOCKET_TOPK_MAX_M 16384
 size_t socket_select_workspace_bytes(int B, int Hq, int T, int M);

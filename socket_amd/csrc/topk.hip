@@ -2,31 +2,38 @@
 // fused with the [sink | window | heavy] index-list assembly of
 // GPT-FAST/kernels/sparse.py:57-95.
 //
-// One workgroup (1024 lanes) per score row.  Scores are mapped to
-// order-preserving 32-bit keys.  The k-th largest key is located by range
-// refinement: a 2048-bin LDS histogram over [lo, hi] (initially the row's
-// min/max key, so bins are spread over the values that actually occur and the
-// LDS atomics rarely collide), then the bin holding the k-th key becomes the
-// new range.  As soon as that bin holds at most kCandCap keys the row is read
-// one last time: keys above the bin go straight to an LDS buffer, the bin's
-// keys are sorted on the side and the best of them appended, and one bitonic
-// sort of (key, ~index) composites puts the k winners in descending order.  A
-// bin that is a single key value with more than kCandCap copies (mass ties) is
-// resolved by a histogram over index ranges instead, taking the lowest indices.
-// Only the first read of a row comes from HBM; the row stays in L2 for the later
-// passes.  The scorer can hand over each row's key range (per-tile partial
-// minima / maxima), which saves the first pass.
+// Scores are mapped to order-preserving 32-bit keys and paired with the
+// complemented index into 64-bit composites (key << 32 | ~index), so "larger
+// composite" is exactly "higher score, then lower index" and all composites of a
+// row are distinct.
 //
-// A single workgroup is bound by one CU's VALU rate (about ten operations per
-// score per pass), so long rows are processed by the split path instead when
-// the caller provides a workspace: the row is cut into slices of kSliceLen
-// scores and four kernels run over (slice, row) or (row) grids --
-//   select_hist_kernel       per-slice histograms over the row's key range
-//   select_threshold_kernel  sums them, finds the bin of the k-th key
-//   select_collect_kernel    appends winners / bin candidates to per-row lists
-// -- after which the one-workgroup kernel only has to rank the gathered keys of
-// each row (or, for a row whose k-th bin turned out too crowded for the
-// candidate list -- mass ties -- does the whole job as before).
+// select_list_kernel, one workgroup (1024 lanes) per row, selects in two ways:
+//  * pooled: a superset of the row's m winners, at most kPoolCap composites, is
+//    put into LDS and the m-th largest located there by range refinement -- a
+//    2048-bin LDS histogram over [lo, hi] (initially the pool's min / max, so the
+//    bins spread over the values that occur and LDS atomics rarely collide), then
+//    the bin holding the m-th becomes the new range, until it holds at most
+//    kCandCap entries.  Because the composites are distinct, ties need no special
+//    case.  The pool is the whole row when that fits; otherwise everything at or
+//    above a threshold estimated from a fixed sample of the row and aimed at
+//    about 2m entries.  For long rows select_local_kernel applies the threshold
+//    beforehand, one 256-lane workgroup per slice of 16384 scores held in
+//    registers (one HBM read of the scores in all), and the row kernel only
+//    gathers the slices' lists.  A pool that comes out shorter than m or longer
+//    than kPoolCap (the sample misjudged the row, or one key value is massively
+//    repeated) is dropped and the row redone from scratch: the result is always
+//    exact, only the time differs.
+//  * from scratch: the same refinement over the row itself, one pass per level
+//    (the row stays in L2), until the m-th key's bin holds at most kCandCap keys;
+//    one more pass collects the keys above the bin and the bin's own.  A single
+//    key value with more than kCandCap copies (mass ties) is resolved by a
+//    histogram over index ranges (lowest indices win).  The scorer can hand over
+//    the row's key range, which saves the first pass.
+// Either way the winners are put in order without a full sort: their level-0
+// histogram bins already order them coarsely and a bin seldom holds more than a
+// few, so each winner goes to (#winners in higher bins) + (#bin-mates beating
+// it); crowded bins fall back to an in-LDS bitonic sort whose short exchange
+// distances stay in registers and wave shuffles.
 #include "socket_common.h"
 
 namespace {
@@ -34,20 +41,37 @@ namespace {
 constexpr int kThreads = 1024;
 constexpr int kWaves = kThreads / SOCKET_WAVE;
 constexpr int kBins = 2048;
-constexpr int kCandCap = 2048;
+constexpr int kCandCap = 2048;           // entries of the k-th bin kept in LDS
+constexpr int kMaxBinForCounting = 128;  // larger bins are sorted, not rank-counted
+
+constexpr int kSliceLen = 16384;  // scores per select_local_kernel workgroup
+constexpr int kLocThreads = 256;
+constexpr int kLocWaves = kLocThreads / SOCKET_WAVE;
+constexpr int kLocPerLane = kSliceLen / kLocThreads;  // 64 keys in registers
+constexpr int kPoolCap = 8192;    // composites pooled per row in LDS
+constexpr int kMaxSlices = 64;
+
+typedef unsigned long long u64;
 
 struct SelectShared {
-  uint32_t lo, hi;      // current key range (inclusive)
-  int need;             // keys still to take from inside [lo, hi]
-  int bin_count;        // keys in the bin holding the k-th key
-  int done;             // refinement finished
-  int fill_above;       // append cursor: keys above the bin
-  int fill_cand;        // append cursor: keys inside the bin
-  int idx_star;         // mass-tie case: largest index taken among the ties
+  u64 lo, hi;           // current key / composite range (inclusive)
+  int need;             // winners still to take from inside [lo, hi]
+  int bin_count;        // entries in the bin holding the k-th
+  int done;
+  int fill_above, fill_cand, fill_pool;
+  int idx_star;         // mass ties: largest index taken among the ties
   int found_bin, found_before, found_count;
-  uint32_t wmin[kWaves], wmax[kWaves];
+  u64 wmin[kWaves], wmax[kWaves];
   int wsum[kWaves];
+  int wflag[kWaves];
 };
+
+__device__ __forceinline__ u64 composite(uint32_t key, int idx) {
+  return ((u64)key << 32) | (u64)(0xffffffffu - (uint32_t)idx);
+}
+__device__ __forceinline__ int32_t composite_index(u64 c) {
+  return (int32_t)(0xffffffffu - (uint32_t)(c & 0xffffffffull));
+}
 
 __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 #pragma unroll
@@ -58,35 +82,46 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
   return v;
 }
 
-// All lanes of the workgroup.  Ranks the bins from the top (descending != 0) or
-// from the bottom, two per lane, and publishes in `sh` the bin where the running
-// count first reaches `need`, the count ranked before it and its own count.
+__device__ __forceinline__ u64 shfl_xor_u64(u64 v, int mask) {
+  const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, SOCKET_WAVE);
+  const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, SOCKET_WAVE);
+  return ((u64)hi << 32) | lo;
+}
+
+// All THREADS lanes.  Ranks the bins from the top (descending != 0) or from the
+// bottom, kBins / THREADS per lane, and publishes in `sh` the bin where the
+// running count first reaches `need`, the count ranked before it and its own.
+template <int THREADS>
 __device__ __forceinline__ void find_bin(const uint32_t* hist, int need, int descending,
                                          SelectShared& sh, int tid) {
+  constexpr int PER = kBins / THREADS;
   const int lane = tid & 63, wave = tid >> 6;
-  const int r0 = 2 * tid, r1 = 2 * tid + 1;
-  const int b0 = descending ? (kBins - 1 - r0) : r0;
-  const int b1 = descending ? (kBins - 1 - r1) : r1;
-  const int c0 = (int)hist[b0], c1 = (int)hist[b1];
-  const int incl_w = wave_incl_scan(c0 + c1, lane);
+  int c[PER], mine = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int r = tid * PER + i;
+    c[i] = (int)hist[descending ? (kBins - 1 - r) : r];
+    mine += c[i];
+  }
+  const int incl_w = wave_incl_scan(mine, lane);
   if (lane == 63) sh.wsum[wave] = incl_w;
   __syncthreads();
-  int base = 0;
-  for (int w = 0; w < wave; ++w) base += sh.wsum[w];
-  const int excl = base + incl_w - (c0 + c1);
-  if (excl < need && need <= excl + c0) {
-    sh.found_bin = b0;
-    sh.found_before = excl;
-    sh.found_count = c0;
-  } else if (excl + c0 < need && need <= excl + c0 + c1) {
-    sh.found_bin = b1;
-    sh.found_before = excl + c0;
-    sh.found_count = c1;
+  int run = incl_w - mine;
+  for (int w = 0; w < wave; ++w) run += sh.wsum[w];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    if (run < need && need <= run + c[i]) {
+      const int r = tid * PER + i;
+      sh.found_bin = descending ? (kBins - 1 - r) : r;
+      sh.found_before = run;
+      sh.found_count = c[i];
+    }
+    run += c[i];
   }
   __syncthreads();
 }
 
-// Visit scores[0:n] once, 16 bytes per lane per load and eight loads in flight
+// Visit row[begin:n) once, 16 bytes per lane per load and eight loads in flight
 // per lane (a lone workgroup per row has to cover the memory latency itself).
 template <bool VEC, int THREADS, class F>
 __device__ __forceinline__ void for_each_in(const float* row, int begin, int n, int tid, F&& f) {
@@ -128,16 +163,10 @@ __device__ __forceinline__ void for_each_in(const float* row, int begin, int n, 
   }
 }
 
-template <bool VEC, class F>
-__device__ __forceinline__ void for_each_score(const float* row, int n, int tid, F&& f) {
-  for_each_in<VEC, kThreads>(row, 0, n, tid, f);
-}
-
-// Append `value` to an LDS list if `take`: one atomic per wave, positions handed
+// Append `value` to a list if `take`: one LDS atomic per wave, positions handed
 // out by a ballot prefix count.  Safe under divergence (only active lanes vote).
-__device__ __forceinline__ void wave_append(bool take, unsigned long long value, int* cursor,
-                                            unsigned long long* list, int cap) {
-  const unsigned long long mask = __ballot(take);
+__device__ __forceinline__ void wave_append(bool take, u64 value, int* cursor, u64* list, int cap) {
+  const u64 mask = __ballot(take);
   if (mask == 0) return;
   const int lane = threadIdx.x & 63;
   const int leader = __ffsll((long long)mask) - 1;
@@ -150,21 +179,15 @@ __device__ __forceinline__ void wave_append(bool take, unsigned long long value,
   }
 }
 
-__device__ __forceinline__ unsigned long long shfl_xor_u64(unsigned long long v, int mask) {
-  const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, SOCKET_WAVE);
-  const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, SOCKET_WAVE);
-  return ((unsigned long long)hi << 32) | lo;
-}
-
 // Bitonic sort of buf[0:np] (np a power of two) into descending order by the
-// whole workgroup.  Lane t owns elements [t*E, (t+1)*E): exchange distances
-// below E stay in registers, below 64*E go through wave shuffles, and only the
-// longer ones through LDS with a barrier.  Callers sync before and get a synced
-// buffer back.
+// whole 1024-lane workgroup.  Lane t owns elements [t*E, (t+1)*E): exchange
+// distances below E stay in registers, below 64*E go through wave shuffles, and
+// only the longer ones through LDS with a barrier.  Callers sync before and get
+// a synced buffer back.
 template <int E>
-__device__ __forceinline__ void sort_desc_impl(unsigned long long* buf, int np, int tid) {
+__device__ __forceinline__ void sort_desc_impl(u64* buf, int np, int tid) {
   const bool active = tid * E < np;
-  unsigned long long r[E];
+  u64 r[E];
   auto load = [&]() {
 #pragma unroll
     for (int e = 0; e < E; ++e) r[e] = active ? buf[tid * E + e] : 0ull;
@@ -180,10 +203,10 @@ __device__ __forceinline__ void sort_desc_impl(unsigned long long* buf, int np, 
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         const int i = tid * E + e;
-        const unsigned long long other = shfl_xor_u64(r[e], j / E);
+        const u64 other = shfl_xor_u64(r[e], j / E);
         const bool lower = (i & j) == 0, desc = (i & k) == 0;
-        const unsigned long long mx = r[e] > other ? r[e] : other;
-        const unsigned long long mn = r[e] > other ? other : r[e];
+        const u64 mx = r[e] > other ? r[e] : other;
+        const u64 mn = r[e] > other ? other : r[e];
         r[e] = (lower == desc) ? mx : mn;
       }
     }
@@ -195,8 +218,8 @@ __device__ __forceinline__ void sort_desc_impl(unsigned long long* buf, int np, 
         if (e & j) continue;
         const int p = e | j;
         const bool desc = ((tid * E + e) & k) == 0;
-        const unsigned long long a = r[e], c = r[p];
-        const unsigned long long mx = a > c ? a : c, mn = a > c ? c : a;
+        const u64 a = r[e], c = r[p];
+        const u64 mx = a > c ? a : c, mn = a > c ? c : a;
         r[e] = desc ? mx : mn;
         r[p] = desc ? mn : mx;
       }
@@ -212,7 +235,7 @@ __device__ __forceinline__ void sort_desc_impl(unsigned long long* buf, int np, 
       for (int i = tid; i < np; i += kThreads) {
         const int p = i ^ j;
         if (p > i) {
-          const unsigned long long a = buf[i], c = buf[p];
+          const u64 a = buf[i], c = buf[p];
           const bool desc = (i & k) == 0;
           if (desc ? (a < c) : (a > c)) {
             buf[i] = c;
@@ -229,7 +252,7 @@ __device__ __forceinline__ void sort_desc_impl(unsigned long long* buf, int np, 
   }
 }
 
-__device__ __forceinline__ void sort_desc(unsigned long long* buf, int np, int tid) {
+__device__ __forceinline__ void sort_desc(u64* buf, int np, int tid) {
   if (np <= kThreads) sort_desc_impl<1>(buf, np, tid);
   else if (np == 2 * kThreads) sort_desc_impl<2>(buf, np, tid);
   else if (np == 4 * kThreads) sort_desc_impl<4>(buf, np, tid);
@@ -243,20 +266,34 @@ __device__ __forceinline__ int next_pow2_dev(int x) {
   return p;
 }
 
-// Sink / window part of a list row, its length and the -1 padding; clips the
-// heavy budget m to the room left in the row.  Returns the base length.
-__device__ __forceinline__ int write_list_base(int32_t* out, int n, int& m, int sink, int window,
-                                               int write_base, int list_width, int32_t* len_out,
-                                               int tid, int nthreads) {
-  int nbase = 0;
+// Row length n and heavy budget m of a row of sequence b (m clipped to the room
+// the list row leaves after the sink / window part), and that part's length.
+__device__ __forceinline__ void row_shape(const int32_t* lens, const int32_t* budgets, int b, int T,
+                                          int M, int sink, int window, int write_base, int list_width,
+                                          int& n, int& m, int& nbase) {
+  n = lens ? max(0, min(lens[b], T)) : T;
+  m = budgets ? budgets[b] : M;
+  m = max(0, min(min(m, M), n));
+  nbase = 0;
   if (write_base) {
     const int s_e = max(0, min(sink, n));
     const int w_e = max(0, min(window, n));
     const int win_start = max(n - w_e, s_e);
-    const int nwin = (w_e > 0 && win_start < n) ? n - win_start : 0;
-    nbase = s_e + nwin;
-    if (nbase == 0) {
-      nbase = 1;
+    nbase = s_e + ((w_e > 0 && win_start < n) ? n - win_start : 0);
+    if (nbase == 0) nbase = 1;
+  }
+  m = max(0, min(nbase + m, list_width) - nbase);
+}
+
+// Sink / window part of a list row, its length and the -1 padding.
+__device__ __forceinline__ void write_list_base(int32_t* out, int n, int m, int nbase, int sink,
+                                                int window, int write_base, int list_width,
+                                                int32_t* len_out, int tid, int nthreads) {
+  if (write_base) {
+    const int s_e = max(0, min(sink, n));
+    const int w_e = max(0, min(window, n));
+    const int win_start = max(n - w_e, s_e);
+    if (s_e + ((w_e > 0 && win_start < n) ? n - win_start : 0) == 0) {
       if (tid == 0 && list_width > 0) out[0] = n - 1;
     } else {
       for (int i = tid; i < nbase && i < list_width; i += nthreads)
@@ -264,95 +301,77 @@ __device__ __forceinline__ int write_list_base(int32_t* out, int n, int& m, int 
     }
   }
   const int total = min(nbase + m, list_width);
-  m = max(0, total - nbase);
   for (int i = total + tid; i < list_width; i += nthreads) out[i] = -1;
   if (len_out && tid == 0) *len_out = total;
-  return nbase;
 }
 
-struct RowRecord {   // per row, written by select_threshold_kernel
-  uint32_t range_lo;  // lowest key of the row (origin of the histogram bins)
-  uint32_t blo, bhi;  // key range of the bin holding the k-th key
-  int need;           // keys to take from that bin
-  int bin_count;      // keys in that bin
-  int shift;
-  int flag;           // 1: left to the one-workgroup kernel
-  int cur_above;      // append cursors of the row's global lists
-  int cur_cand;
-  int pad;
-};
+// Smallest shift for which [lo, hi] maps onto at most kBins bins.
+__device__ __forceinline__ int range_shift(u64 lo, u64 hi) {
+  const u64 span = hi - lo;
+  int shift = 0;
+  while ((span >> shift) >= (u64)kBins) ++shift;
+  return shift;
+}
 
-// Split path, last step, run by select_list_kernel for the rows the split
-// kernels prepared: the winners sit in `win` in no order.  Their bins (the
-// histogram bins above the k-th key's bin) already sort them coarsely, and a bin
-// rarely holds more than a few, so each winner is placed at
-//   (#winners in higher bins) + (#winners of its own bin that beat it)
-// and the `need` best candidates of the k-th bin follow, ranked the same way.
-// Crowded bins fall back to the bitonic sort.
-constexpr int kMaxBinForCounting = 128;
-
-__device__ __forceinline__ void finish_row(
-    const RowRecord& rec, uint32_t range_lo, const unsigned long long* __restrict__ win_g,
-    const unsigned long long* __restrict__ cand_g, unsigned long long* buf, unsigned long long* tmp,
-    unsigned long long* cand, uint32_t* hist, SelectShared& sh, bool counting_ok, int32_t* out,
-    int nbase, int m, int tid) {
-  const int need = rec.need, n_above = m - need, ncand = min(rec.bin_count, kCandCap);
+// Final step of both paths.  buf[0:n_above) holds the winners above the k-th
+// bin, cand[0:ncand) the k-th bin's entries of which the best `need` win; the
+// n_above + need winners are written in descending order at out[0:...).
+// Winners are placed by their level-0 bin (c - lo0) >> shift0 with counting ranks
+// when `counting_ok` (tmp then has 2 * cap_above slots) and no bin is crowded,
+// else by the bitonic sort.  All 1024 lanes; callers sync before; no barrier at
+// the end.
+__device__ __forceinline__ void order_and_write(u64* buf, int n_above, u64* cand, int ncand, int need,
+                                                u64 lo0, int shift0, u64* tmp, uint32_t* hist,
+                                                SelectShared& sh, bool counting_ok, int32_t* out,
+                                                int tid) {
   const int lane = tid & 63, wave = tid >> 6;
-  for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
-  for (int i = tid; i < n_above; i += kThreads) buf[i] = win_g[i];
-  for (int i = tid; i < ncand; i += kThreads) cand[i] = cand_g[i];
-  __syncthreads();
-
-  // ---- candidates of the k-th bin -------------------------------------------------
-  if (ncand <= kMaxBinForCounting) {
+  // ---- the k-th bin: rank its entries, the best `need` follow the winners ----------
+  if (ncand <= kMaxBinForCounting || need == ncand) {
     for (int i = tid; i < ncand; i += kThreads) {
-      const unsigned long long v = cand[i];
+      const u64 v = cand[i];
       int r = 0;
       for (int j = 0; j < ncand; ++j) r += cand[j] > v;
-      if (r < need) out[nbase + n_above + r] = (int32_t)(0xffffffffu - (uint32_t)(v & 0xffffffffull));
+      if (r < need) out[n_above + r] = composite_index(v);
     }
   } else {
     const int npc = next_pow2_dev(ncand);
     for (int i = ncand + tid; i < npc; i += kThreads) cand[i] = 0ull;
     __syncthreads();
     sort_desc(cand, npc, tid);
-    for (int i = tid; i < need; i += kThreads)
-      out[nbase + n_above + i] = (int32_t)(0xffffffffu - (uint32_t)(cand[i] & 0xffffffffull));
+    for (int i = tid; i < need; i += kThreads) out[n_above + i] = composite_index(cand[i]);
   }
+  if (n_above == 0) return;
 
-  // ---- winners ----------------------------------------------------------------------
+  // ---- winners above the bin ----------------------------------------------------------
   if (counting_ok) {
-    // slot of each winner inside its bin, bin populations
+    for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
+    __syncthreads();
     for (int i = tid; i < n_above; i += kThreads) {
-      const uint32_t k = (uint32_t)(buf[i] >> 32);
-      const int bin = (int)((k - range_lo) >> rec.shift);
+      const int bin = (int)((buf[i] - lo0) >> shift0);
       const uint32_t slot = atomicAdd(&hist[bin], 1u);
-      tmp[i] = ((unsigned long long)bin << 32) | slot;  // parked until the offsets are known
+      tmp[i] = ((u64)bin << 32) | slot;  // parked until the offsets are known
     }
     __syncthreads();
-    // descending exclusive scan: off[bin] = winners in higher bins; crowded-bin check
+    // descending exclusive scan over the bins, two per lane; crowded-bin check
     const int b0 = kBins - 1 - 2 * tid, b1 = b0 - 1;
     const int c0 = (int)hist[b0], c1 = (int)hist[b1];
     const int incl_w = wave_incl_scan(c0 + c1, lane);
-    int crowded = (c0 > kMaxBinForCounting || c1 > kMaxBinForCounting) ? 1 : 0;
-    crowded = __any(crowded);
+    const int crowded = __any((c0 > kMaxBinForCounting || c1 > kMaxBinForCounting) ? 1 : 0);
     if (lane == 63) sh.wsum[wave] = incl_w;
-    if (lane == 0) sh.wmin[wave] = (uint32_t)crowded;
+    if (lane == 0) sh.wflag[wave] = crowded;
     __syncthreads();
     int base = 0, any_crowded = 0;
     for (int w = 0; w < kWaves; ++w) {
       if (w < wave) base += sh.wsum[w];
-      any_crowded |= (int)sh.wmin[w];
+      any_crowded |= sh.wflag[w];
     }
     const int excl = base + incl_w - (c0 + c1);
     __syncthreads();
     if (!any_crowded) {
-      hist[b0] = (uint32_t)excl | ((uint32_t)c0 << 16);        // offset | population << 16
+      hist[b0] = (uint32_t)excl | ((uint32_t)c0 << 16);  // offset | population << 16
       hist[b1] = (uint32_t)(excl + c0) | ((uint32_t)c1 << 16);
       __syncthreads();
-      // group by bin: cand[] is free again and doubles as the grouped copy when it is
-      // large enough, else tmp's upper half (tmp has 2*cap_above slots)
-      unsigned long long* grouped = tmp + n_above;
+      u64* grouped = tmp + n_above;
       for (int i = tid; i < n_above; i += kThreads) {
         const int bin = (int)(tmp[i] >> 32);
         const int slot = (int)(tmp[i] & 0xffffffffull);
@@ -360,13 +379,12 @@ __device__ __forceinline__ void finish_row(
       }
       __syncthreads();
       for (int p = tid; p < n_above; p += kThreads) {
-        const unsigned long long v = grouped[p];
-        const uint32_t k = (uint32_t)(v >> 32);
-        const uint32_t h = hist[(k - range_lo) >> rec.shift];
+        const u64 v = grouped[p];
+        const uint32_t h = hist[(int)((v - lo0) >> shift0)];
         const int s0 = (int)(h & 0xffffu), c = (int)(h >> 16);
         int r = 0;
         for (int q = s0; q < s0 + c; ++q) r += grouped[q] > v;
-        out[nbase + s0 + r] = (int32_t)(0xffffffffu - (uint32_t)(v & 0xffffffffull));
+        out[s0 + r] = composite_index(v);
       }
       return;
     }
@@ -375,52 +393,344 @@ __device__ __forceinline__ void finish_row(
   for (int i = n_above + tid; i < np; i += kThreads) buf[i] = 0ull;
   __syncthreads();
   sort_desc(buf, np, tid);
-  for (int j = tid; j < n_above; j += kThreads)
-    out[nbase + j] = (int32_t)(0xffffffffu - (uint32_t)(buf[j] & 0xffffffffull));
+  for (int j = tid; j < n_above; j += kThreads) out[j] = composite_index(buf[j]);
 }
 
+// ---------------------------------------------------------------------------
+// threshold from a sample
+// ---------------------------------------------------------------------------
+// A pool of kPoolCap composites can be relied on to hold a row's m winners when
+// it is filled with everything above a threshold aimed at max(2m, 1024) entries.
+__host__ __device__ __forceinline__ bool sampling_ok(int m) {
+  const int target = 2 * m > 1024 ? 2 * m : 1024;
+  return target + target / 2 <= kPoolCap;
+}
+
+// All THREADS lanes; returns (to every lane) a key tau such that about
+// max(2m, 1024) of the row's n scores have keys >= tau.  The estimate comes from
+// a fixed sample of the row -- runs of 64 consecutive scores at evenly spaced
+// places, 4096 scores in all (16384 for rows beyond 262144) -- whose r-th largest
+// key is located with the same histogram refinement as everywhere else; tau is
+// the lower edge of its bin.  Every workgroup that calls this for a row gets the
+// same tau.  Needs n > kPoolCap.  Ends with a barrier.
+template <int THREADS, bool VEC>
+__device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, int m, uint32_t* hist,
+                                                     SelectShared& sh, int tid) {
+  constexpr int kMaxQ = 16384 / 4 / THREADS;  // float4 groups per lane at most
+  const int lane = tid & 63, wave = tid >> 6;
+  const int nsample = n <= 262144 ? 4096 : 16384;
+  const int nchunk = nsample / 64;
+  const int nq = nsample / 4 / THREADS;  // 1 or 4 (1024 lanes), 4 or 16 (256 lanes)
+  uint32_t key[kMaxQ * 4];
+#pragma unroll
+  for (int j = 0; j < kMaxQ; ++j) {
+    if (j < nq) {
+      const int q = j * THREADS + tid;
+      const int chunk = q >> 4;
+      const int at = (int)(((int64_t)chunk * n / nchunk) & ~3ll) + (q & 15) * 4;
+      float x[4];
+      if (VEC) {
+        const float4 v = *reinterpret_cast<const float4*>(row + at);
+        x[0] = v.x;
+        x[1] = v.y;
+        x[2] = v.z;
+        x[3] = v.w;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) x[c] = row[at + c];
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) key[j * 4 + c] = score_to_key(x[c]);
+    }
+  }
+  uint32_t kmin = 0xffffffffu, kmax = 0u;
+#pragma unroll
+  for (int j = 0; j < kMaxQ; ++j) {
+    if (j < nq) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        kmin = min(kmin, key[j * 4 + c]);
+        kmax = max(kmax, key[j * 4 + c]);
+      }
+    }
+  }
+#pragma unroll
+  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
+    kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
+    kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, SOCKET_WAVE));
+  }
+  if (lane == 0) {
+    sh.wmin[wave] = kmin;
+    sh.wmax[wave] = kmax;
+  }
+  __syncthreads();
+  const int target = max(2 * m, 1024);
+  const int r = (int)min((int64_t)nsample, ((int64_t)target * nsample + n - 1) / n);
+  if (tid == 0) {
+    for (int w = 1; w < THREADS / SOCKET_WAVE; ++w) {
+      kmin = min(kmin, (uint32_t)sh.wmin[w]);
+      kmax = max(kmax, (uint32_t)sh.wmax[w]);
+    }
+    sh.lo = kmin;
+    sh.hi = max(kmin, kmax);
+    sh.need = r;
+    sh.done = 0;
+  }
+  __syncthreads();
+  const int fine = max(4, r / 8);  // a bin this small pins tau well enough
+  for (int iter = 0; iter < 4; ++iter) {
+    const uint32_t lo = (uint32_t)sh.lo, hi = (uint32_t)sh.hi;
+    const int need_in = sh.need;
+    const int shift = range_shift(lo, hi);
+    for (int i = tid; i < kBins; i += THREADS) hist[i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kMaxQ; ++j) {
+      if (j < nq) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const uint32_t k = key[j * 4 + c];
+          if (k >= lo && k <= hi) atomicAdd(&hist[(k - lo) >> shift], 1u);
+        }
+      }
+    }
+    __syncthreads();
+    find_bin<THREADS>(hist, need_in, 1, sh, tid);
+    if (tid == 0) {
+      const uint32_t blo = lo + ((uint32_t)sh.found_bin << shift);
+      const uint32_t bspan = (shift == 0) ? 0u : ((1u << shift) - 1u);
+      sh.lo = blo;
+      sh.hi = (hi - blo < bspan) ? hi : blo + bspan;
+      sh.need = need_in - sh.found_before;
+      sh.done = (sh.found_count <= fine || shift == 0) ? 1 : 0;
+    }
+    __syncthreads();
+    if (sh.done) break;
+  }
+  const uint32_t tau = (uint32_t)sh.lo;
+  __syncthreads();
+  return tau;
+}
+
+// ---------------------------------------------------------------------------
+// slices: everything at or above the row's sampled threshold
+// ---------------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(kLocThreads) void select_local_kernel(
+    const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
+    const int32_t* __restrict__ budgets, int Hq, int T, int M, int sink, int window, int write_base,
+    int list_width, int S, int k_cap, u64* __restrict__ loc, int32_t* __restrict__ loc_count) {
+  __shared__ uint32_t hist[kBins];
+  __shared__ SelectShared sh;
+  const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  int n, m, nbase;
+  row_shape(lens, budgets, rowi / Hq, T, M, sink, window, write_base, list_width, n, m, nbase);
+  const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
+  const int64_t slot = (int64_t)rowi * S + s;
+  // short rows are pooled whole by the row kernel; it also takes over when no
+  // threshold can be relied on
+  if (m == 0 || n <= kPoolCap || end <= begin || !sampling_ok(m)) {
+    if (tid == 0) loc_count[slot] = 0;
+    return;
+  }
+  const float* row = scores + (int64_t)rowi * score_stride;
+  const uint32_t tau = sample_threshold<kLocThreads, VEC>(row, n, m, hist, sh, tid);
+
+  // the slice's keys, 64 per lane: element e of lane t is index
+  // begin + ((e / 4) * 256 + t) * 4 + e % 4; places past the row's end get key 0
+  // and are excluded by their index
+  uint32_t key[kLocPerLane];
+#pragma unroll
+  for (int u = 0; u < kLocPerLane / 4; ++u) {
+    const int i0 = begin + (u * kLocThreads + tid) * 4;
+    float x[4] = {0.f, 0.f, 0.f, 0.f};
+    if (VEC && i0 + 4 <= end) {
+      const float4 v = *reinterpret_cast<const float4*>(row + i0);
+      x[0] = v.x;
+      x[1] = v.y;
+      x[2] = v.z;
+      x[3] = v.w;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (i0 + c < end) x[c] = row[i0 + c];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) key[u * 4 + c] = score_to_key(x[c]);
+  }
+  auto index_of = [&](int e) { return begin + ((e >> 2) * kLocThreads + tid) * 4 + (e & 3); };
+
+  int cnt = 0;
+#pragma unroll
+  for (int e = 0; e < kLocPerLane; ++e) cnt += (key[e] >= tau && index_of(e) < end) ? 1 : 0;
+  const int incl = wave_incl_scan(cnt, lane);
+  if (lane == 63) sh.wsum[wave] = incl;
+  __syncthreads();
+  int at = incl - cnt, total = 0;
+#pragma unroll
+  for (int w = 0; w < kLocWaves; ++w) {
+    if (w < wave) at += sh.wsum[w];
+    total += sh.wsum[w];
+  }
+  if (total > k_cap) {  // more than the slice's share of the pool: the row kernel starts over
+    if (tid == 0) loc_count[slot] = k_cap + 1;
+    return;
+  }
+  u64* my = loc + slot * k_cap;
+#pragma unroll
+  for (int e = 0; e < kLocPerLane; ++e) {
+    const int i = index_of(e);
+    if (key[e] >= tau && i < end) my[at++] = composite(key[e], i);
+  }
+  if (tid == 0) loc_count[slot] = total;
+}
+
+// ---------------------------------------------------------------------------
+// rows
+// ---------------------------------------------------------------------------
 template <bool VEC>
 __global__ __launch_bounds__(kThreads) void select_list_kernel(
     const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
     const int32_t* __restrict__ budgets, const uint32_t* __restrict__ row_range, int range_parts,
     int Hq, int T, int M, int sink, int window, int write_base, int32_t* __restrict__ sparse_list,
     int64_t list_stride, int list_width, int32_t* __restrict__ sparse_len, int cap_above,
-    const RowRecord* __restrict__ records, const unsigned long long* __restrict__ win_g,
-    const unsigned long long* __restrict__ cand_g, int counting_ok) {
+    int counting_ok, int use_pool, const u64* __restrict__ loc, const int32_t* __restrict__ loc_count,
+    int S, int k_cap) {
   __shared__ uint32_t hist[kBins];
   __shared__ SelectShared sh;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  unsigned long long* buf = reinterpret_cast<unsigned long long*>(lds_raw);  // winners
-  unsigned long long* cand = buf + cap_above;                                // keys of the k-th bin
-  unsigned long long* tmp = cand + kCandCap;  // 2*cap_above more slots when counting_ok
+  u64* buf = reinterpret_cast<u64*>(lds_raw);  // winners                  [cap_above]
+  u64* cand = buf + cap_above;                 // entries of the k-th bin  [kCandCap]
+  u64* pool = cand + kCandCap;                 // pooled composites        [kPoolCap] if use_pool
+  u64* tmp = pool + (use_pool ? kPoolCap : 0); // counting placement       [2*cap_above] if counting_ok
 
   const int rowi = blockIdx.x;
   const int b = rowi / Hq;
   const int tid = threadIdx.x;
   const int lane = tid & (SOCKET_WAVE - 1);
   const int wave = tid / SOCKET_WAVE;
-  const int n = lens ? max(0, min(lens[b], T)) : T;
-  int m = budgets ? budgets[b] : M;
-  m = max(0, min(min(m, M), n));
+  int n, m, nbase;
+  row_shape(lens, budgets, b, T, M, sink, window, write_base, list_width, n, m, nbase);
   const float* row = scores + (int64_t)rowi * score_stride;
   int32_t* out = sparse_list + (int64_t)rowi * list_stride;
-
-  // ---- sink / window part, length, padding ---------------------------------
-  const int nbase = write_list_base(out, n, m, sink, window, write_base, list_width,
-                                    sparse_len ? sparse_len + rowi : nullptr, tid, kThreads);
+  write_list_base(out, n, m, nbase, sink, window, write_base, list_width,
+                  sparse_len ? sparse_len + rowi : nullptr, tid, kThreads);
   if (m == 0) return;
+  int32_t* heavy = out + nbase;
 
-  // split path: the slice kernels have located the k-th key and gathered the
-  // winners unless the row is flagged (then it is done here from scratch)
-  if (records) {
-    const RowRecord rec = records[rowi];
-    if (!rec.flag) {
-      finish_row(rec, rec.range_lo, win_g + (int64_t)rowi * cap_above, cand_g + (int64_t)rowi * kCandCap,
-                 buf, tmp, cand, hist, sh, counting_ok != 0, out, nbase, m, tid);
+  // ================================ pooled select ======================================
+  if (use_pool) {
+    if (tid == 0) {
+      sh.fill_above = 0;
+      sh.fill_cand = 0;
+      sh.fill_pool = 0;
+    }
+    int total = -1;  // uniform; stays -1 when no pool could be formed
+    if (n <= kPoolCap) {  // the whole row
+      for_each_in<VEC, kThreads>(row, 0, n, tid,
+                                 [&](int i, float x) { pool[i] = composite(score_to_key(x), i); });
+      total = n;
+    } else if (loc) {  // what the slices found above the sampled threshold
+      int sum = 0;
+      bool ok = true;
+      for (int s = 0; s < S; ++s) {
+        const int cnt = loc_count[(int64_t)rowi * S + s];
+        ok = ok && cnt <= k_cap;
+        sum += cnt;
+      }
+      if (ok && sum >= m && sum <= kPoolCap) {
+        int at = 0;
+        for (int s = 0; s < S; ++s) {
+          const int cnt = loc_count[(int64_t)rowi * S + s];
+          const u64* src = loc + ((int64_t)rowi * S + s) * k_cap;
+          for (int i = tid; i < cnt; i += kThreads) pool[at + i] = src[i];
+          at += cnt;
+        }
+        total = sum;
+      }
+    } else if (sampling_ok(m)) {  // one workgroup: threshold from the sample, one pass
+      const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
+      for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
+        const uint32_t k = score_to_key(x);
+        wave_append(k >= tau, composite(k, i), &sh.fill_pool, pool, kPoolCap);
+      });
+      __syncthreads();
+      const int got = sh.fill_pool;
+      if (got >= m && got <= kPoolCap) total = got;
+    }
+    __syncthreads();
+    if (total >= 0) {
+      // range of the pooled composites
+      u64 cmin = ~0ull, cmax = 0ull;
+      for (int i = tid; i < total; i += kThreads) {
+        const u64 v = pool[i];
+        cmin = min(cmin, v);
+        cmax = max(cmax, v);
+      }
+#pragma unroll
+      for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
+        cmin = min(cmin, shfl_xor_u64(cmin, d));
+        cmax = max(cmax, shfl_xor_u64(cmax, d));
+      }
+      if (lane == 0) {
+        sh.wmin[wave] = cmin;
+        sh.wmax[wave] = cmax;
+      }
+      __syncthreads();
+      if (tid == 0) {
+        for (int w = 1; w < kWaves; ++w) {
+          cmin = min(cmin, sh.wmin[w]);
+          cmax = max(cmax, sh.wmax[w]);
+        }
+        sh.lo = cmin;
+        sh.hi = max(cmin, cmax);
+        sh.need = m;
+        sh.done = 0;
+      }
+      __syncthreads();
+      const u64 lo0 = sh.lo;
+      const int shift0 = range_shift(sh.lo, sh.hi);
+      // refinement on the composites; they are distinct, so it ends with a bin of
+      // at most kCandCap entries (ties need no special case here)
+      for (int iter = 0; iter < 8; ++iter) {
+        const u64 lo = sh.lo, hi = sh.hi;
+        const int need_in = sh.need;
+        const int shift = range_shift(lo, hi);
+        for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
+        __syncthreads();
+        for (int i = tid; i < total; i += kThreads) {
+          const u64 v = pool[i];
+          if (v >= lo && v <= hi) atomicAdd(&hist[(int)((v - lo) >> shift)], 1u);
+        }
+        __syncthreads();
+        find_bin<kThreads>(hist, need_in, 1, sh, tid);
+        if (tid == 0) {
+          const u64 blo = lo + ((u64)sh.found_bin << shift);
+          const u64 bspan = (shift == 0) ? 0ull : ((1ull << shift) - 1ull);
+          sh.lo = blo;
+          sh.hi = (hi - blo < bspan) ? hi : blo + bspan;
+          sh.need = need_in - sh.found_before;
+          sh.done = (sh.found_count <= kCandCap || shift == 0) ? 1 : 0;
+        }
+        __syncthreads();
+        if (sh.done) break;
+      }
+      const u64 blo = sh.lo, bhi = sh.hi;
+      const int need = sh.need;
+      for (int i = tid; i < total; i += kThreads) {
+        const u64 v = pool[i];
+        wave_append(v > bhi, v, &sh.fill_above, buf, cap_above);
+        wave_append(v >= blo && v <= bhi, v, &sh.fill_cand, cand, kCandCap);
+      }
+      __syncthreads();
+      order_and_write(buf, m - need, cand, min(sh.fill_cand, kCandCap), need, lo0, shift0, tmp, hist, sh,
+                      counting_ok != 0, heavy, tid);
       return;
     }
   }
 
+  // ================================ from scratch ======================================
   // ---- key range of the row -----------------------------------------------------
   {
     uint32_t kmin = 0xffffffffu, kmax = 0u;
@@ -431,7 +741,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         kmax = max(kmax, rr[2 * i + 1]);
       }
     } else {
-      for_each_score<VEC>(row, n, tid, [&](int, float x) {
+      for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int, float x) {
         const uint32_t k = score_to_key(x);
         kmin = min(kmin, k);
         kmax = max(kmax, k);
@@ -449,8 +759,8 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     __syncthreads();
     if (tid == 0) {
       for (int w = 1; w < kWaves; ++w) {
-        kmin = min(kmin, sh.wmin[w]);
-        kmax = max(kmax, sh.wmax[w]);
+        kmin = min(kmin, (uint32_t)sh.wmin[w]);
+        kmax = max(kmax, (uint32_t)sh.wmax[w]);
       }
       sh.lo = kmin;
       sh.hi = max(kmin, kmax);
@@ -462,28 +772,27 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     }
     __syncthreads();
   }
+  const uint32_t lo0 = (uint32_t)sh.lo;
+  const int shift0 = range_shift(sh.lo, sh.hi);
 
   // ---- range refinement -------------------------------------------------------
   for (int iter = 0; iter < 4; ++iter) {
-    const uint32_t lo = sh.lo, hi = sh.hi;
+    const uint32_t lo = (uint32_t)sh.lo, hi = (uint32_t)sh.hi;
     const int need_in = sh.need;
-    const uint32_t span = hi - lo;  // width - 1
-    int shift = 0;
-    while ((span >> shift) >= (uint32_t)kBins) ++shift;
+    const int shift = range_shift(lo, hi);
     for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
     __syncthreads();
-    for_each_score<VEC>(row, n, tid, [&](int, float x) {
+    for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int, float x) {
       const uint32_t k = score_to_key(x);
       if (k >= lo && k <= hi) atomicAdd(&hist[(k - lo) >> shift], 1u);
     });
     __syncthreads();
-    find_bin(hist, need_in, 1, sh, tid);
+    find_bin<kThreads>(hist, need_in, 1, sh, tid);
     if (tid == 0) {
       const uint32_t blo = lo + ((uint32_t)sh.found_bin << shift);
       const uint32_t bspan = (shift == 0) ? 0u : ((1u << shift) - 1u);
-      const uint32_t bhi = (hi - blo < bspan) ? hi : blo + bspan;
       sh.lo = blo;
-      sh.hi = bhi;
+      sh.hi = (hi - blo < bspan) ? hi : blo + bspan;
       sh.need = need_in - sh.found_before;
       sh.bin_count = sh.found_count;
       sh.done = (sh.found_count <= kCandCap || shift == 0) ? 1 : 0;
@@ -492,10 +801,9 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     if (sh.done) break;
   }
 
-  const uint32_t blo = sh.lo, bhi = sh.hi;
-  const int need = sh.need;         // keys to take from [blo, bhi]
+  const uint32_t blo = (uint32_t)sh.lo, bhi = (uint32_t)sh.hi;
+  const int need = sh.need;  // keys to take from [blo, bhi]
   const int bin_count = sh.bin_count;
-  const int n_above = m - need;     // keys > bhi, all taken
   const bool mass_ties = bin_count > kCandCap;  // then blo == bhi
 
   if (mass_ties) {
@@ -504,22 +812,22 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     const int binw = (n + kBins - 1) / kBins;
     for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
     __syncthreads();
-    for_each_score<VEC>(row, n, tid, [&](int i, float x) {
+    for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
       if (score_to_key(x) == blo) atomicAdd(&hist[i / binw], 1u);
     });
     __syncthreads();
-    find_bin(hist, need, 0, sh, tid);
+    find_bin<kThreads>(hist, need, 0, sh, tid);
     if (wave == 0) {
       int rest = need - sh.found_before;  // >= 1 ties to take inside this index range
       const int i0 = sh.found_bin * binw, i1 = min(n, i0 + binw);
       int star = i0;
       for (int base = i0; base < i1 && rest > 0; base += SOCKET_WAVE) {
         const int i = base + lane;
-        const bool eq = (i < i1) && (score_to_key(row[i]) == blo);
-        const unsigned long long mask = __ballot(eq);
+        const bool eq = (i < i1) && (score_to_key(row[min(i, i1 - 1)]) == blo);
+        const u64 mask = __ballot(eq);
         const int c = __popcll(mask);
         if (c >= rest) {
-          unsigned long long mm = mask;  // its rest-th set bit is the last tie taken
+          u64 mm = mask;  // its rest-th set bit is the last tie taken
           for (int r = 1; r < rest; ++r) mm &= mm - 1;
           star = base + (__ffsll((long long)mm) - 1);
           rest = 0;
@@ -534,9 +842,9 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
 
   // ---- collect ------------------------------------------------------------------
   const int idx_star = sh.idx_star;
-  for_each_score<VEC>(row, n, tid, [&](int i, float x) {
+  for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
     const uint32_t k = score_to_key(x);
-    const unsigned long long v = ((unsigned long long)k << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
+    const u64 v = composite(k, i);
     const bool in_bin = k >= blo && k <= bhi;
     // mass ties: the ties with the lowest indices are winners outright (there can
     // be more of them than the candidate list holds)
@@ -544,223 +852,11 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     wave_append(!mass_ties && in_bin, v, &sh.fill_cand, cand, kCandCap);
   });
   __syncthreads();
-  // mass ties: sh.fill_above == m, no candidates; else fill_above == n_above, fill_cand == bin_count
-  const int ncand = min(sh.fill_cand, kCandCap);
-  if (ncand > need) {  // uniform: rank the bin's keys, the best `need` of them win
-    const int npc = next_pow2_dev(ncand);
-    for (int i = ncand + tid; i < npc; i += kThreads) cand[i] = 0ull;
-    __syncthreads();
-    sort_desc(cand, npc, tid);
-  }
-  if (!mass_ties)
-    for (int i = tid; i < need; i += kThreads) buf[n_above + i] = cand[i];
-  const int np = next_pow2_dev(m);
-  for (int i = m + tid; i < np; i += kThreads) buf[i] = 0ull;
-  __syncthreads();
-  sort_desc(buf, np, tid);
-
-  for (int j = tid; j < m; j += kThreads)
-    out[nbase + j] = (int32_t)(0xffffffffu - (uint32_t)(buf[j] & 0xffffffffull));
-}
-
-// ---------------------------------------------------------------------------
-// split path
-// ---------------------------------------------------------------------------
-constexpr int kSliceLen = 16384;   // scores per (slice, row) workgroup
-constexpr int kSliceThreads = 256;
-constexpr int kSliceWaves = kSliceThreads / SOCKET_WAVE;
-
-__device__ __forceinline__ void row_shape(const int32_t* lens, const int32_t* budgets, int b, int T,
-                                          int M, int sink, int window, int write_base, int list_width,
-                                          int& n, int& m) {
-  n = lens ? max(0, min(lens[b], T)) : T;
-  m = budgets ? budgets[b] : M;
-  m = max(0, min(min(m, M), n));
-  int nbase = 0;
-  if (write_base) {
-    const int s_e = max(0, min(sink, n));
-    const int w_e = max(0, min(window, n));
-    const int win_start = max(n - w_e, s_e);
-    nbase = s_e + ((w_e > 0 && win_start < n) ? n - win_start : 0);
-    if (nbase == 0) nbase = 1;
-  }
-  m = max(0, min(nbase + m, list_width) - nbase);
-}
-
-// Key range of the row from `parts` (min, max) pairs; every lane gets it.
-template <int THREADS>
-__device__ __forceinline__ void reduce_range(const uint32_t* rr, int parts, int tid, uint32_t* red,
-                                             uint32_t& lo, uint32_t& hi) {
-  uint32_t kmin = 0xffffffffu, kmax = 0u;
-  for (int i = tid; i < parts; i += THREADS) {
-    kmin = min(kmin, rr[2 * i]);
-    kmax = max(kmax, rr[2 * i + 1]);
-  }
-#pragma unroll
-  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
-    kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
-    kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, SOCKET_WAVE));
-  }
-  constexpr int W = THREADS / SOCKET_WAVE;
-  if ((tid & 63) == 0) {
-    red[2 * (tid >> 6)] = kmin;
-    red[2 * (tid >> 6) + 1] = kmax;
-  }
-  __syncthreads();
-  lo = 0xffffffffu;
-  hi = 0u;
-  for (int w = 0; w < W; ++w) {
-    lo = min(lo, red[2 * w]);
-    hi = max(hi, red[2 * w + 1]);
-  }
-  hi = max(lo, hi);
-  __syncthreads();
-}
-
-__device__ __forceinline__ int range_shift(uint32_t lo, uint32_t hi) {
-  const uint32_t span = hi - lo;
-  int shift = 0;
-  while ((span >> shift) >= (uint32_t)kBins) ++shift;
-  return shift;
-}
-
-// Per-slice (min, max) keys, for callers that have no ranges from the scorer.
-template <bool VEC>
-__global__ __launch_bounds__(kSliceThreads) void select_range_kernel(
-    const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens, int Hq,
-    int T, uint32_t* __restrict__ parts, int S) {
-  __shared__ uint32_t red[2 * kSliceWaves];
-  const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
-  const int n = lens ? max(0, min(lens[rowi / Hq], T)) : T;
-  const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
-  uint32_t kmin = 0xffffffffu, kmax = 0u;
-  if (begin < end) {
-    for_each_in<VEC, kSliceThreads>(scores + (int64_t)rowi * score_stride, begin, end, tid, [&](int, float x) {
-      const uint32_t k = score_to_key(x);
-      kmin = min(kmin, k);
-      kmax = max(kmax, k);
-    });
-  }
-#pragma unroll
-  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
-    kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
-    kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, SOCKET_WAVE));
-  }
-  if ((tid & 63) == 0) {
-    red[2 * (tid >> 6)] = kmin;
-    red[2 * (tid >> 6) + 1] = kmax;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    for (int w = 1; w < kSliceWaves; ++w) {
-      kmin = min(kmin, red[2 * w]);
-      kmax = max(kmax, red[2 * w + 1]);
-    }
-    parts[((int64_t)rowi * S + s) * 2] = kmin;
-    parts[((int64_t)rowi * S + s) * 2 + 1] = kmax;
-  }
-}
-
-template <bool VEC>
-__global__ __launch_bounds__(kSliceThreads) void select_hist_kernel(
-    const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
-    const uint32_t* __restrict__ row_range, int range_parts, int Hq, int T,
-    uint32_t* __restrict__ hist_parts, int S) {
-  __shared__ uint32_t hist[kBins];
-  __shared__ uint32_t red[2 * kSliceWaves];
-  const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
-  const int n = lens ? max(0, min(lens[rowi / Hq], T)) : T;
-  const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
-  uint32_t* dst = hist_parts + ((int64_t)rowi * S + s) * kBins;
-  for (int i = tid; i < kBins; i += kSliceThreads) hist[i] = 0;
-  uint32_t lo, hi;
-  reduce_range<kSliceThreads>(row_range + (int64_t)rowi * range_parts * 2, range_parts, tid, red, lo, hi);
-  if (begin < end) {
-    const int shift = range_shift(lo, hi);
-    for_each_in<VEC, kSliceThreads>(scores + (int64_t)rowi * score_stride, begin, end, tid, [&](int, float x) {
-      const uint32_t k = score_to_key(x);
-      if (k >= lo && k <= hi) atomicAdd(&hist[(k - lo) >> shift], 1u);
-    });
-  }
-  __syncthreads();
-  for (int i = tid; i < kBins; i += kSliceThreads) dst[i] = hist[i];
-}
-
-__global__ __launch_bounds__(kThreads) void select_threshold_kernel(
-    const int32_t* __restrict__ lens, const int32_t* __restrict__ budgets,
-    const uint32_t* __restrict__ row_range, int range_parts, int Hq, int T, int M, int sink, int window,
-    int write_base, int list_width, const uint32_t* __restrict__ hist_parts, int S,
-    RowRecord* __restrict__ records) {
-  __shared__ uint32_t hist[kBins];
-  __shared__ uint32_t red[2 * kWaves];
-  __shared__ SelectShared sh;
-  const int rowi = blockIdx.x, tid = threadIdx.x;
-  int n, m;
-  row_shape(lens, budgets, rowi / Hq, T, M, sink, window, write_base, list_width, n, m);
-  uint32_t lo, hi;
-  reduce_range<kThreads>(row_range + (int64_t)rowi * range_parts * 2, range_parts, tid, red, lo, hi);
-  RowRecord rec{lo, 0u, 0u, 0, 0, 0, 0, 0, 0, 0};
-  if (m > 0) {
-    const uint32_t* src = hist_parts + (int64_t)rowi * S * kBins;
-    uint32_t c0 = 0, c1 = 0;
-    for (int s = 0; s < S; ++s) {
-      c0 += src[(int64_t)s * kBins + 2 * tid];
-      c1 += src[(int64_t)s * kBins + 2 * tid + 1];
-    }
-    hist[2 * tid] = c0;
-    hist[2 * tid + 1] = c1;
-    __syncthreads();
-    find_bin(hist, m, 1, sh, tid);
-    const int shift = range_shift(lo, hi);
-    const uint32_t blo = lo + ((uint32_t)sh.found_bin << shift);
-    const uint32_t bspan = (shift == 0) ? 0u : ((1u << shift) - 1u);
-    rec.blo = blo;
-    rec.bhi = (hi - blo < bspan) ? hi : blo + bspan;
-    rec.need = m - sh.found_before;
-    rec.bin_count = sh.found_count;
-    rec.shift = shift;
-    rec.flag = sh.found_count > kCandCap ? 1 : 0;
-  }
-  if (tid == 0) records[rowi] = rec;
-}
-
-// Winners and bin candidates of the slice are gathered in LDS first, so each
-// workgroup makes two global atomics (to reserve its runs in the row's lists),
-// not one per wave and load.
-template <bool VEC>
-__global__ __launch_bounds__(kSliceThreads) void select_collect_kernel(
-    const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens, int Hq,
-    int T, RowRecord* __restrict__ records, unsigned long long* __restrict__ win, int cap_above,
-    unsigned long long* __restrict__ cand) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  unsigned long long* lw = reinterpret_cast<unsigned long long*>(lds_raw);  // [cap_above]
-  unsigned long long* lc = lw + cap_above;                                  // [kCandCap]
-  __shared__ int cur[4];  // local counts, then global bases
-  const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
-  const int n = lens ? max(0, min(lens[rowi / Hq], T)) : T;
-  const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
-  RowRecord* rec = records + rowi;
-  if (begin >= end || rec->flag || rec->need <= 0) return;
-  const uint32_t blo = rec->blo, bhi = rec->bhi;
-  if (tid < 2) cur[tid] = 0;
-  __syncthreads();
-  for_each_in<VEC, kSliceThreads>(scores + (int64_t)rowi * score_stride, begin, end, tid, [&](int i, float x) {
-    const uint32_t k = score_to_key(x);
-    const unsigned long long v = ((unsigned long long)k << 32) | (unsigned long long)(0xffffffffu - (uint32_t)i);
-    wave_append(k > bhi, v, &cur[0], lw, cap_above);
-    wave_append(k >= blo && k <= bhi, v, &cur[1], lc, kCandCap);
-  });
-  __syncthreads();
-  const int nw = min(cur[0], cap_above), nc = min(cur[1], kCandCap);
-  if (tid == 0) cur[2] = nw ? atomicAdd(&rec->cur_above, nw) : 0;
-  if (tid == 1) cur[3] = nc ? atomicAdd(&rec->cur_cand, nc) : 0;
-  __syncthreads();
-  unsigned long long* w = win + (int64_t)rowi * cap_above + cur[2];
-  unsigned long long* c = cand + (int64_t)rowi * kCandCap + cur[3];
-  for (int i = tid; i < nw; i += kSliceThreads)
-    if (cur[2] + i < cap_above) w[i] = lw[i];
-  for (int i = tid; i < nc; i += kSliceThreads)
-    if (cur[3] + i < kCandCap) c[i] = lc[i];
+  // mass ties: all m winners are in buf and there are no candidates
+  const int ncand = mass_ties ? 0 : min(sh.fill_cand, kCandCap);
+  const int n_above = mass_ties ? m : m - need;
+  order_and_write(buf, n_above, cand, ncand, mass_ties ? 0 : need, (u64)lo0 << 32, shift0 + 32, tmp, hist,
+                  sh, counting_ok != 0, heavy, tid);
 }
 
 int next_pow2(int x) {
@@ -769,38 +865,45 @@ int next_pow2(int x) {
   return p;
 }
 
+// Slices pay off once a row is several of them long.  Each gets room for k_cap
+// composites, several times an even share of the pool; 0 means "one workgroup
+// per row does everything".
+int slice_cap(int T, int m_max, int* S_out) {
+  const int S = (T + kSliceLen - 1) / kSliceLen;
+  *S_out = S;
+  if (S < 4 || S > kMaxSlices || m_max <= 0 || !sampling_ok(m_max)) return 0;
+  int k = 4 * kPoolCap / S;
+  if (k > 4096) k = 4096;
+  if (k < 512) k = 512;
+  return k;
+}
+
 struct SplitLayout {
-  int S;
-  size_t off_records, off_parts, off_hist, off_win, off_cand, total;
+  size_t off_loc, off_count, total;
 };
 
-SplitLayout split_layout(int rows, int T, int cap_above) {
+SplitLayout split_layout(int rows, int S, int k_cap) {
   SplitLayout l;
-  l.S = (T + kSliceLen - 1) / kSliceLen;
   size_t o = 0;
   auto take = [&](size_t bytes) {
     const size_t at = o;
     o += (bytes + 255) / 256 * 256;
     return at;
   };
-  l.off_records = take((size_t)rows * sizeof(RowRecord));
-  l.off_parts = take((size_t)rows * l.S * 2 * sizeof(uint32_t));
-  l.off_hist = take((size_t)rows * l.S * kBins * sizeof(uint32_t));
-  l.off_win = take((size_t)rows * cap_above * sizeof(unsigned long long));
-  l.off_cand = take((size_t)rows * kCandCap * sizeof(unsigned long long));
+  l.off_loc = take((size_t)rows * S * k_cap * sizeof(u64));
+  l.off_count = take((size_t)rows * S * sizeof(int32_t));
   l.total = o;
   return l;
 }
 
-// The split path pays off once a row is several slices long.
-bool use_split(int T) { return T >= 4 * kSliceLen; }
-
 }  // namespace
 
 extern "C" size_t socket_select_workspace_bytes(int B, int Hq, int T, int M) {
-  if (B <= 0 || Hq <= 0 || T <= 0 || M < 0 || !use_split(T)) return 0;
-  const int m_max = M < T ? M : T;
-  return split_layout(B * Hq, T, next_pow2(m_max > 0 ? m_max : 1)).total;
+  if (B <= 0 || Hq <= 0 || T <= 0 || M < 0) return 0;
+  int S = 0;
+  const int k_cap = slice_cap(T, M < T ? M : T, &S);
+  if (k_cap == 0) return 0;
+  return split_layout(B * Hq, S, k_cap).total;
 }
 
 extern "C" int socket_select_list(const float* scores, int64_t score_stride, const int32_t* lens,
@@ -814,68 +917,64 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
   SOCKET_REQUIRE(score_stride >= T && list_width >= 0 && list_stride >= list_width, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(row_range == nullptr || range_parts > 0, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(M <= SOCKET_TOPK_MAX_M, SOCKET_ERR_UNSUPPORTED);
-  const int m_max = M < T ? M : T;
-  const int cap_above = next_pow2(m_max > 0 ? m_max : 1);
-  const size_t lds_base = (size_t)(cap_above + kCandCap) * sizeof(unsigned long long);
-  const SocketDeviceLimits& lim = socket_device_limits();
-  const size_t lds_static = kBins * 4 + sizeof(SelectShared) + 256;
-  SOCKET_REQUIRE(lds_base + lds_static <= (size_t)lim.max_lds_per_block, SOCKET_ERR_UNSUPPORTED);
-  // ranking by bins needs two more arrays of cap_above slots
-  const size_t lds_counting = lds_base + (size_t)2 * cap_above * sizeof(unsigned long long);
-  const int counting_ok = lds_counting + lds_static <= (size_t)lim.max_lds_per_block ? 1 : 0;
-  const bool vec = socket_aligned16(scores) && (score_stride % 4 == 0);
-  hipStream_t s = (hipStream_t)stream;
   const int rows = B * Hq;
   SOCKET_REQUIRE(rows <= 65535, SOCKET_ERR_SHAPE);
+  const int m_max = M < T ? M : T;
+  const int cap_above = next_pow2(m_max > 0 ? m_max : 1);
+  const SocketDeviceLimits& lim = socket_device_limits();
+  const size_t lds_max = (size_t)lim.max_lds_per_block;
+  const size_t lds_static = kBins * 4 + sizeof(SelectShared) + 256;
+  size_t lds = (size_t)(cap_above + kCandCap) * sizeof(u64);
+  SOCKET_REQUIRE(lds + lds_static <= lds_max, SOCKET_ERR_UNSUPPORTED);
+  const bool vec = socket_aligned16(scores) && (score_stride % 4 == 0);
+  hipStream_t s = (hipStream_t)stream;
 
-  const RowRecord* records_arg = nullptr;
-  const unsigned long long *win_arg = nullptr, *cand_arg = nullptr;
-  if (workspace != nullptr && use_split(T) && M > 0) {
-    const SplitLayout l = split_layout(rows, T, cap_above);
+  // extras as LDS allows: the pool (where a pooled select can apply at all), then
+  // counting placement (2 * cap_above more slots)
+  int use_pool = 0, counting_ok = 0;
+  if ((T <= kPoolCap || sampling_ok(m_max)) && lds + (size_t)kPoolCap * sizeof(u64) + lds_static <= lds_max) {
+    use_pool = 1;
+    lds += (size_t)kPoolCap * sizeof(u64);
+  }
+  if (lds + (size_t)2 * cap_above * sizeof(u64) + lds_static <= lds_max) {
+    counting_ok = 1;
+    lds += (size_t)2 * cap_above * sizeof(u64);
+  }
+  int S = 0;
+  const int k_cap = (workspace && use_pool) ? slice_cap(T, m_max, &S) : 0;
+
+  const u64* loc = nullptr;
+  const int32_t* loc_count = nullptr;
+  if (k_cap) {
+    const SplitLayout l = split_layout(rows, S, k_cap);
     SOCKET_REQUIRE(workspace_bytes >= l.total, SOCKET_ERR_WORKSPACE);
     SOCKET_REQUIRE(socket_aligned16(workspace), SOCKET_ERR_ALIGN);
     char* ws = (char*)workspace;
-    RowRecord* records = (RowRecord*)(ws + l.off_records);
-    uint32_t* parts = (uint32_t*)(ws + l.off_parts);
-    uint32_t* hist_parts = (uint32_t*)(ws + l.off_hist);
-    unsigned long long* win = (unsigned long long*)(ws + l.off_win);
-    unsigned long long* cand = (unsigned long long*)(ws + l.off_cand);
-    const dim3 sgrid(l.S, rows);
-    if (row_range == nullptr) {
-      if (vec) hipLaunchKernelGGL(select_range_kernel<true>, sgrid, dim3(kSliceThreads), 0, s, scores, score_stride, lens, Hq, T, parts, l.S);
-      else hipLaunchKernelGGL(select_range_kernel<false>, sgrid, dim3(kSliceThreads), 0, s, scores, score_stride, lens, Hq, T, parts, l.S);
-      row_range = parts;
-      range_parts = l.S;
-    }
-    if (vec) hipLaunchKernelGGL(select_hist_kernel<true>, sgrid, dim3(kSliceThreads), 0, s, scores, score_stride, lens, row_range, range_parts, Hq, T, hist_parts, l.S);
-    else hipLaunchKernelGGL(select_hist_kernel<false>, sgrid, dim3(kSliceThreads), 0, s, scores, score_stride, lens, row_range, range_parts, Hq, T, hist_parts, l.S);
-    hipLaunchKernelGGL(select_threshold_kernel, dim3(rows), dim3(kThreads), 0, s, lens, budgets, row_range,
-                       range_parts, Hq, T, M, sink, window, write_base, list_width, hist_parts, l.S, records);
-    {
-      auto ck = vec ? select_collect_kernel<true> : select_collect_kernel<false>;
-      if (lds_base > 32 * 1024 &&
-          hipFuncSetAttribute(reinterpret_cast<const void*>(ck),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_base) != hipSuccess)
-        return SOCKET_ERR_LAUNCH;
-      hipLaunchKernelGGL(ck, sgrid, dim3(kSliceThreads), lds_base, s, scores, score_stride, lens, Hq, T,
-                         records, win, cap_above, cand);
-    }
+    u64* loc_w = (u64*)(ws + l.off_loc);
+    int32_t* count_w = (int32_t*)(ws + l.off_count);
+    const dim3 sgrid(S, rows);
+    if (vec)
+      hipLaunchKernelGGL(select_local_kernel<true>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride,
+                         lens, budgets, Hq, T, M, sink, window, write_base, list_width, S, k_cap, loc_w,
+                         count_w);
+    else
+      hipLaunchKernelGGL(select_local_kernel<false>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride,
+                         lens, budgets, Hq, T, M, sink, window, write_base, list_width, S, k_cap, loc_w,
+                         count_w);
     SOCKET_LAUNCH_CHECK();
-    records_arg = records;
-    win_arg = win;
-    cand_arg = cand;
+    loc = loc_w;
+    loc_count = count_w;
   }
 
   auto kern = vec ? select_list_kernel<true> : select_list_kernel<false>;
-  const size_t lds = (records_arg && counting_ok) ? lds_counting : lds_base;
   if (lds > 32 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return SOCKET_ERR_LAUNCH;
   hipLaunchKernelGGL(kern, dim3(rows), dim3(kThreads), lds, s, scores, score_stride, lens, budgets,
                      row_range, range_parts, Hq, T, M, sink, window, write_base, sparse_list,
-                     list_stride, list_width, sparse_len, cap_above, records_arg, win_arg, cand_arg,
-                     counting_ok);
+                     list_stride, list_width, sparse_len, cap_above, counting_ok, use_pool, loc,
+                     loc_count, S, k_cap);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }

@@ -251,6 +251,28 @@ def test_select_ties_and_special_values(dev, T):
         _check_select(s, 4, 16, M, dev)
 
 
+@pytest.mark.parametrize("T,M", [(131072, 2048), (40000, 700), (300000, 1024)])
+def test_select_rows_that_mislead_the_sampled_threshold(dev, T, M):
+    """Long rows are selected from a pool of everything above a threshold that
+    is estimated from runs of 64 scores at evenly spaced places.  These rows make
+    that estimate wrong in every direction (pool too small, too large, one slice
+    holding all winners); the result must still be the exact top-M."""
+    g = torch.Generator().manual_seed(T)
+    base = torch.rand(6, T, generator=g)
+    s = base.clone()
+    nchunk = (4096 if T <= 262144 else 16384) // 64
+    starts = (torch.arange(nchunk) * T // nchunk) // 4 * 4
+    sampled = (starts[:, None] + torch.arange(64)[None, :]).flatten()
+    s[0, sampled] += 100.0                                   # only the sampled places are hot: pool < M
+    s[1] = base[1] * 0.001
+    s[1, sampled] = -5.0                                     # sampled places are cold: threshold too low
+    s[2] = base[2] + torch.arange(T) * (50.0 / T)            # trend: winners all in the last slice
+    s[3, 12345] = 1e30                                       # one outlier stretches the key range
+    s[4, T // 3: T // 3 + 3 * M] += 10.0                     # a contiguous hot block larger than M
+    s[5] = (base[5] * 4).floor()                             # four values: the threshold sits in a huge tie
+    _check_select(s.view(1, 6, T), 4, 32, M, dev)
+
+
 @pytest.mark.parametrize("T", [9000, 66000])
 def test_select_ragged_lengths_and_budgets(dev, T):
     g = torch.Generator().manual_seed(11)
