@@ -1,0 +1,450 @@
+"""Llama-style decoder with the SOCKET attention hook on the HIP decode path.
+
+Host-side mirror of GPT-FAST/model.py (ModelArgs :103-136, KVCache :157-229,
+Transformer :232-329, TransformerBlock :332-349, Attention :352-589,
+FeedForward :592-600, RMSNorm :603-614, rotary helpers :617-639): same class,
+method and argument names, same math for projections, rotary embedding, norms
+and the soft / hard hashes.  What differs is how the attention hook keeps and
+walks its state:
+
+  * the cache stores packed, table-major bucket codes per KV head
+    (`KVCache.codes`, int32 [B,Hkv,NW,Tcap]) instead of int16 `k_hard`
+    [B,Hkv,T,L]; new keys are hashed and their value norms taken by one kernel
+    as they are appended (model.py:449-451 + :222-226 in one launch);
+  * lengths live on the device (`KVCache.lens`), so a decode step reads nothing
+    back to the host (the reference syncs at model.py:211-212,228,483) and the
+    whole step can be recorded into a HIP graph;
+  * no per-step code relayout (model.py:490-509), no K/V prefix copies
+    (:541-542), no T x T boolean mask (:279-281): prefill attends causally
+    through torch's flash SDPA, decode through the HIP kernels.
+
+Everything outside the attention hook (embedding, linears, norms, rotary) is
+plain torch: it is plumbing around the path, not part of it.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+import torch.nn as nn
+from torch import Tensor
+from torch.nn import functional as F
+
+from . import hash_cache
+from .socket_kernels import dense_decode_fwd
+
+
+def find_multiple(n: int, k: int) -> int:
+    return n if n % k == 0 else n + k - (n % k)
+
+
+@dataclass
+class ModelArgs:
+    """Same fields and defaults as GPT-FAST/model.py:103-118; `sink_size` and
+    `window_size` are the attributes the reference reads with
+    getattr(config, ..., 120) at model.py:511-512."""
+    block_size: int = 300000
+    vocab_size: int = 32000
+    n_layer: int = 1
+    n_head: int = 32
+    dim: int = 4096
+    intermediate_size: int = None
+    n_local_heads: int = -1
+    head_dim: int = 64
+    rope_base: float = 40000
+    norm_eps: float = 1e-5
+    L: int = 60
+    R: int = 1024
+    K: int = 10
+    heavy_const: int = 3600
+    sink_size: int = 120
+    window_size: int = 120
+
+    def __post_init__(self):
+        if self.n_local_heads == -1:
+            self.n_local_heads = self.n_head
+        if self.intermediate_size is None:
+            self.intermediate_size = find_multiple(int(2 * (4 * self.dim) / 3), 256)
+        self.head_dim = self.dim // self.n_head
+
+    @classmethod
+    def from_name(cls, name: str):
+        if name in transformer_configs:
+            return cls(**transformer_configs[name])
+        hits = [c for c in transformer_configs if c in str(name).upper() or c in str(name)]
+        assert len(hits) == 1, name
+        return cls(**transformer_configs[hits[0]])
+
+
+transformer_configs = {
+    # the reference's table (GPT-FAST/model.py:138-154)
+    "CodeLlama-7b-Python-hf": dict(block_size=16384, vocab_size=32000, n_layer=1, dim=4096, rope_base=1000000),
+    "Llama-2-7b-chat-hf": dict(block_size=300000, vocab_size=32000, n_layer=1, n_head=32, dim=4096, rope_base=10000),
+    "7B": dict(n_layer=1, n_head=32, dim=4096),
+    "13B": dict(n_layer=1, n_head=40, dim=5120),
+    "30B": dict(n_layer=1, n_head=52, dim=6656),
+    "34B": dict(n_layer=1, n_head=64, dim=8192, vocab_size=32000, n_local_heads=8, intermediate_size=22016,
+                rope_base=1000000),
+    "70B": dict(n_layer=1, n_head=64, dim=8192, n_local_heads=8, intermediate_size=28672),
+    # the long-context decode benchmark's model: Llama-3.1-8B geometry, random weights
+    "Llama-3.1-8B": dict(block_size=131072, vocab_size=128256, n_layer=32, n_head=32, n_local_heads=8, dim=4096,
+                         intermediate_size=14336, rope_base=500000, heavy_const=2048, sink_size=4,
+                         window_size=256),
+}
+
+
+class KVCache(nn.Module):
+    """K/V [B,Hkv,Tcap,D] plus the hash state of every cached key.
+
+    Constructor as GPT-FAST/model.py:162-171 with two keyword additions (`K`,
+    the bits per table, which fixes the packing; `device`).  `update` keeps the
+    reference's signature and bounds error (model.py:187-229); positions must be
+    one ascending run (they always are: arange(T) for prefill, [pos] for a decode
+    step)."""
+
+    def __init__(self, max_batch_size: int, max_seq_length: int, n_heads: int, head_dim: int, L: int, R: int,
+                 dtype=torch.bfloat16, K: int = 10, device=None):
+        super().__init__()
+        B, H, D = max_batch_size, n_heads, head_dim
+        T = find_multiple(max_seq_length, 8)
+        self.L, self.R, self.K = L, R, K
+        self.NW = hash_cache.words_per_key(L, K)
+        self.register_buffer("k_cache", torch.zeros((B, H, T, D), dtype=dtype, device=device))
+        self.register_buffer("v_cache", torch.zeros((B, H, T, D), dtype=dtype, device=device))
+        self.register_buffer("codes", torch.zeros((B, H, self.NW, T), dtype=torch.int32, device=device))
+        self.register_buffer("v_norm", torch.zeros((B, H, T), dtype=torch.float16, device=device))
+        self.register_buffer("attn_out", torch.zeros((B, H, D), dtype=dtype, device=device))
+        self.register_buffer("lens", torch.zeros((B,), dtype=torch.int32, device=device))
+        self.planes_words: Optional[Tensor] = None   # set by Attention once the planes are known
+
+    @property
+    def prefill_len(self) -> Tensor:
+        """0-d int32 count of cached positions (the reference's buffer of that name)."""
+        return self.lens.max()
+
+    def k_hard(self, T: int) -> Tensor:
+        """int16 codes [B,Hkv,T,L] as the reference's `k_hard` buffer holds them."""
+        return hash_cache.unpack_codes(self.codes, self.L, self.K, 0, T, layout="bhlt").permute(0, 1, 3, 2)
+
+    def _bounds(self, pos0: int, S: int) -> None:
+        Tcap = self.k_cache.size(2)
+        if pos0 < 0 or pos0 + S > Tcap:
+            raise RuntimeError(
+                f"KVCache.update out-of-bounds: input_pos in [{pos0},{pos0 + S - 1}] but cache T={Tcap}. "
+                f"Did you call setup_caches(max_seq_length >= max(input_pos)+1)?")
+
+    @torch.no_grad()
+    def update(self, input_pos: Tensor, k_val: Tensor, v_val: Tensor, v_norm: Optional[Tensor] = None,
+               k_hard: Optional[Tensor] = None, *, pos0: Optional[int] = None, hash_keys: bool = False):
+        """Write k_val / v_val [B,S,H,D] at positions input_pos [S].
+
+        With v_norm [B,S,H] and k_hard [B,S,H,L] given (the reference's calling
+        convention) they are stored as passed; with `hash_keys=True` the codes and
+        norms are computed from the rows by the fused kernel instead.  `pos0` is
+        the host's copy of input_pos[0]; a decode step (S == 1) never needs it,
+        a prefill without it reads it back from the device once."""
+        assert input_pos.ndim == 1, f"input_pos must be [S], got {tuple(input_pos.shape)}"
+        S = int(input_pos.numel())
+        assert k_val.ndim == 4 and v_val.ndim == 4
+        assert k_val.shape[1] == S and v_val.shape[1] == S, "k/v S dim must match input_pos length"
+        if S == 0:
+            return self.k_cache, self.v_cache
+        if S == 1 and pos0 is None:
+            # decode step: positions stay on the device
+            pos = input_pos.long()
+            self.k_cache.index_copy_(2, pos, k_val.permute(0, 2, 1, 3))
+            self.v_cache.index_copy_(2, pos, v_val.permute(0, 2, 1, 3))
+            pos_b = input_pos.to(torch.int32).expand(self.lens.numel()).contiguous()
+            if hash_keys:
+                _hash_rows(self, k_val, v_val, pos_b=pos_b)
+            elif k_hard is not None:
+                raise RuntimeError("KVCache.update: precomputed k_hard needs the host position (pass pos0)")
+            torch.maximum(self.lens, pos_b + 1, out=self.lens)
+            return self.k_cache, self.v_cache
+        if pos0 is None:
+            pos0 = int(input_pos[0])
+        self._bounds(pos0, S)
+        self.k_cache[:, :, pos0:pos0 + S].copy_(k_val.permute(0, 2, 1, 3))
+        self.v_cache[:, :, pos0:pos0 + S].copy_(v_val.permute(0, 2, 1, 3))
+        if hash_keys:
+            _hash_rows(self, k_val, v_val, t0=pos0)
+        else:
+            if v_norm is not None:
+                self.v_norm[:, :, pos0:pos0 + S].copy_(v_norm.permute(0, 2, 1))
+            if k_hard is not None:
+                hash_cache.pack_codes_into(k_hard.permute(0, 2, 3, 1), self.codes, self.K, t0=pos0)
+        self.lens.clamp_(min=pos0 + S)
+        return self.k_cache, self.v_cache
+
+
+# The three places where the attention hook enters the HIP library.  They are
+# module-level so that a test can stand a checker in for one of them; the
+# product has no other route.
+def _hash_rows(cache: KVCache, k_bshd: Tensor, v_bshd: Tensor, t0: int = 0, pos_b: Optional[Tensor] = None) -> None:
+    assert cache.planes_words is not None, "hash planes were not set on this cache"
+    hash_cache.hash_keys_into(k_bshd, v_bshd, cache.planes_words, cache.codes, cache.v_norm, cache.L, cache.K,
+                              t0=t0, pos_b=pos_b, layout="bshd")
+
+
+def _sparse_step(q_bhd: Tensor, q_probs: Tensor, cache: KVCache, T: int, sink: int, window: int, M: int) -> Tensor:
+    return hash_cache.sparse_decode_step(q_bhd, q_probs, cache.k_cache, cache.v_cache, cache.codes, cache.v_norm,
+                                         T, cache.K, sink, window, M, lens=cache.lens)
+
+
+def _dense_step(q_bhd: Tensor, cache: KVCache) -> Tensor:
+    return dense_decode_fwd(q_bhd, cache.k_cache, cache.v_cache, cache.lens)
+
+
+def _planes_to_words(planes: Tensor) -> Tensor:
+    return hash_cache.permute_planes(planes)
+
+
+class Transformer(nn.Module):
+    def __init__(self, config: ModelArgs) -> None:
+        super().__init__()
+        self.config = config
+        self.tok_embeddings = nn.Embedding(config.vocab_size, config.dim)
+        self.layers = nn.ModuleList(TransformerBlock(config) for _ in range(config.n_layer))
+        self.norm = RMSNorm(config.dim, eps=config.norm_eps)
+        self.output = nn.Linear(config.dim, config.vocab_size, bias=False)
+        self.register_buffer("freqs_cis", None, persistent=False)
+        self.max_batch_size = -1
+        self.max_seq_length = -1
+
+    def setup_caches(self, max_batch_size, max_seq_length):
+        if self.max_seq_length >= max_seq_length and self.max_batch_size >= max_batch_size:
+            return
+        device = self.tok_embeddings.weight.device
+        dtype = self.tok_embeddings.weight.dtype
+        cfg = self.config
+        max_seq_length = find_multiple(max_seq_length, 8)
+        self.max_seq_length = max_seq_length
+        self.max_batch_size = max_batch_size
+        for b in self.layers:
+            b.attention.kv_cache = KVCache(max_batch_size, max_seq_length, cfg.n_local_heads, cfg.head_dim,
+                                           L=cfg.L, R=cfg.R, dtype=dtype, K=cfg.K, device=device)
+            b.attention.sync_planes()
+        self.freqs_cis = precompute_freqs_cis(cfg.block_size, cfg.head_dim, cfg.rope_base).to(device=device)
+
+    def _positions(self, idx: Tensor, input_pos: Tensor, pos0: Optional[int]):
+        """Device positions (long) and, for a prefill, the host's first position."""
+        assert self.freqs_cis is not None, "Caches must be initialized first"
+        if input_pos.dtype != torch.long:
+            input_pos = input_pos.long()
+        S = idx.shape[1]
+        if S == 1 and pos0 is None:
+            return input_pos, None               # decode step: no read-back, kernels clamp by the cache's lengths
+        if pos0 is None:
+            pos0 = int(input_pos[0])
+        if pos0 < 0 or pos0 + S > self.max_seq_length:
+            raise RuntimeError(
+                f"input_pos out of bounds: [{pos0},{pos0 + S - 1}] vs max_seq_length={self.max_seq_length}. "
+                f"Call setup_caches(max_seq_length >= max(input_pos)+1).")
+        return input_pos, pos0
+
+    def _run(self, idx: Tensor, input_pos: Tensor, sparse: bool, pos0: Optional[int], last_only: bool) -> Tensor:
+        input_pos, pos0 = self._positions(idx, input_pos, pos0)
+        if idx.dtype != torch.long:
+            idx = idx.long()
+        freqs_cis = self.freqs_cis[input_pos]
+        x = self.tok_embeddings(idx)
+        for layer in self.layers:
+            x = layer._run(x, input_pos, freqs_cis, sparse, pos0)
+        if last_only:
+            x = x[:, -1:]
+        return self.output(self.norm(x))
+
+    def forward(self, idx: Tensor, input_pos: Optional[Tensor] = None, *, pos0: Optional[int] = None,
+                last_only: bool = False) -> Tensor:
+        """Dense attention everywhere (GPT-FAST/model.py:296-316).  `last_only`
+        returns logits of the last position only (a long prefill needs no more)."""
+        return self._run(idx, input_pos, False, pos0, last_only)
+
+    def sparse_forward(self, idx: Tensor, input_pos: Optional[Tensor] = None, *, pos0: Optional[int] = None,
+                       last_only: bool = False) -> Tensor:
+        """Hash-maintaining prefill, sparse decode (GPT-FAST/model.py:314-329)."""
+        return self._run(idx, input_pos, True, pos0, last_only)
+
+    @classmethod
+    def from_name(cls, name: str):
+        return cls(ModelArgs.from_name(name))
+
+
+class TransformerBlock(nn.Module):
+    def __init__(self, config: ModelArgs) -> None:
+        super().__init__()
+        self.attention = Attention(config)
+        self.feed_forward = FeedForward(config)
+        self.ffn_norm = RMSNorm(config.dim, config.norm_eps)
+        self.attention_norm = RMSNorm(config.dim, config.norm_eps)
+
+    def _run(self, x, input_pos, freqs_cis, sparse: bool, pos0):
+        h = x + self.attention._run(self.attention_norm(x), freqs_cis, input_pos, sparse, pos0)
+        return h + self.feed_forward(self.ffn_norm(h))
+
+    def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Tensor = None) -> Tensor:
+        return self._run(x, input_pos, freqs_cis, False, None)
+
+    def sparse_forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Tensor = None) -> Tensor:
+        return self._run(x, input_pos, freqs_cis, True, None)
+
+
+class Attention(nn.Module):
+    def __init__(self, config: ModelArgs):
+        super().__init__()
+        assert config.dim % config.n_head == 0
+        total_head_dim = (config.n_head + 2 * config.n_local_heads) * config.head_dim
+        self.wqkv = nn.Linear(config.dim, total_head_dim, bias=False)
+        self.wo = nn.Linear(config.dim, config.dim, bias=False)
+        self.kv_cache: Optional[KVCache] = None
+        self.n_head = config.n_head
+        self.head_dim = config.head_dim
+        self.n_local_heads = config.n_local_heads
+        self.dim = config.dim
+        self._register_load_state_dict_pre_hook(self.load_hook)
+        self.config = config
+        self.L, self.R, self.K = config.L, config.R, config.K
+        self.heavy_const = config.heavy_const
+        self.register_buffer("planes", torch.randn(self.L, self.K, self.head_dim) * 0.02)
+        self.register_buffer("protos_T", torch.randn(self.K, self.R) * 0.02)
+
+    def load_hook(self, state_dict, prefix, *args):
+        if prefix + "wq.weight" in state_dict:
+            wq = state_dict.pop(prefix + "wq.weight")
+            wk = state_dict.pop(prefix + "wk.weight")
+            wv = state_dict.pop(prefix + "wv.weight")
+            state_dict[prefix + "wqkv.weight"] = torch.cat([wq, wk, wv])
+
+    def sync_planes(self) -> None:
+        """Hand the current hyperplanes to the cache in the hashing kernel's
+        column order; call again after changing `planes`."""
+        if self.kv_cache is not None:
+            self.kv_cache.planes_words = _planes_to_words(self.planes)
+
+    # ---- hashes (GPT-FAST/model.py:392-413) ------------------------------------------
+    def soft_hash(self, queries_bhd: Tensor) -> Tensor:
+        """softmax_r( tanh(q . planes) / sqrt(D) @ protos_T ): [B,H,D] -> [B,H,L,R]."""
+        proj = torch.einsum("bhd,lkd->bhlk", queries_bhd, self.planes)
+        temp = max(math.sqrt(queries_bhd.size(-1)), 1e-6)
+        logits = torch.einsum("bhlk,kr->bhlr", torch.tanh(proj) / temp, self.protos_T)
+        return torch.softmax(logits, dim=-1)
+
+    def pack_bits(self, bits: Tensor) -> Tensor:
+        """Big-endian pack of the last dim: code = sum_k bit_k << (K-1-k), int16."""
+        K = bits.shape[-1]
+        weights = 1 << torch.arange(K - 1, -1, -1, device=bits.device, dtype=torch.int16)
+        return (bits.to(torch.int16) * weights).sum(dim=-1).to(torch.int16)
+
+    @torch.no_grad()
+    def hard_hash_keys(self, keys_bshd: Tensor) -> Tensor:
+        """int16 codes [B,S,Hkv,L] of keys [B,S,Hkv,D]: sign bits of the K
+        projections of each table, zero counting as set.  On the device the
+        packed words come from the hashing kernel and are unpacked into the
+        reference's layout; the cache itself never takes this detour."""
+        if keys_bshd.is_cuda:
+            B, S, H, _ = keys_bshd.shape
+            NW = hash_cache.words_per_key(self.L, self.K)
+            words = torch.empty((B, H, NW, find_multiple(S, 4)), dtype=torch.int32, device=keys_bshd.device)
+            hash_cache.hash_keys_into(keys_bshd, None, _planes_to_words(self.planes), words, None, self.L, self.K,
+                                      t0=0, layout="bshd")
+            return hash_cache.unpack_codes(words, self.L, self.K, 0, S, layout="bthl")
+        proj = torch.einsum("bshd,lkd->bshlk", keys_bshd, self.planes)
+        return self.pack_bits(proj >= 0)
+
+    # ---- the hook -------------------------------------------------------------------------
+    def _run(self, x: Tensor, freqs_cis: Tensor, input_pos: Tensor, sparse: bool, pos0: Optional[int]) -> Tensor:
+        bsz, seqlen, _ = x.shape
+        kv_size = self.n_local_heads * self.head_dim
+        q, k, v = self.wqkv(x).split([self.dim, kv_size, kv_size], dim=-1)
+        q = q.view(bsz, seqlen, self.n_head, self.head_dim)
+        k = k.view(bsz, seqlen, self.n_local_heads, self.head_dim)
+        v = v.view(bsz, seqlen, self.n_local_heads, self.head_dim)
+        q = apply_rotary_emb(q, freqs_cis)
+        k = apply_rotary_emb(k, freqs_cis)
+
+        cache = self.kv_cache
+        if sparse:
+            assert cache is not None, "Call setup_caches() first so kv_cache exists"
+        if cache is not None:
+            cache.update(input_pos, k, v, pos0=pos0, hash_keys=sparse)
+
+        if seqlen != 1 or cache is None:
+            y = self._prefill_attention(q, k, v, input_pos, pos0)             # [B,S,H,D]
+            return self.wo(y.reshape(bsz, seqlen, self.dim))
+
+        q_bhd = q[:, 0]                                                       # [B,H,D]
+        if sparse:
+            T = cache.k_cache.size(2)       # upper bound; the kernels stop at cache.lens
+            cfg = self.config
+            out_bhd = _sparse_step(q_bhd, self.soft_hash(q_bhd), cache, T, int(cfg.sink_size),
+                                   int(cfg.window_size), int(self.heavy_const))
+        else:
+            out_bhd = _dense_step(q_bhd, cache)
+        return self.wo(out_bhd.reshape(bsz, 1, self.dim))
+
+    def _prefill_attention(self, q, k, v, input_pos, pos0) -> Tensor:
+        """Causal attention of a block of new tokens over the cache prefix and
+        itself (dense in both modes, as GPT-FAST/model.py:466-481)."""
+        gqa = self.n_head != self.n_local_heads
+        qh = q.transpose(1, 2)
+        if self.kv_cache is None or pos0 == 0:
+            y = F.scaled_dot_product_attention(qh, k.transpose(1, 2), v.transpose(1, 2), is_causal=True,
+                                               enable_gqa=gqa)
+        else:
+            end = pos0 + q.shape[1]
+            kc, vc = self.kv_cache.k_cache[:, :, :end], self.kv_cache.v_cache[:, :, :end]
+            mask = torch.arange(end, device=q.device)[None, :] <= input_pos[:, None]      # [S,end]
+            y = F.scaled_dot_product_attention(qh, kc, vc, attn_mask=mask, enable_gqa=gqa)
+        return y.transpose(1, 2)
+
+    def forward(self, x: Tensor, freqs_cis: Tensor, mask: Tensor, input_pos: Optional[Tensor] = None) -> Tensor:
+        """Dense attention (GPT-FAST/model.py:562-589); `mask` is accepted and unused."""
+        return self._run(x, freqs_cis, input_pos.long(), False, None)
+
+    def sparse_forward(self, x: Tensor, freqs_cis: Tensor, mask1: Tensor, mask2: Tensor,
+                       input_pos: Optional[Tensor] = None) -> Tensor:
+        """The SOCKET hook (GPT-FAST/model.py:415-560); the masks are accepted and unused."""
+        assert input_pos is not None, "sparse_forward expects input_pos"
+        return self._run(x, freqs_cis, input_pos.long(), True, None)
+
+
+class FeedForward(nn.Module):
+    def __init__(self, config: ModelArgs) -> None:
+        super().__init__()
+        self.w1 = nn.Linear(config.dim, config.intermediate_size, bias=False)
+        self.w3 = nn.Linear(config.dim, config.intermediate_size, bias=False)
+        self.w2 = nn.Linear(config.intermediate_size, config.dim, bias=False)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return self.w2(F.silu(self.w1(x)) * self.w3(x))
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: Tensor) -> Tensor:
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)).type_as(x) * self.weight
+
+
+def precompute_freqs_cis(seq_len: int, n_elem: int, base: float = 10000) -> Tensor:
+    """[seq_len, n_elem/2, 2] (cos, sin) table, stored in bfloat16 as
+    GPT-FAST/model.py:617-623 stores it."""
+    inv = 1.0 / (base ** (torch.arange(0, n_elem, 2)[: n_elem // 2].float() / n_elem))
+    ang = torch.outer(torch.arange(seq_len).float(), inv)
+    return torch.stack([ang.cos(), ang.sin()], dim=-1).to(torch.bfloat16)
+
+
+def apply_rotary_emb(x: Tensor, freqs_cis: Tensor) -> Tensor:
+    """Rotate the (2i, 2i+1) pairs of x [B,S,H,D] by the angles of freqs_cis
+    [S,D/2,2], in fp32 (GPT-FAST/model.py:626-639)."""
+    xs = x.float().reshape(*x.shape[:-1], -1, 2)
+    fc = freqs_cis.view(1, xs.size(1), 1, xs.size(3), 2)
+    re = xs[..., 0] * fc[..., 0] - xs[..., 1] * fc[..., 1]
+    im = xs[..., 1] * fc[..., 0] + xs[..., 0] * fc[..., 1]
+    return torch.stack([re, im], dim=-1).flatten(3).type_as(x)

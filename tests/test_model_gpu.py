@@ -1,0 +1,151 @@
+"""The model hook and the generation harness on the MI355X: every attention
+step goes through libsocket_hip; the oracle stand-ins of tests/oracle_backend.py
+are swapped in only to produce the expected values."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import socket_oracle as orc
+from socket_amd import generate as gen
+from socket_amd import model as M
+from tests import oracle_backend
+
+pytestmark = pytest.mark.gpu
+
+
+def toy_args(**kw):
+    base = dict(block_size=1024, vocab_size=331, n_layer=2, n_head=4, n_local_heads=2, dim=512, L=20, K=10, R=1024,
+                heavy_const=48, sink_size=4, window_size=16, rope_base=10000)
+    base.update(kw)
+    return M.ModelArgs(**base)
+
+
+def toy_model(dev, dtype=torch.float32, seed=0, **kw):
+    torch.manual_seed(seed)
+    model = M.Transformer(toy_args(**kw)).eval()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if not name.endswith("norm.weight"):
+                p.normal_(0, 0.06)
+        for blk in model.layers:
+            blk.attention.planes.normal_(0, 1.0)
+            blk.attention.protos_T.copy_(orc.hypercube_protos_T(model.config.K) * 3.0)
+    return model.to(device=dev, dtype=dtype)
+
+
+def _reset(model):
+    for layer in model.layers:
+        layer.attention.kv_cache.lens.zero_()
+
+
+@torch.no_grad()
+def _run_steps(model, ids, n_prompt, sparse=True):
+    fwd = model.sparse_forward if sparse else model.forward
+    dev = ids.device
+    logits = [fwd(ids[:, :n_prompt], torch.arange(n_prompt, device=dev), pos0=0, last_only=True)[:, -1]]
+    for t in range(n_prompt, ids.shape[1]):
+        logits.append(fwd(ids[:, t:t + 1], torch.tensor([t], device=dev))[:, -1])
+    return torch.stack(logits, 1).float().cpu()
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-3), (torch.bfloat16, 6e-2)])
+def test_sparse_hook_matches_oracle_attention(dev, monkeypatch, dtype, tol):
+    """Same model, same cache contents; the decode attention once through the
+    HIP kernels and once through the oracle (scorer -> stable top-k -> list ->
+    textbook softmax).  The selected lists coincide (scores are bit-exact), so
+    the logits agree to the attention tolerance."""
+    model = toy_model(dev, dtype)
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, 331, (2, 150), generator=g).to(dev)
+    model.setup_caches(2, 160)
+    have = _run_steps(model, ids, 140)
+    _reset(model)
+    oracle_backend.install(monkeypatch, M, hashing=False, sparse=True, dense=False)
+    want = _run_steps(model, ids, 140)
+    assert torch.isfinite(have).all()
+    scale = float(want.abs().max())
+    assert float((have - want).abs().max()) <= tol * max(scale, 1.0)
+    if dtype == torch.float32:
+        assert torch.equal(have.argmax(-1), want.argmax(-1))
+
+
+def test_cache_hash_state_after_prefill_and_decode(dev):
+    """Codes and value norms written by the fused append equal the oracle's hash
+    of the cached rows wherever the fp64 projection is clear of zero."""
+    model = toy_model(dev, torch.bfloat16, seed=3)
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, 331, (2, 70), generator=g).to(dev)
+    model.setup_caches(2, 80)
+    _run_steps(model, ids, 61)
+    for layer in model.layers:
+        attn, cache = layer.attention, layer.attention.kv_cache
+        assert cache.lens.tolist() == [70, 70]
+        keys = cache.k_cache[:, :, :70].permute(0, 2, 1, 3).float().cpu()           # [B,T,H,D]
+        planes = attn.planes.float().cpu()
+        proj = orc.projections_f64(keys, planes.to(torch.bfloat16).float())          # the kernel hashes with bf16 planes
+        want = orc.pack_bits(proj >= 0)                                              # [B,T,H,L]
+        have = cache.k_hard(70).cpu()                                                # [B,H,T,L]
+        assert have.dtype == torch.int16 and tuple(have.shape) == (2, 2, 70, 20)
+        clear = (proj.abs() > 1e-3 * proj.abs().mean()).all(-1)                      # every bit of the code is safe
+        assert clear.float().mean() > 0.9
+        assert torch.equal(have.permute(0, 2, 1, 3)[clear], want[clear])
+        vn = cache.v_cache[:, :, :70].float().norm(dim=-1).cpu()
+        torch.testing.assert_close(cache.v_norm[:, :, :70].float().cpu(), vn, rtol=2e-3, atol=1e-3)
+
+
+def test_hard_hash_keys_on_device_uses_reference_layout(dev):
+    attn = M.Attention(toy_args()).to(dev)
+    g = torch.Generator().manual_seed(4)
+    attn.planes.copy_(torch.randn(20, 10, 128, generator=g))
+    keys = torch.randn(2, 37, 2, 128, generator=g).to(torch.bfloat16)
+    have = attn.hard_hash_keys(keys.to(dev)).cpu()
+    assert have.dtype == torch.int16 and tuple(have.shape) == (2, 37, 2, 20)
+    proj = orc.projections_f64(keys.float(), attn.planes.cpu().to(torch.bfloat16).float())
+    clear = (proj.abs() > 1e-3 * proj.abs().mean()).all(-1)
+    assert torch.equal(have[clear], orc.pack_bits(proj >= 0)[clear])
+
+
+def test_kv_cache_takes_precomputed_codes_in_the_reference_convention(dev):
+    c = M.KVCache(2, 64, 2, 128, L=20, R=1024, dtype=torch.bfloat16, K=10, device=dev)
+    g = torch.Generator().manual_seed(5)
+    k = torch.randn(2, 9, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(2, 9, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    k_hard = torch.randint(0, 1024, (2, 9, 2, 20), generator=g).to(torch.int16).to(dev)
+    v_norm = torch.rand(2, 9, 2, generator=g).to(torch.float16).to(dev)
+    c.update(torch.arange(5, 14, device=dev), k, v, v_norm=v_norm, k_hard=k_hard)
+    assert c.lens.tolist() == [14, 14]
+    assert torch.equal(c.k_hard(14)[:, :, 5:14], k_hard.permute(0, 2, 1, 3))
+    assert torch.equal(c.v_norm[:, :, 5:14], v_norm.permute(0, 2, 1))
+    assert torch.equal(c.k_cache[:, :, 5:14], k.permute(0, 2, 1, 3))
+
+
+@pytest.mark.parametrize("decode_type", ["sparse", "dense"])
+def test_decode_graph_replays_equal_the_eager_step(dev, decode_type):
+    model = toy_model(dev, torch.bfloat16, seed=6)
+    g = torch.Generator().manual_seed(6)
+    prompt = torch.randint(0, 331, (2, 200), generator=g).to(dev)
+    seq_g, st = gen.generate(model, prompt, 12, decode_type=decode_type, use_graph=True, check_graph=True)
+    assert st["graph"] and st["graph_check"]["same_token"]
+    assert st["graph_check"]["max_abs_logit_diff"] <= 1e-2
+    seq_e, st_e = gen.generate(model, prompt, 12, decode_type=decode_type, use_graph=False)
+    assert not st_e["graph"]
+    assert torch.equal(seq_g, seq_e)
+
+
+def test_all_covering_window_reproduces_dense_tokens_on_device(dev):
+    model = toy_model(dev, torch.float32, seed=7, sink_size=0, window_size=4096, heavy_const=0)
+    g = torch.Generator().manual_seed(7)
+    prompt = torch.randint(0, 331, (2, 90), generator=g).to(dev)
+    seq_d, _ = gen.generate(model, prompt, 10, decode_type="dense")
+    seq_s, _ = gen.generate(model, prompt, 10, decode_type="sparse")
+    assert torch.equal(seq_s, seq_d)
+
+
+def test_load_random_model_and_warmup(dev):
+    model = gen.load_random_model(toy_args(n_layer=1), dev, torch.bfloat16, seed=1)
+    assert model.layers[0].attention.planes.dtype == torch.bfloat16 and model.norm.weight.eq(1).all()
+    assert 0.015 < float(model.output.weight.float().std()) < 0.025
+    model.setup_caches(1, 512)
+    gen.warmup_sparse_decode(model, dev, T=300)
