@@ -14,7 +14,7 @@ HBM peak; `kernels` does the same for every kernel; `dense` is the dense
 flash-decode comparator on the same GPU; `cpu_baseline` is the CPU oracle timed
 on the host's cores on a slice of the same workload.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c5]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5]
                   [--only score|select|attend|hash|dense] [--no-cpu] [--no-parity]
 """
 from __future__ import annotations
@@ -162,7 +162,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--only", default=None,
                     choices=["score", "score_f32", "select", "attend", "hash", "dense", "copy"])
     ap.add_argument("--no-cpu", action="store_true")

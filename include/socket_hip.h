@@ -148,6 +148,23 @@ int socket_soft_hash_score_f16(const uint16_t* q_probs, const int16_t* key_bucke
                                const uint16_t* v_norm, const uint8_t* allowed, float* out,
                                int B, int H, int L, int R, int T, void* stream);
 
+/* Query soft hash: bucket probabilities of every query head for every table,
+ *   probs[b,h,l,:] = softmax_r( inv_temperature * sum_k tanh(q[b,h,:] . planes[l,k,:]) * tanh_scale
+ *                                                 * protos_T[k,r] )
+ * with tanh_scale = 1 / max(sqrt(D), 1e-6) in both callers and inv_temperature = 1
+ * (GPT-FAST/model.py:392-401) or 1 / 0.3
+ * (pipeline/train_quest/modeling/modeling_llama.py:618-638).
+ * q [B,Hq,D] (element strides, unit-stride last dim), planes [L,K,D] and protos_T
+ * [K,R] contiguous, all of `dtype`; out [B,Hq,L,R] contiguous, out_dtype
+ * SOCKET_F32 or SOCKET_BF16, 16-byte aligned.  Computed in fp32 and rounded once.
+ * Requires D <= 256, K <= 16, Hq / Hkv <= 8, R % 4 == 0, B * Hkv <= 65535.
+ * Hkv only groups the heads that share a workgroup; any divisor of Hq with
+ * Hq / Hkv <= 8 gives the same result. */
+int socket_soft_hash(const void* q, int dtype, int64_t q_stride_b, int64_t q_stride_h,
+                     const void* planes, const void* protos_T, void* out, int out_dtype,
+                     int B, int Hq, int Hkv, int D, int L, int K, int R,
+                     float tanh_scale, float inv_temperature, void* stream);
+
 /* ------------------------------------------------------------------------
  * K3  top-k select and index list
  * ---------------------------------------------------------------------- */
@@ -204,6 +221,7 @@ int socket_attend_stage1(const void* q, const void* k, const void* v, int dtype,
 
 /* Stage 2: merge the ceil(len / block_seq) splits of every (b,h) into
  * out[b,h,:] (out_dtype); len == 0 gives NaN like the reference's 0/0.
+ * mid_o must be 16-byte aligned.
  * Replaces sparse_decode_stage2, kernels/socket_triton_kernels.py:208-235
  * (kernel :121-164). */
 int socket_attend_stage2(const float* mid_o, const float* mid_lse,

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p, POINTER
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p, POINTER
 
 import torch
 
@@ -46,6 +46,7 @@ SIGNATURES = {
     "socket_score_packed": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
     "socket_soft_hash_collision": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "socket_soft_hash_score_f16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "socket_soft_hash": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),
     "socket_select_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "socket_select_list": (_I, [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _P, _Z, _P]),
     "socket_attend_stage1": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L,

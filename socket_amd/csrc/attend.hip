@@ -187,33 +187,75 @@ __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
   finish_split<E, LPR, 1>(m, l, acc, 1, mo, ml, 0, 0, lds);
 }
 
+constexpr int kMergeThreads = 256;
+
+// Merge of the per-split partials.  One workgroup of 256 lanes per (b, h): the
+// largest log-sum-exp first, then the lanes, four output coordinates each and
+// 256 / (D/4) splits side by side, add up weight * partial with independent
+// loads, and LDS folds the side-by-side groups.
 template <int D>
-__global__ __launch_bounds__(D) void stage2_kernel(
+__global__ __launch_bounds__(kMergeThreads) void stage2_kernel(
     const float* __restrict__ mid_o, const float* __restrict__ mid_lse,
     const int32_t* __restrict__ sparse_len, int64_t len_sb, int64_t len_sh, void* __restrict__ out,
     int out_dtype, int64_t out_sb, int64_t out_sh, int Hq, int nsplit, int block_seq) {
-  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  constexpr int LPD = D / 4;                    // lanes across the head dimension
+  constexpr int NG = kMergeThreads / LPD;       // splits handled side by side
+  constexpr int kW = kMergeThreads / SOCKET_WAVE;
+  __shared__ float red[kW];
+  __shared__ float part[NG][D + 4];
+  __shared__ float psum[NG];
+  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
   const int len = sparse_len[b * len_sb + h * len_sh];
   int nblk = len <= 0 ? 0 : (len + block_seq - 1) / block_seq;
   nblk = min(nblk, nsplit);
   const float* mo = mid_o + ((int64_t)b * Hq + h) * nsplit * D;
   const float* ml = mid_lse + ((int64_t)b * Hq + h) * nsplit;
-  float m = -INFINITY, sum = 0.f, acc = 0.f;
-  for (int s = 0; s < nblk; ++s) {
+
+  float m = -INFINITY;
+  for (int s = tid; s < nblk; s += kMergeThreads) m = fmaxf(m, ml[s]);
+#pragma unroll
+  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, SOCKET_WAVE));
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = red[0];
+#pragma unroll
+  for (int w = 1; w < kW; ++w) m = fmaxf(m, red[w]);
+
+  const int grp = tid / LPD, d4 = (tid % LPD) * 4;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float sum = 0.f;
+  for (int s = grp; s < nblk; s += NG) {
     const float lse = ml[s];
-    if (lse == -INFINITY) continue;  // split without a live row
-    const float nm = fmaxf(m, lse);
-    const float old = (m == nm) ? 1.f : fast_exp(m - nm);
-    const float w = (lse == nm) ? 1.f : fast_exp(lse - nm);
-    acc = acc * old + w * mo[(int64_t)s * D + d];
-    sum = sum * old + w;
-    m = nm;
+    // a split without a live row has lse = -inf and weight 0; so has every split
+    // when nothing at all was attended (m = -inf), which leaves 0/0 below
+    const float w = (lse == -INFINITY) ? 0.f : fast_exp(lse - m);
+    const float4 o = *reinterpret_cast<const float4*>(mo + (int64_t)s * D + d4);
+    acc.x += w * o.x;
+    acc.y += w * o.y;
+    acc.z += w * o.z;
+    acc.w += w * o.w;
+    sum += w;
   }
-  const float r = acc / sum;  // 0/0 -> NaN when nothing was attended, as the reference
-  const int64_t o = b * out_sb + h * out_sh + d;
-  if (out_dtype == SOCKET_F32) store_elem<DType_f32>(out, o, r);
-  else if (out_dtype == SOCKET_BF16) store_elem<DType_bf16>(out, o, r);
-  else store_elem<DType_f16>(out, o, r);
+  part[grp][d4] = acc.x;
+  part[grp][d4 + 1] = acc.y;
+  part[grp][d4 + 2] = acc.z;
+  part[grp][d4 + 3] = acc.w;
+  if (d4 == 0) psum[grp] = sum;
+  __syncthreads();
+  if (tid < D) {
+    float a = 0.f, t = 0.f;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      a += part[g][tid];
+      t += psum[g];
+    }
+    const float r = a / t;  // 0/0 -> NaN when nothing was attended, as the reference
+    const int64_t o = b * out_sb + h * out_sh + tid;
+    if (out_dtype == SOCKET_F32) store_elem<DType_f32>(out, o, r);
+    else if (out_dtype == SOCKET_BF16) store_elem<DType_bf16>(out, o, r);
+    else store_elem<DType_f16>(out, o, r);
+  }
 }
 
 // Dense flash-decode: rows [s*rows_per_split, ...) of one kv head, all G heads
@@ -379,8 +421,9 @@ int launch_dense_stage1(const AttArgs& a, const int32_t* lens, float* mid_o, flo
 int launch_stage2(const float* mid_o, const float* mid_lse, const int32_t* len, int64_t len_sb,
                   int64_t len_sh, void* out, int out_dtype, int64_t out_sb, int64_t out_sh, int B,
                   int Hq, int D, int nsplit, int block_seq, hipStream_t s) {
+  SOCKET_REQUIRE(socket_aligned16(mid_o), SOCKET_ERR_ALIGN);
 #define SOCKET_S2(DD)                                                                              \
-  hipLaunchKernelGGL((stage2_kernel<DD>), dim3(Hq, B), dim3(DD), 0, s, mid_o, mid_lse, len, len_sb, \
+  hipLaunchKernelGGL((stage2_kernel<DD>), dim3(Hq, B), dim3(kMergeThreads), 0, s, mid_o, mid_lse, len, len_sb, \
                      len_sh, out, out_dtype, out_sb, out_sh, Hq, nsplit, block_seq)
   if (D == 128) SOCKET_S2(128);
   else if (D == 64) SOCKET_S2(64);

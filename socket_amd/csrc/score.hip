@@ -69,6 +69,18 @@ __device__ __forceinline__ RawEntry<BYTES> load_entry(const void* lds) {
 // exactly.
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// Streamed once: loads and stores that should not displace the table slices,
+// which every tile of a (b, kv head) pair re-reads, from the L2.
+__device__ __forceinline__ uint4 load_stream16(const uint32_t* p) {
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void store_stream16(float* p, float a, float b, float c, float d) {
+  float4_t v = {a, b, c, d};
+  __builtin_nontemporal_store(v, reinterpret_cast<float4_t*>(p));
+}
 
 struct Bf16Select {
   short4_t identity_row;  // e_{lane % 4} as four bf16
@@ -252,14 +264,13 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   for (int d = 0; d < kPrefetch; ++d)
 #pragma unroll
     for (int j = 0; j < KT4; ++j)
-      ring[d][j] = *reinterpret_cast<const uint4*>(codes_pair + (int64_t)min(d, NW - 1) * Tcap + tsafe[j]);
+      ring[d][j] = load_stream16(codes_pair + (int64_t)min(d, NW - 1) * Tcap + tsafe[j]);
   // group j has consumed its current word: shift the ring and fetch the word
   // kPrefetch steps ahead (past the end it refetches the last word, unused)
   auto advance = [&](int j, int w) {
 #pragma unroll
     for (int d = 0; d + 1 < kPrefetch; ++d) ring[d][j] = ring[d + 1][j];
-    ring[kPrefetch - 1][j] = *reinterpret_cast<const uint4*>(
-        codes_pair + (int64_t)min(w + kPrefetch, NW - 1) * Tcap + tsafe[j]);
+    ring[kPrefetch - 1][j] = load_stream16(codes_pair + (int64_t)min(w + kPrefetch, NW - 1) * Tcap + tsafe[j]);
   };
 
   // slice staging: slot s covers table elements [s*EPV, (s+1)*EPV) of every head
@@ -418,7 +429,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
       }
       float* dst = scores + ((int64_t)(b * Hq + kvh * G + g)) * score_stride + tbase[j];
       if (tbase[j] + 4 <= T) {
-        *reinterpret_cast<float4*>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+        store_stream16(dst, o[0], o[1], o[2], o[3]);
       } else {
         for (int i = 0; i < 4 && tbase[j] + i < T; ++i) dst[i] = o[i];
       }
@@ -521,14 +532,15 @@ int dispatch_p(const ScoreArgs& a) {
   return launch_score_packed<GP, TT, KT4, THREADS, 0>(a);
 }
 
-// Tile size: the largest of 8192 / 4096 / 1024 tokens per workgroup that still
-// gives every CU a workgroup.  (16 tokens per lane would halve the table
+// Tile size: the largest of 8192 / 4096 / 2048 / 1024 tokens per workgroup that
+// still gives every CU a workgroup.  (16 tokens per lane would halve the table
 // refills again but does not fit 128 registers next to the prefetched codes.)
 int tile_tokens(int B, int Hkv, int G, int T) {
   const SocketDeviceLimits& lim = socket_device_limits();
   const int64_t pairs = (int64_t)B * Hkv;
   if (G <= 4 && pairs * ((T + 8191) / 8192) >= lim.cu_count) return 8192;
   if (pairs * ((T + 4095) / 4096) >= lim.cu_count) return 4096;
+  if (pairs * ((T + 2047) / 2048) >= lim.cu_count) return 2048;
   return 1024;
 }
 
@@ -539,6 +551,7 @@ int dispatch_tile(const ScoreArgs& a) {
     if (tw == 8192) return dispatch_p<GP, TT, 2, 1024>(a);
   }
   if (tw == 4096) return dispatch_p<GP, TT, 2, 512>(a);
+  if (tw == 2048) return dispatch_p<GP, TT, 1, 512>(a);
   return dispatch_p<GP, TT, 1, 256>(a);
 }
 

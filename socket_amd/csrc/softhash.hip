@@ -1,0 +1,189 @@
+// K5: query soft hash -- the producer of the scorer's bucket-probability table.
+//
+//   proj[l,k]  = q . planes[l,k,:]
+//   t[k]       = tanh(proj[l,k]) * tanh_scale            (tanh_scale = 1 / sqrt(D))
+//   logit[l,r] = inv_temperature * sum_k t[k] * protos_T[k,r]
+//   probs[l,:] = softmax_r(logit[l,:])
+//
+// GPT-FAST/model.py:392-401 (inv_temperature 1) and the HuggingFace twin
+// pipeline/train_quest/modeling/modeling_llama.py:618-638 (logits / 0.3), which
+// run this as two einsums, a tanh, a division and a softmax, five launches with
+// [B,H,L,K] and [B,H,L,R] intermediates rounded to the model dtype.  Here it is
+// one launch computing in fp32 from the inputs as stored and rounding once, to
+// the output dtype.
+//
+// One workgroup per (table l, batch b, KV head): the K planes of the table and
+// the G query heads of the group sit in LDS, G*K lanes take the projections,
+// then every lane owns runs of four buckets and makes three sweeps over them
+// (maximum, sum of exponentials, normalised write), recomputing the K-term
+// logits each time rather than holding R/64 of them per head in registers.
+#include "socket_common.h"
+
+namespace {
+
+constexpr int kSHThreads = 256;
+constexpr int kSHWaves = kSHThreads / SOCKET_WAVE;
+constexpr int kSHMaxK = 16;
+constexpr int kSHMaxG = 8;
+constexpr int kSHMaxD = 256;
+
+template <class DT>
+__device__ __forceinline__ float sh_load(const void* p, int64_t i);
+template <>
+__device__ __forceinline__ float sh_load<DType_f32>(const void* p, int64_t i) {
+  return ((const float*)p)[i];
+}
+template <>
+__device__ __forceinline__ float sh_load<DType_bf16>(const void* p, int64_t i) {
+  return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+template <>
+__device__ __forceinline__ float sh_load<DType_f16>(const void* p, int64_t i) {
+  return f16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+
+template <class DT>
+__global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
+    const void* __restrict__ q, int64_t q_sb, int64_t q_sh, const void* __restrict__ planes,
+    const void* __restrict__ protos_T, void* __restrict__ out, int out_dtype, int Hq, int Hkv, int G,
+    int D, int L, int K, int R, float tanh_scale, float inv_temperature) {
+  __shared__ float qs[kSHMaxG][kSHMaxD];
+  __shared__ float ps[kSHMaxK][kSHMaxD + 1];
+  __shared__ float ts[kSHMaxG][kSHMaxK];
+  __shared__ float red[kSHWaves][kSHMaxG];
+  const int l = blockIdx.x, pair = blockIdx.y;
+  const int b = pair / Hkv, kvh = pair % Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  for (int i = tid; i < G * D; i += kSHThreads) {
+    const int g = i / D, d = i % D;
+    qs[g][d] = sh_load<DT>(q, b * q_sb + (int64_t)(kvh * G + g) * q_sh + d);
+  }
+  for (int i = tid; i < K * D; i += kSHThreads) ps[i / D][i % D] = sh_load<DT>(planes, (int64_t)l * K * D + i);
+  __syncthreads();
+  if (tid < G * K) {
+    const int g = tid / K, k = tid % K;
+    float s = 0.f;
+    for (int d = 0; d < D; ++d) s += qs[g][d] * ps[k][d];
+    ts[g][k] = tanhf(s) * tanh_scale * inv_temperature;
+  }
+  __syncthreads();
+
+  // logits of buckets r0..r0+3 for every head of the group
+  auto logits4 = [&](int r0, float (&lg)[kSHMaxG][4]) {
+#pragma unroll
+    for (int g = 0; g < kSHMaxG; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) lg[g][i] = 0.f;
+    for (int k = 0; k < K; ++k) {
+      float pr[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pr[i] = sh_load<DT>(protos_T, (int64_t)k * R + r0 + i);
+#pragma unroll
+      for (int g = 0; g < kSHMaxG; ++g) {
+        if (g < G) {
+          const float t = ts[g][k];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) lg[g][i] += t * pr[i];
+        }
+      }
+    }
+  };
+  // workgroup-wide reduction of one value per head; every lane gets the result
+  auto reduce = [&](float (&v)[kSHMaxG], bool is_max) {
+#pragma unroll
+    for (int g = 0; g < kSHMaxG; ++g) {
+#pragma unroll
+      for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
+        const float o = __shfl_xor(v[g], d, SOCKET_WAVE);
+        v[g] = is_max ? fmaxf(v[g], o) : v[g] + o;
+      }
+    }
+    __syncthreads();  // earlier readers of `red` are done
+    if (lane == 0) {
+#pragma unroll
+      for (int g = 0; g < kSHMaxG; ++g) red[wave][g] = v[g];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < kSHMaxG; ++g) {
+      float a = red[0][g];
+#pragma unroll
+      for (int w = 1; w < kSHWaves; ++w) a = is_max ? fmaxf(a, red[w][g]) : a + red[w][g];
+      v[g] = a;
+    }
+  };
+
+  float lg[kSHMaxG][4];
+  float mx[kSHMaxG], sm[kSHMaxG];
+#pragma unroll
+  for (int g = 0; g < kSHMaxG; ++g) {
+    mx[g] = -INFINITY;
+    sm[g] = 0.f;
+  }
+  for (int r0 = tid * 4; r0 < R; r0 += kSHThreads * 4) {
+    logits4(r0, lg);
+#pragma unroll
+    for (int g = 0; g < kSHMaxG; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx[g] = fmaxf(mx[g], lg[g][i]);
+  }
+  reduce(mx, true);
+  for (int r0 = tid * 4; r0 < R; r0 += kSHThreads * 4) {
+    logits4(r0, lg);
+#pragma unroll
+    for (int g = 0; g < kSHMaxG; ++g)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sm[g] += expf(lg[g][i] - mx[g]);
+  }
+  reduce(sm, false);
+  for (int r0 = tid * 4; r0 < R; r0 += kSHThreads * 4) {
+    logits4(r0, lg);
+#pragma unroll
+    for (int g = 0; g < kSHMaxG; ++g) {
+      if (g < G) {
+        float p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[i] = expf(lg[g][i] - mx[g]) / sm[g];
+        const int64_t o = (((int64_t)b * Hq + kvh * G + g) * L + l) * R + r0;
+        if (out_dtype == SOCKET_F32) {
+          *reinterpret_cast<float4*>((float*)out + o) = make_float4(p[0], p[1], p[2], p[3]);
+        } else {
+          uint2 w;
+          w.x = (uint32_t)f32_to_bf16_bits(p[0]) | ((uint32_t)f32_to_bf16_bits(p[1]) << 16);
+          w.y = (uint32_t)f32_to_bf16_bits(p[2]) | ((uint32_t)f32_to_bf16_bits(p[3]) << 16);
+          *reinterpret_cast<uint2*>((uint16_t*)out + o) = w;
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int socket_soft_hash(const void* q, int dtype, int64_t q_stride_b, int64_t q_stride_h,
+                                const void* planes, const void* protos_T, void* out, int out_dtype,
+                                int B, int Hq, int Hkv, int D, int L, int K, int R,
+                                float tanh_scale, float inv_temperature, void* stream) {
+  SOCKET_REQUIRE(q && planes && protos_T && out, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(socket_dtype_bytes(dtype) != 0, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(out_dtype == SOCKET_F32 || out_dtype == SOCKET_BF16, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L > 0, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(D >= 1 && D <= kSHMaxD && K >= 1 && K <= kSHMaxK, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(Hq / Hkv <= kSHMaxG, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(R >= 4 && R % 4 == 0, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE((int64_t)B * Hkv <= 65535, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(socket_aligned16(out), SOCKET_ERR_ALIGN);
+  const dim3 grid(L, B * Hkv);
+  hipStream_t s = (hipStream_t)stream;
+#define SOCKET_SH(DT)                                                                               \
+  hipLaunchKernelGGL((soft_hash_kernel<DT>), grid, dim3(kSHThreads), 0, s, q, q_stride_b, q_stride_h, \
+                     planes, protos_T, out, out_dtype, Hq, Hkv, Hq / Hkv, D, L, K, R, tanh_scale,     \
+                     inv_temperature)
+  if (dtype == SOCKET_F32) SOCKET_SH(DType_f32);
+  else if (dtype == SOCKET_BF16) SOCKET_SH(DType_bf16);
+  else SOCKET_SH(DType_f16);
+#undef SOCKET_SH
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}

@@ -16,6 +16,7 @@ Nothing on the step path reads a length back to the host.
 """
 from __future__ import annotations
 
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -107,6 +108,36 @@ def pack_codes_into(codes_i16_bhlt: torch.Tensor, codes: torch.Tensor, P: int, t
         check("socket_pack_codes", lib().socket_pack_codes(
             ptr(c), c.stride(0), c.stride(1), c.stride(2), c.stride(3), ptr(codes), B, Hkv, L, int(P),
             int(t0), T, codes.shape[3], stream_ptr(codes.device)))
+
+
+@torch.no_grad()
+def soft_hash(queries_bhd: torch.Tensor, planes_lkd: torch.Tensor, protos_T: torch.Tensor,
+              temperature: float = 1.0, n_kv_heads: Optional[int] = None,
+              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Query soft bucket probabilities [B,Hq,L,R] in one launch:
+    softmax_r((tanh(q . planes) / sqrt(D)) @ protos_T / temperature)
+    (GPT-FAST/model.py:392-401 with temperature 1; modeling_llama.py:618-638 with
+    0.3).  fp32 arithmetic on the stored inputs, one rounding to `out_dtype`
+    (bfloat16 for bfloat16 queries, else float32)."""
+    assert queries_bhd.is_cuda and queries_bhd.dim() == 3 and queries_bhd.stride(-1) == 1
+    B, Hq, D = queries_bhd.shape
+    L, K, D2 = planes_lkd.shape
+    K2, R = protos_T.shape
+    assert D2 == D and K2 == K
+    dt = queries_bhd.dtype
+    planes_lkd = planes_lkd.to(dt).contiguous()
+    protos_T = protos_T.to(dt).contiguous()
+    if out_dtype is None:
+        out_dtype = torch.bfloat16 if dt == torch.bfloat16 else torch.float32
+    Hkv = n_kv_heads if n_kv_heads else Hq
+    if Hq % Hkv != 0 or Hq // Hkv > 8:
+        Hkv = Hq
+    out = torch.empty((B, Hq, L, R), dtype=out_dtype, device=queries_bhd.device)
+    check("socket_soft_hash", lib().socket_soft_hash(
+        ptr(queries_bhd), dtype_enum(dt), queries_bhd.stride(0), queries_bhd.stride(1), ptr(planes_lkd),
+        ptr(protos_T), ptr(out), dtype_enum(out_dtype), B, Hq, Hkv, D, L, K, R,
+        1.0 / max(math.sqrt(D), 1e-6), 1.0 / float(temperature), stream_ptr(queries_bhd.device)))
+    return out
 
 
 @torch.no_grad()

@@ -179,7 +179,7 @@ class KVCache(nn.Module):
         return self.k_cache, self.v_cache
 
 
-# The three places where the attention hook enters the HIP library.  They are
+# The places where the attention hook enters the HIP library.  They are
 # module-level so that a test can stand a checker in for one of them; the
 # product has no other route.
 def _hash_rows(cache: KVCache, k_bshd: Tensor, v_bshd: Tensor, t0: int = 0, pos_b: Optional[Tensor] = None) -> None:
@@ -195,6 +195,10 @@ def _sparse_step(q_bhd: Tensor, q_probs: Tensor, cache: KVCache, T: int, sink: i
 
 def _dense_step(q_bhd: Tensor, cache: KVCache) -> Tensor:
     return dense_decode_fwd(q_bhd, cache.k_cache, cache.v_cache, cache.lens)
+
+
+def _soft_hash(q_bhd: Tensor, planes: Tensor, protos_T: Tensor, n_kv_heads: int) -> Tensor:
+    return hash_cache.soft_hash(q_bhd, planes, protos_T, 1.0, n_kv_heads)
 
 
 def _planes_to_words(planes: Tensor) -> Tensor:
@@ -325,7 +329,10 @@ class Attention(nn.Module):
 
     # ---- hashes (GPT-FAST/model.py:392-413) ------------------------------------------
     def soft_hash(self, queries_bhd: Tensor) -> Tensor:
-        """softmax_r( tanh(q . planes) / sqrt(D) @ protos_T ): [B,H,D] -> [B,H,L,R]."""
+        """softmax_r( tanh(q . planes) / sqrt(D) @ protos_T ): [B,H,D] -> [B,H,L,R].
+        One fused kernel on the device; the torch expression below on the host."""
+        if queries_bhd.is_cuda:
+            return _soft_hash(queries_bhd, self.planes, self.protos_T, self.n_local_heads)
         proj = torch.einsum("bhd,lkd->bhlk", queries_bhd, self.planes)
         temp = max(math.sqrt(queries_bhd.size(-1)), 1e-6)
         logits = torch.einsum("bhlk,kr->bhlr", torch.tanh(proj) / temp, self.protos_T)

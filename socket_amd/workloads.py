@@ -59,6 +59,9 @@ WORKLOADS = {
                    planted_frac=0.005, channel_scale=True),
     "c3": Workload("c3", 3, 4, 32, 8, 128, 131072, 60, 10, 2048, 4, 256, torch.bfloat16,
                    planted_frac=0.005, channel_scale=True),
+    # one attention layer of the 32-layer model run: one sequence, 65536 cached tokens
+    "c4": Workload("c4", 4, 1, 32, 8, 128, 65536, 60, 10, 2048, 4, 256, torch.bfloat16,
+                   planted_frac=0.005, channel_scale=True),
     "c5": Workload("c5", 5, 16, 28, 4, 128, 98304, 48, 10, 1966, 4, 128, torch.bfloat16,
                    planted_frac=0.005, channel_scale=True, ragged=True, t_min=16384, budget_frac=0.02),
 }

@@ -501,6 +501,54 @@ def test_pack_unpack_round_trip(dev):
         assert torch.equal(back, codes)
 
 
+# ---------------------------------------------------------------- K5 query soft hash
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,Hq,Hkv,D,L,K,R,temp,cube", [
+    (2, 8, 2, 128, 20, 10, 1024, 1.0, False),      # GPT-FAST: random prototypes, no temperature
+    (1, 28, 4, 128, 12, 10, 1024, 0.3, True),      # HF twin: hypercube corners, logits / 0.3, G = 7
+    (3, 4, 4, 64, 5, 4, 16, 1.0, True),            # small R, one head per group
+    (1, 6, 3, 32, 3, 3, 8, 0.3, False),
+])
+def test_soft_hash_matches_oracle(dev, dtype, B, Hq, Hkv, D, L, K, R, temp, cube):
+    g = torch.Generator().manual_seed(B * 1000 + Hq + L)
+    q = torch.randn(B, Hq, D, generator=g).to(dtype)
+    planes = (torch.randn(L, K, D, generator=g) * (1.0 if cube else 0.3)).to(dtype)
+    protos = (orc.hypercube_protos_T(K) if cube else torch.randn(K, R, generator=g) * 3.0).to(dtype)
+    want = orc.soft_hash(q.float(), planes.float(), protos.float(), temperature=temp)       # fp32 on the stored values
+    have32 = hash_cache.soft_hash(q.to(dev), planes.to(dev), protos.to(dev), temp, Hkv, out_dtype=torch.float32).cpu()
+    assert have32.dtype == torch.float32 and tuple(have32.shape) == (B, Hq, L, R)
+    torch.testing.assert_close(have32, want, rtol=2e-5, atol=1e-9)
+    torch.testing.assert_close(have32.sum(-1), torch.ones(B, Hq, L), rtol=1e-5, atol=1e-5)
+    # grouping of heads into workgroups does not change the values
+    alone = hash_cache.soft_hash(q.to(dev), planes.to(dev), protos.to(dev), temp, Hq, out_dtype=torch.float32).cpu()
+    assert torch.equal(alone, have32)
+    # bf16 output: the fp32 value rounded once
+    have16 = hash_cache.soft_hash(q.to(dev), planes.to(dev), protos.to(dev), temp, Hkv, out_dtype=torch.bfloat16).cpu()
+    assert have16.dtype == torch.bfloat16 and torch.equal(have16, have32.to(torch.bfloat16))
+    if cube and R == 1 << K:
+        # hypercube prototypes: the most probable bucket is the query's hard hash
+        proj = orc.projections_f64(q.float().unsqueeze(1).permute(0, 1, 2, 3).reshape(B, 1, Hq, D), planes.float())
+        clear = (proj.abs() > 1e-4).all(-1)[:, 0]                                            # [B,Hq,L]
+        hard = orc.pack_bits(proj >= 0)[:, 0].long()
+        assert torch.equal(have32.argmax(-1)[clear], hard[clear])
+
+
+def test_soft_hash_strided_queries_and_argument_checks(dev):
+    g = torch.Generator().manual_seed(9)
+    qkv = torch.randn(2, 1, 12, 128, generator=g).to(torch.bfloat16).to(dev)      # queries are heads 0..7 of a wider row
+    q = qkv[:, 0, :8]
+    planes = torch.randn(6, 10, 128, generator=g).to(torch.bfloat16).to(dev)
+    protos = torch.randn(10, 1024, generator=g).to(torch.bfloat16).to(dev)
+    a = hash_cache.soft_hash(q, planes, protos, 1.0, 2)
+    b = hash_cache.soft_hash(q.contiguous(), planes, protos, 1.0, 2)
+    assert a.dtype == torch.bfloat16 and torch.equal(a, b)
+    from socket_amd._lib import SocketHipError
+    with pytest.raises(SocketHipError):
+        hash_cache.soft_hash(q, planes, protos[:, :6].contiguous(), 1.0, 2)       # R not a multiple of 4
+    with pytest.raises(AssertionError):
+        hash_cache.soft_hash(q, planes[:, :4], protos, 1.0, 2)
+
+
 # ---------------------------------------------------------------- whole step
 @pytest.mark.parametrize("name,T", [("c1", 4096), ("c2", 8192)])
 def test_decode_step_end_to_end(dev, name, T):
