@@ -198,7 +198,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens,
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
     int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
-    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range) {
+    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit) {
   typedef typename TT::elem TE;
   const Bf16Select sel = make_bf16_select(bf16_one);
   constexpr int EPV = 16 / (int)sizeof(TE);   // table elements per 16-byte vector
@@ -226,12 +226,39 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     }
   }
   if (pair >= n_pairs) return;
+  // A group of more than GP query heads is shared out over `hsplit` workgroups
+  // (each streams the pair's codes): this one takes heads [h0, h0 + G) of it.
+  const int h0 = (pair % hsplit) * GP;
+  pair /= hsplit;
   const int b = pair / Hkv, kvh = pair % Hkv;
+  const int head0 = b * Hq + kvh * G + h0;   // first of this workgroup's query heads (rows of q_probs, scores)
+  G = min(GP, G - h0);
   const int tid = threadIdx.x;
   const int len = lens ? min(lens[b], T) : T;
 
+  if (tile * TW >= len) {
+    // nothing cached this far out for this sequence: the tile is all masked
+    for (int g = 0; g < G; ++g) {
+      float* dst = scores + ((int64_t)(head0 + g)) * score_stride + tile * TW;
+      const int n = min(TW, T - tile * TW);
+      for (int t = tid * 4; t < n; t += THREADS * 4) {
+        if (t + 4 <= n) {
+          store_stream16(dst + t, -INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        } else {
+          for (int i = t; i < n; ++i) dst[i] = -INFINITY;
+        }
+      }
+    }
+    if (row_range && tid < G) {
+      uint32_t* dst = row_range + (((int64_t)(head0 + tid)) * n_tiles + tile) * 2;
+      dst[0] = 0xffffffffu;
+      dst[1] = 0u;
+    }
+    return;
+  }
+
   const uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
-  const TE* qp_pair = q_probs + ((int64_t)(b * Hq + kvh * G)) * L * R;
+  const TE* qp_pair = q_probs + ((int64_t)head0) * L * R;
   const int chunk_tables = chunk_words * cpw;
   const int chunk_elems = chunk_tables * R * GP;  // table elements per LDS buffer
 
@@ -427,7 +454,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
           kmax[g] = max(kmax[g], key);
         }
       }
-      float* dst = scores + ((int64_t)(b * Hq + kvh * G + g)) * score_stride + tbase[j];
+      float* dst = scores + ((int64_t)(head0 + g)) * score_stride + tbase[j];
       if (tbase[j] + 4 <= T) {
         store_stream16(dst, o[0], o[1], o[2], o[3]);
       } else {
@@ -461,7 +488,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
         lo = min(lo, red[(w * GP + tid) * 2]);
         hi = max(hi, red[(w * GP + tid) * 2 + 1]);
       }
-      uint32_t* dst = row_range + (((int64_t)(b * Hq + kvh * G + tid)) * n_tiles + tile) * 2;
+      uint32_t* dst = row_range + (((int64_t)(head0 + tid)) * n_tiles + tile) * 2;
       dst[0] = lo;
       dst[1] = hi;
     }
@@ -514,13 +541,14 @@ int launch_score_packed(const ScoreArgs& a) {
   constexpr int TW = THREADS * 4 * KT4;
   const int n_tiles = (a.T + TW - 1) / TW;
   if (a.row_range && a.range_parts != n_tiles) return SOCKET_ERR_SHAPE;
-  const int n_pairs = a.B * a.Hkv;
+  const int hsplit = (G + GP - 1) / GP;
+  const int n_pairs = a.B * a.Hkv * hsplit;
   const int xcd_remap = (n_pairs % 8 == 0) ? 1 : 0;
   const int n_wg = n_pairs * n_tiles;
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
                      a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
                      a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, xcd_remap, 0x3f80u,
-                     a.row_range);
+                     a.row_range, hsplit);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }
@@ -537,8 +565,8 @@ int dispatch_p(const ScoreArgs& a) {
 // refills again but does not fit 128 registers next to the prefetched codes.)
 int tile_tokens(int B, int Hkv, int G, int T) {
   const SocketDeviceLimits& lim = socket_device_limits();
-  const int64_t pairs = (int64_t)B * Hkv;
-  if (G <= 4 && pairs * ((T + 8191) / 8192) >= lim.cu_count) return 8192;
+  const int64_t pairs = (int64_t)B * Hkv * ((G + 3) / 4);  // groups of 5..8 heads go as two workgroups
+  if (pairs * ((T + 8191) / 8192) >= lim.cu_count) return 8192;
   if (pairs * ((T + 4095) / 4096) >= lim.cu_count) return 4096;
   if (pairs * ((T + 2047) / 2048) >= lim.cu_count) return 2048;
   return 1024;
@@ -547,9 +575,7 @@ int tile_tokens(int B, int Hkv, int G, int T) {
 template <int GP, class TT>
 int dispatch_tile(const ScoreArgs& a) {
   const int tw = tile_tokens(a.B, a.Hkv, a.Hq / a.Hkv, a.T);
-  if constexpr (GP <= 4) {
-    if (tw == 8192) return dispatch_p<GP, TT, 2, 1024>(a);
-  }
+  if (tw == 8192) return dispatch_p<GP, TT, 2, 1024>(a);
   if (tw == 4096) return dispatch_p<GP, TT, 2, 512>(a);
   if (tw == 2048) return dispatch_p<GP, TT, 1, 512>(a);
   return dispatch_p<GP, TT, 1, 256>(a);
@@ -560,8 +586,7 @@ int dispatch_g(const ScoreArgs& a) {
   const int G = a.Hq / a.Hkv;
   if (G == 1) return dispatch_tile<1, TT>(a);
   if (G == 2) return dispatch_tile<2, TT>(a);
-  if (G <= 4) return dispatch_tile<4, TT>(a);
-  return dispatch_tile<8, TT>(a);
+  return dispatch_tile<4, TT>(a);
 }
 
 // ---------------------------------------------------------------------------
