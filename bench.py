@@ -59,6 +59,7 @@ def algorithmic_bytes(w, lens=None, budgets=None):
         "score": w.Hkv * tok * (wc + 2 + 4 * G),
         "score_f32": w.Hkv * tok * (wc + 2 + 4 * G),
         "score_f32_table": w.Hkv * tok * (wc + 2 + 4 * G),
+        "score_reference_layout": w.Hkv * tok * (wc + 2 + 4 * G),
         "select": sel,
         "select_own_range": sel,
         "attend": w.Hq * kt * (4 * w.D + 4) + w.B * w.Hq * 4 * w.D,
@@ -164,7 +165,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--only", default=None,
-                    choices=["score", "score_f32", "select", "attend", "hash", "dense", "copy"])
+                    choices=["score", "score_f32", "score_grouped", "select", "attend", "hash", "dense", "copy"])
+    ap.add_argument("--reference-table-layout", action="store_true",
+                    help="feed the scorer q_probs as [B,Hq,L,R] instead of the grouped layout the soft-hash kernel writes")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of a recorded HIP graph")
@@ -235,6 +238,15 @@ def main():
     def k_score():
         return hash_cache.score_packed(q_table, codes, v_norm, T, w.P, lens=lens, out=scores_buf, with_range=True)
 
+    # ... and in the layout the fused soft-hash kernel writes it in (heads of a KV head
+    # interleaved per bucket: the scorer's LDS image); same values
+    q_table_grouped = hash_cache.group_q_probs(q_table, Hkv)
+    use_grouped = not args.reference_table_layout
+
+    def k_score_grouped():
+        return hash_cache.score_packed(q_table_grouped, codes, v_norm, T, w.P, lens=lens, out=scores_buf,
+                                       with_range=True, n_heads=Hq)
+
     def k_score_f32():
         return hash_cache.score_packed(q_table_f32, codes, v_norm, T, w.P, lens=lens, out=scores_buf)
 
@@ -251,11 +263,11 @@ def main():
 
     def step():
         k_hash()
-        s, r = k_score()
+        s, r = k_score_grouped() if use_grouped else k_score()
         sl, ln = k_select(s, r)
         return k_attend(sl, ln)
 
-    scores, rng = k_score()
+    scores, rng = k_score_grouped() if use_grouped else k_score()
     sl, ln = k_select(scores, rng)
     out = k_attend(sl, ln)
     torch.cuda.synchronize()
@@ -271,11 +283,11 @@ def main():
                           "us": round(us, 2), "gbs": round(2 * a.numel() * 4 / us / 1e3, 1), "iters": iters}))
         return
     if args.only:
-        fn = {"score": k_score, "score_f32": k_score_f32, "select": lambda: k_select(scores, rng), "attend": lambda: k_attend(sl, ln),
+        fn = {"score": k_score, "score_f32": k_score_f32, "score_grouped": k_score_grouped, "select": lambda: k_select(scores, rng), "attend": lambda: k_attend(sl, ln),
               "hash": k_hash, "dense": k_dense}[args.only]
         us = time_launches(fn, iters, warmup=args.warmup)
         print(json.dumps({"only": args.only, "workload": w.name, "us": round(us, 2),
-                          "gbs": round(abytes[args.only] / us / 1e3, 1), "iters": iters}))
+                          "gbs": round(abytes[args.only.replace("_grouped", "")] / us / 1e3, 1), "iters": iters}))
         return
 
     # ---- parity gates on the full-size run (device-side checks, not timed) --------------
@@ -309,7 +321,8 @@ def main():
     # ---- per-kernel timings ------------------------------------------------------------------
     per = {
         "hash": time_launches(k_hash, iters),
-        "score": time_launches(k_score, iters),
+        "score": time_launches(k_score_grouped if use_grouped else k_score, iters),
+        "score_reference_layout": time_launches(k_score, iters),
         "score_f32_table": time_launches(k_score_f32, iters),
         "select": time_launches(lambda: k_select(scores, rng), iters),
         "select_own_range": time_launches(lambda: k_select(scores), iters),
@@ -385,7 +398,8 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"{w.name}: B{B} Hq{Hq}/Hkv{Hkv} D{D} T{T} bf16 KV cache, L{w.L}xP{w.P} packed codes, "
-                               f"{str(q_table.dtype).split('.')[-1]} soft-hash table, "
+                               f"{str(q_table.dtype).split('.')[-1]} soft-hash table "
+                               f"({'grouped' if use_grouped else '[B,Hq,L,R]'} layout), "
                                f"top-k {w.M} + sink {w.sink} + window {w.window}"
                                + (", ragged lengths" if w.ragged else ""),
                    "layers_timed": 1, "new_keys_hashed_per_step": B * Hkv * w.new_keys,

@@ -132,6 +132,27 @@ int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
                         int B, int Hq, int Hkv, int L, int P, int R, int T, int64_t Tcap,
                         int64_t score_stride, void* stream);
 
+/* Grouped table layout.  The scorer gathers from an LDS image of the table in which
+ * the query heads that share a KV head are interleaved: [table][bucket][head].
+ * A table already stored that way is copied into LDS as it is:
+ *   q_table [B*Hkv*parts, L, R, width]  (same element type as q_probs)
+ *   element (b*Hkv + kvh, part, l, r, g) = q_probs[b, kvh*G + part*width + g, l, r],
+ *   zero where part*width + g >= G;  socket_group_shape gives width (1, 2 or 4)
+ *   and parts (2 for G = 5..8, else 1).
+ * socket_group_q_probs converts a [B,Hq,L,R] table; socket_soft_hash_grouped
+ * produces the layout directly.  socket_score_packed_grouped is socket_score_packed
+ * on such a table: same arguments, same results, except that its row_range has
+ * socket_score_range_parts_grouped(...) parts (its tiles can be of another size). */
+int socket_group_shape(int Hq, int Hkv, int* parts, int* width);
+int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int P, int R);
+int socket_group_q_probs(const void* q_probs, int q_dtype, void* q_table, int B, int Hq, int Hkv,
+                         int L, int R, void* stream);
+int socket_score_packed_grouped(const void* q_table, int q_dtype, const uint32_t* codes,
+                                const uint16_t* v_norm, const int32_t* lens, float* scores,
+                                uint32_t* row_range, int range_parts,
+                                int B, int Hq, int Hkv, int L, int P, int R, int T, int64_t Tcap,
+                                int64_t score_stride, void* stream);
+
 /* The reference extension's entry point on its own layout:
  * q_probs f32 [B,H,1,L,R], key_buckets i16 [B,H,L,T], allowed bool [B,H,1,T],
  * v_hist f32 [B,H,1,T] -> out f32 [B,H,1,T], all contiguous.
@@ -164,6 +185,12 @@ int socket_soft_hash(const void* q, int dtype, int64_t q_stride_b, int64_t q_str
                      const void* planes, const void* protos_T, void* out, int out_dtype,
                      int B, int Hq, int Hkv, int D, int L, int K, int R,
                      float tanh_scale, float inv_temperature, void* stream);
+/* The same, written in the grouped table layout described at
+ * socket_score_packed_grouped (Hkv must then be the real number of KV heads). */
+int socket_soft_hash_grouped(const void* q, int dtype, int64_t q_stride_b, int64_t q_stride_h,
+                             const void* planes, const void* protos_T, void* q_table, int out_dtype,
+                             int B, int Hq, int Hkv, int D, int L, int K, int R,
+                             float tanh_scale, float inv_temperature, void* stream);
 
 /* ------------------------------------------------------------------------
  * K3  top-k select and index list

@@ -46,6 +46,11 @@ SIGNATURES = {
     "socket_score_packed": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
     "socket_soft_hash_collision": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "socket_soft_hash_score_f16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "socket_group_shape": (_I, [_I, _I, POINTER(c_int), POINTER(c_int)]),
+    "socket_score_range_parts_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I]),
+    "socket_group_q_probs": (_I, [_P, _I, _P, _I, _I, _I, _I, _I, _P]),
+    "socket_score_packed_grouped": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
+    "socket_soft_hash_grouped": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),
     "socket_soft_hash": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),
     "socket_select_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "socket_select_list": (_I, [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _P, _Z, _P]),

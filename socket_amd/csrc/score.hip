@@ -15,6 +15,9 @@
 //    lane, fully coalesced, three words ahead of their use.  The table may be
 //    fp32 or bf16 (a bf16 soft-hash producer loses nothing, halves the LDS bytes
 //    per gather and lets the matrix core do the four head adds of a lookup).
+//    A table given in the grouped layout (the LDS image itself, written by the
+//    soft-hash kernel) is copied rather than interleaved, and for large launches
+//    the copy is global_load_lds: global memory straight into LDS.
 //  * collision_i16_kernel: the reference's own operand layout (int16 codes per
 //    query head), for drop-in callers.
 #include "socket_common.h"
@@ -77,6 +80,37 @@ __device__ __forceinline__ uint4 load_stream16(const uint32_t* p) {
   const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+// 16 bytes per lane from global memory straight into LDS: lane i's bytes land at
+// lds_dst + 16 * i (lds_dst is the same for the whole wave).  Written as assembly
+// so that the compiler does not serialise later LDS reads behind it; M0, which
+// carries the LDS address, is saved and restored.  Completion: vmcnt.
+__device__ __forceinline__ void lds_dma16(const void* src_lane, void* lds_dst) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_dst);
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src_lane), "s"(base)
+      : "memory");
+}
+
+// s_waitcnt vmcnt(n) only (n <= 15 here; larger requests wait for 15)
+__device__ __forceinline__ void wait_vmcnt(int n) {
+#define SOCKET_VM(k) \
+  case k: __builtin_amdgcn_s_waitcnt((k) | (7 << 4) | (15 << 8)); break;
+  switch (n) {
+    SOCKET_VM(0) SOCKET_VM(1) SOCKET_VM(2) SOCKET_VM(3) SOCKET_VM(4) SOCKET_VM(5) SOCKET_VM(6) SOCKET_VM(7)
+    SOCKET_VM(8) SOCKET_VM(9) SOCKET_VM(10) SOCKET_VM(11) SOCKET_VM(12) SOCKET_VM(13) SOCKET_VM(14)
+    default: __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (15 << 8)); break;
+  }
+#undef SOCKET_VM
+}
+
 __device__ __forceinline__ void store_stream16(float* p, float a, float b, float c, float d) {
   float4_t v = {a, b, c, d};
   __builtin_nontemporal_store(v, reinterpret_cast<float4_t*>(p));
@@ -192,13 +226,14 @@ __device__ __forceinline__ void interleave_heads(const uint4 (&x)[GP], uint4 (&o
 // The table slice of the tables held by `chunk_words` packed words sits in LDS;
 // with two LDS buffers the next slice is fetched into registers while the
 // current one is being gathered from, and there is one barrier per slice.
-template <int GP, class TT, int KT4, int THREADS, int PT>
+template <int GP, class TT, int KT4, int THREADS, int PT, bool DMA>
 __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     const typename TT::elem* __restrict__ q_probs, const uint32_t* __restrict__ codes,
     const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens,
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
     int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
-    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit) {
+    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit,
+    int grouped) {
   typedef typename TT::elem TE;
   const Bf16Select sel = make_bf16_select(bf16_one);
   constexpr int EPV = 16 / (int)sizeof(TE);   // table elements per 16-byte vector
@@ -208,7 +243,11 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   const int P = PT ? PT : P_rt;
   const int cpw = 32 / P;
   const uint32_t code_mask = (1u << P) - 1u;
-  constexpr int TW = THREADS * 4 * KT4;
+  // DMA: table slices (grouped layout only) go from global memory straight into
+  // LDS, 1 KB per instruction, shared out over the waves; no staging registers,
+  // no interleave, no LDS store instructions.
+  constexpr int CT = THREADS;  // lanes that own tokens
+  constexpr int TW = CT * 4 * KT4;
 
   // Workgroup -> (pair, tile).  Workgroups are dealt to the 8 XCDs round-robin
   // by linear id; with the remap all tiles of one (b, kv head) land on one XCD,
@@ -228,6 +267,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   if (pair >= n_pairs) return;
   // A group of more than GP query heads is shared out over `hsplit` workgroups
   // (each streams the pair's codes): this one takes heads [h0, h0 + G) of it.
+  const int vpair = pair;  // (b, kv head, part of the head group)
   const int h0 = (pair % hsplit) * GP;
   pair /= hsplit;
   const int b = pair / Hkv, kvh = pair % Hkv;
@@ -258,7 +298,9 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   }
 
   const uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
-  const TE* qp_pair = q_probs + ((int64_t)head0) * L * R;
+  // reference layout: row `head0` of [B*Hq, L, R]; grouped layout: block `vpair` of
+  // [B*Hkv*hsplit, L, R, GP], which is the LDS layout itself
+  const TE* qp_pair = grouped ? q_probs + (int64_t)vpair * L * R * GP : q_probs + ((int64_t)head0) * L * R;
   const int chunk_tables = chunk_words * cpw;
   const int chunk_elems = chunk_tables * R * GP;  // table elements per LDS buffer
 
@@ -268,8 +310,8 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   bool live[KT4];
 #pragma unroll
   for (int j = 0; j < KT4; ++j) {
-    tbase[j] = tile * TW + j * (THREADS * 4) + tid * 4;
-    live[j] = tbase[j] < T;
+    tbase[j] = tile * TW + j * (CT * 4) + tid * 4;
+    live[j] = tid < CT && tbase[j] < T;
     tsafe[j] = live[j] ? tbase[j] : tile * TW;
   }
 
@@ -285,7 +327,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   // word being consumed, ring[d] the word d steps ahead.  The code stream is the
   // HBM traffic of this kernel and a CU needs tens of KB of it in flight to cover
   // the memory latency; one word ahead (16 B x tokens/4 per lane) is not enough.
-  constexpr int kPrefetch = 3;
+  constexpr int kPrefetch = DMA ? 4 : 3;  // the direct-to-LDS variant has the registers for one more
   uint4 ring[kPrefetch][KT4];
 #pragma unroll
   for (int d = 0; d < kPrefetch; ++d)
@@ -305,6 +347,17 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   auto stage_load = [&](int l0) {
     const int nt = min(chunk_tables, L - l0);
     const int nslots = (nt * R) / EPV;
+    if (grouped) {  // straight copy: 16-byte vector i of the slice goes to vector i of the buffer
+      const uint4* src = reinterpret_cast<const uint4*>(qp_pair + (int64_t)l0 * R * GP);
+#pragma unroll
+      for (int k = 0; k < SL; ++k)
+#pragma unroll
+        for (int g = 0; g < GP; ++g) {
+          const int i = tid + (k * GP + g) * THREADS;
+          if (i < nslots * GP) stage[k][g] = src[i];
+        }
+      return;
+    }
     const TE* src = qp_pair + (int64_t)l0 * R;
 #pragma unroll
     for (int k = 0; k < SL; ++k) {
@@ -321,6 +374,16 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     const int nt = min(chunk_tables, L - l0);
     const int nslots = (nt * R) / EPV;
     uint4* dst = reinterpret_cast<uint4*>(lds_raw + (size_t)buf * chunk_elems * sizeof(TE));
+    if (grouped) {
+#pragma unroll
+      for (int k = 0; k < SL; ++k)
+#pragma unroll
+        for (int g = 0; g < GP; ++g) {
+          const int i = tid + (k * GP + g) * THREADS;
+          if (i < nslots * GP) dst[i] = stage[k][g];
+        }
+      return;
+    }
 #pragma unroll
     for (int k = 0; k < SL; ++k) {
       const int s = tid + k * THREADS;
@@ -333,8 +396,24 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     }
   };
 
+  // DMA: this wave's share of the slice that starts at table l0 -> buffer `buf`
+  // (every 16th 1 KB piece); returns nothing, completion is awaited with vmcnt
+  auto dma_slice = [&](int l0, int buf) {
+    const int nt = min(chunk_tables, L - l0);
+    const int bytes = nt * R * GP * (int)sizeof(TE);
+    const char* src = reinterpret_cast<const char*>(qp_pair + (int64_t)l0 * R * GP);
+    unsigned char* dst = lds_raw + (size_t)buf * chunk_elems * sizeof(TE);
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int o = wave * 1024; o < bytes; o += (THREADS / SOCKET_WAVE) * 1024) {
+      if (o + lane * 16 < bytes) lds_dma16(src + o + lane * 16, dst + o);
+    }
+  };
   const bool staged = nbuf == 2;
-  if (staged) {
+  if (DMA) {
+    dma_slice(0, 0);
+    wait_vmcnt(0);    // (the code prefetches above are waited for too; once per workgroup)
+    __syncthreads();  // slice 0 is in place
+  } else if (staged) {
     stage_load(0);
     stage_store(0, 0);
     __syncthreads();
@@ -345,7 +424,9 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     const int l0 = w0 * cpw;
     const int buf = staged ? (chunk & 1) : 0;
     const bool more = w0 + chunk_words < NW;
-    if (staged) {
+    if (DMA) {
+      if (more) dma_slice(l0 + chunk_tables, buf ^ 1);
+    } else if (staged) {
       if (more) stage_load(l0 + chunk_tables);
     } else {
       __syncthreads();  // gathers of the previous slice are done
@@ -353,7 +434,11 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
       const int nslots = (nt * R) / EPV;
       const TE* src = qp_pair + (int64_t)l0 * R;
       uint4* dst = reinterpret_cast<uint4*>(lds_raw);
-      for (int s = tid; s < nslots; s += THREADS) {
+      if (grouped) {
+        const uint4* src16 = reinterpret_cast<const uint4*>(qp_pair + (int64_t)l0 * R * GP);
+        for (int i = tid; i < nslots * GP; i += THREADS) dst[i] = src16[i];
+      }
+      for (int s = tid; s < (grouped ? 0 : nslots); s += THREADS) {
         uint4 x[GP], o[GP];
 #pragma unroll
         for (int g = 0; g < GP; ++g)
@@ -416,7 +501,14 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
       }
     }
 
-    if (staged) {
+    if (DMA) {
+      // The direct loads were issued at the top of the slice; since then this wave
+      // has issued one code prefetch per word and token group.  Loads retire in
+      // order, so allowing that many to be outstanding, less one word's worth as a
+      // margin, means the direct loads have landed.
+      wait_vmcnt(max(0, (min(w0 + chunk_words, NW) - w0 - 1) * KT4));
+      __syncthreads();
+    } else if (staged) {
       if (more) stage_store(l0 + chunk_tables, buf ^ 1);
       __syncthreads();
     }
@@ -506,9 +598,10 @@ struct ScoreArgs {
   uint32_t* row_range;
   int range_parts;
   hipStream_t stream;
+  int grouped;  // table layout: 0 = [B,Hq,L,R], 1 = [B*Hkv*parts, L, R, group width]
 };
 
-template <int GP, class TT, int KT4, int THREADS, int PT>
+template <int GP, class TT, int KT4, int THREADS, int PT, bool DMA>
 int launch_score_packed(const ScoreArgs& a) {
   typedef typename TT::elem TE;
   const SocketDeviceLimits& lim = socket_device_limits();
@@ -518,11 +611,15 @@ int launch_score_packed(const ScoreArgs& a) {
   constexpr int EPV = 16 / (int)sizeof(TE);
   const size_t bytes_per_word = (size_t)cpw * a.R * GP * sizeof(TE);
   const size_t slots_per_word = (size_t)cpw * a.R / EPV;
-  // Double-buffered when one word's tables fit twice in LDS and in the staging
-  // registers (1024 vector slots per workgroup); as many words per slice as that
-  // allows.  Otherwise a single buffer filled in place.
   int nbuf = 2, chunk_words = 1;
-  if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && slots_per_word <= 1024) {
+  if (DMA) {
+    // two buffers, as many words per slice as LDS holds (no register staging to fit)
+    if (!a.grouped || 2 * bytes_per_word > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
+    while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= (size_t)lim.max_lds_per_block) ++chunk_words;
+  } else if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && slots_per_word <= 1024) {
+    // Double-buffered when one word's tables fit twice in LDS and in the staging
+    // registers (1024 vector slots per workgroup); as many words per slice as that
+    // allows.  Otherwise a single buffer filled in place.
     while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= (size_t)lim.max_lds_per_block / 2 &&
            slots_per_word * (chunk_words + 1) <= 1024)
       ++chunk_words;
@@ -532,7 +629,7 @@ int launch_score_packed(const ScoreArgs& a) {
   }
   const size_t lds_bytes = bytes_per_word * chunk_words * nbuf;
 
-  auto kern = score_packed_kernel<GP, TT, KT4, THREADS, PT>;
+  auto kern = score_packed_kernel<GP, TT, KT4, THREADS, PT, DMA>;
   if (lds_bytes > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
@@ -548,24 +645,34 @@ int launch_score_packed(const ScoreArgs& a) {
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
                      a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
                      a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, xcd_remap, 0x3f80u,
-                     a.row_range, hsplit);
+                     a.row_range, hsplit, a.grouped);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }
 
-template <int GP, class TT, int KT4, int THREADS>
+template <int GP, class TT, int KT4, int THREADS, bool DMA = false>
 int dispatch_p(const ScoreArgs& a) {
-  if (a.P == 10) return launch_score_packed<GP, TT, KT4, THREADS, 10>(a);
-  if (a.P == 8) return launch_score_packed<GP, TT, KT4, THREADS, 8>(a);
-  return launch_score_packed<GP, TT, KT4, THREADS, 0>(a);
+  if (a.P == 10) return launch_score_packed<GP, TT, KT4, THREADS, 10, DMA>(a);
+  if (a.P == 8) return launch_score_packed<GP, TT, KT4, THREADS, 8, DMA>(a);
+  return launch_score_packed<GP, TT, KT4, THREADS, 0, DMA>(a);
 }
 
+constexpr int kDmaKT4 = 2;  // token groups of four per lane in the direct-to-LDS variant
+constexpr int kDmaTile = 1024 * 4 * kDmaKT4 + 1;  // 8192-token tiles; the odd value only tags the variant
+
 // Tile size: the largest of 8192 / 4096 / 2048 / 1024 tokens per workgroup that
-// still gives every CU a workgroup.  (16 tokens per lane would halve the table
-// refills again but does not fit 128 registers next to the prefetched codes.)
-int tile_tokens(int B, int Hkv, int G, int T) {
+// still gives every CU a workgroup.  With a grouped table the largest tile uses
+// the direct-to-LDS variant.
+int tile_tokens(int B, int Hkv, int G, int T, int grouped, size_t table_elem_bytes, int P, int R) {
   const SocketDeviceLimits& lim = socket_device_limits();
-  const int64_t pairs = (int64_t)B * Hkv * ((G + 3) / 4);  // groups of 5..8 heads go as two workgroups
+  const int width = G == 1 ? 1 : G == 2 ? 2 : 4;
+  const int64_t pairs = (int64_t)B * Hkv * ((G + width - 1) / width);  // groups of 5..8 heads go as two workgroups
+  if (grouped && P > 0) {
+    const size_t bytes_per_word = (size_t)(32 / P) * R * width * table_elem_bytes;
+    constexpr int tw = 1024 * 4 * kDmaKT4;
+    if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && pairs * ((T + tw - 1) / tw) >= lim.cu_count)
+      return kDmaTile;
+  }
   if (pairs * ((T + 8191) / 8192) >= lim.cu_count) return 8192;
   if (pairs * ((T + 4095) / 4096) >= lim.cu_count) return 4096;
   if (pairs * ((T + 2047) / 2048) >= lim.cu_count) return 2048;
@@ -574,7 +681,8 @@ int tile_tokens(int B, int Hkv, int G, int T) {
 
 template <int GP, class TT>
 int dispatch_tile(const ScoreArgs& a) {
-  const int tw = tile_tokens(a.B, a.Hkv, a.Hq / a.Hkv, a.T);
+  const int tw = tile_tokens(a.B, a.Hkv, a.Hq / a.Hkv, a.T, a.grouped, sizeof(typename TT::elem), a.P, a.R);
+  if (tw == kDmaTile) return dispatch_p<GP, TT, kDmaKT4, 1024, true>(a);
   if (tw == 8192) return dispatch_p<GP, TT, 2, 1024>(a);
   if (tw == 4096) return dispatch_p<GP, TT, 2, 512>(a);
   if (tw == 2048) return dispatch_p<GP, TT, 1, 512>(a);
@@ -657,15 +765,23 @@ int launch_collision_i16(const QT* q_probs, const int16_t* key_buckets, const ui
 
 extern "C" int socket_score_range_parts(int B, int Hq, int Hkv, int T) {
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv != 0) return 0;
-  const int tw = tile_tokens(B, Hkv, Hq / Hkv, T);
+  const int tw = tile_tokens(B, Hkv, Hq / Hkv, T, 0, 0, 0, 0);
   return (T + tw - 1) / tw;
 }
 
-extern "C" int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
-                                   const uint16_t* v_norm, const int32_t* lens, float* scores,
-                                   uint32_t* row_range, int range_parts,
-                                   int B, int Hq, int Hkv, int L, int P, int R, int T,
-                                   int64_t Tcap, int64_t score_stride, void* stream) {
+extern "C" int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int P, int R) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv != 0 || P < 1 || P > 16 || R <= 0) return 0;
+  int tw = tile_tokens(B, Hkv, Hq / Hkv, T, 1, q_dtype == SOCKET_F32 ? 4 : 2, P, R);
+  if (tw == kDmaTile) tw = 1024 * 4 * kDmaKT4;
+  return (T + tw - 1) / tw;
+}
+
+namespace {
+
+int score_entry(const void* q_probs, int q_dtype, const uint32_t* codes, const uint16_t* v_norm,
+                const int32_t* lens, float* scores, uint32_t* row_range, int range_parts, int B, int Hq,
+                int Hkv, int L, int P, int R, int T, int64_t Tcap, int64_t score_stride, void* stream,
+                int grouped) {
   SOCKET_REQUIRE(q_probs && codes && v_norm && scores, SOCKET_ERR_NULL);
   SOCKET_REQUIRE(q_dtype == SOCKET_F32 || q_dtype == SOCKET_BF16, SOCKET_ERR_UNSUPPORTED);
   SOCKET_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0 && T > 0, SOCKET_ERR_SHAPE);
@@ -673,15 +789,85 @@ extern "C" int socket_score_packed(const void* q_probs, int q_dtype, const uint3
   SOCKET_REQUIRE(P >= 1 && P <= 16, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(R >= (1 << P) && (R & (R - 1)) == 0 && R >= 8, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(T <= Tcap && score_stride >= T, SOCKET_ERR_SHAPE);
-  SOCKET_REQUIRE((int64_t)B * Hkv * ((T + 1023) / 1024) < (1LL << 31), SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE((int64_t)B * Hkv * 2 * ((T + 1023) / 1024) < (1LL << 31), SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(Tcap % 4 == 0 && score_stride % 4 == 0, SOCKET_ERR_ALIGN);
   SOCKET_REQUIRE(socket_aligned16(q_probs) && socket_aligned16(codes) && socket_aligned16(v_norm) &&
                      socket_aligned16(scores),
                  SOCKET_ERR_ALIGN);
   SOCKET_REQUIRE(Hq / Hkv <= 8, SOCKET_ERR_UNSUPPORTED);
   const ScoreArgs a{q_probs, codes, v_norm, lens, scores, B, Hq, Hkv, L, P, R, T, Tcap, score_stride,
-                    row_range, range_parts, (hipStream_t)stream};
+                    row_range, range_parts, (hipStream_t)stream, grouped};
   return q_dtype == SOCKET_F32 ? dispatch_g<TabF32>(a) : dispatch_g<TabBF16>(a);
+}
+
+// [B,Hq,L,R] -> [B*Hkv*parts, L, R, width]: element (pair, part, l, r, g) is head
+// kvh*G + part*width + g of the pair, zero where that is past the group.
+template <typename TE>
+__global__ __launch_bounds__(256) void group_q_probs_kernel(const TE* __restrict__ in, TE* __restrict__ out,
+                                                            int Hq, int Hkv, int G, int parts, int width,
+                                                            int64_t LR, int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int g = (int)(i % width);
+    const int64_t lr = (i / width) % LR;
+    const int64_t blk = i / ((int64_t)width * LR);
+    const int part = (int)(blk % parts);
+    const int64_t pair = blk / parts;
+    const int hg = part * width + g;
+    const int b = (int)(pair / Hkv), kvh = (int)(pair % Hkv);
+    out[i] = hg < G ? in[((int64_t)b * Hq + kvh * G + hg) * LR + lr] : (TE)0;
+  }
+}
+
+}  // namespace
+
+extern "C" int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
+                                   const uint16_t* v_norm, const int32_t* lens, float* scores,
+                                   uint32_t* row_range, int range_parts,
+                                   int B, int Hq, int Hkv, int L, int P, int R, int T,
+                                   int64_t Tcap, int64_t score_stride, void* stream) {
+  return score_entry(q_probs, q_dtype, codes, v_norm, lens, scores, row_range, range_parts, B, Hq, Hkv, L, P,
+                     R, T, Tcap, score_stride, stream, 0);
+}
+
+extern "C" int socket_score_packed_grouped(const void* q_table, int q_dtype, const uint32_t* codes,
+                                           const uint16_t* v_norm, const int32_t* lens, float* scores,
+                                           uint32_t* row_range, int range_parts,
+                                           int B, int Hq, int Hkv, int L, int P, int R, int T,
+                                           int64_t Tcap, int64_t score_stride, void* stream) {
+  return score_entry(q_table, q_dtype, codes, v_norm, lens, scores, row_range, range_parts, B, Hq, Hkv, L, P,
+                     R, T, Tcap, score_stride, stream, 1);
+}
+
+extern "C" int socket_group_shape(int Hq, int Hkv, int* parts, int* width) {
+  SOCKET_REQUIRE(parts && width, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(Hq > 0 && Hkv > 0 && Hq % Hkv == 0, SOCKET_ERR_SHAPE);
+  const int G = Hq / Hkv;
+  SOCKET_REQUIRE(G <= 8, SOCKET_ERR_UNSUPPORTED);
+  *width = G == 1 ? 1 : G == 2 ? 2 : 4;
+  *parts = (G + *width - 1) / *width;
+  return SOCKET_OK;
+}
+
+extern "C" int socket_group_q_probs(const void* q_probs, int q_dtype, void* q_table, int B, int Hq, int Hkv,
+                                    int L, int R, void* stream) {
+  SOCKET_REQUIRE(q_probs && q_table, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(q_dtype == SOCKET_F32 || q_dtype == SOCKET_BF16, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(B > 0 && L > 0 && R > 0, SOCKET_ERR_SHAPE);
+  int parts = 0, width = 0;
+  const int st = socket_group_shape(Hq, Hkv, &parts, &width);
+  if (st != SOCKET_OK) return st;
+  const int64_t LR = (int64_t)L * R;
+  const int64_t total = (int64_t)B * Hkv * parts * LR * width;
+  const int blocks = (int)((total + 255) / 256 < 65535 * 16 ? (total + 255) / 256 : 65535 * 16);
+  hipStream_t s = (hipStream_t)stream;
+  if (q_dtype == SOCKET_F32)
+    hipLaunchKernelGGL(group_q_probs_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)q_probs,
+                       (float*)q_table, Hq, Hkv, Hq / Hkv, parts, width, LR, total);
+  else
+    hipLaunchKernelGGL(group_q_probs_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, (const uint16_t*)q_probs,
+                       (uint16_t*)q_table, Hq, Hkv, Hq / Hkv, parts, width, LR, total);
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
 }
 
 extern "C" int socket_soft_hash_collision(const float* q_probs, const int16_t* key_buckets,

@@ -46,7 +46,7 @@ template <class DT>
 __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
     const void* __restrict__ q, int64_t q_sb, int64_t q_sh, const void* __restrict__ planes,
     const void* __restrict__ protos_T, void* __restrict__ out, int out_dtype, int Hq, int Hkv, int G,
-    int D, int L, int K, int R, float tanh_scale, float inv_temperature) {
+    int D, int L, int K, int R, float tanh_scale, float inv_temperature, int parts, int width) {
   __shared__ float qs[kSHMaxG][kSHMaxD];
   __shared__ float ps[kSHMaxK][kSHMaxD + 1];
   __shared__ float ts[kSHMaxG][kSHMaxK];
@@ -140,19 +140,39 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
   for (int r0 = tid * 4; r0 < R; r0 += kSHThreads * 4) {
     logits4(r0, lg);
 #pragma unroll
-    for (int g = 0; g < kSHMaxG; ++g) {
-      if (g < G) {
-        float p[4];
+    for (int g = 0; g < kSHMaxG; ++g)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) p[i] = expf(lg[g][i] - mx[g]) / sm[g];
-        const int64_t o = (((int64_t)b * Hq + kvh * G + g) * L + l) * R + r0;
-        if (out_dtype == SOCKET_F32) {
-          *reinterpret_cast<float4*>((float*)out + o) = make_float4(p[0], p[1], p[2], p[3]);
-        } else {
-          uint2 w;
-          w.x = (uint32_t)f32_to_bf16_bits(p[0]) | ((uint32_t)f32_to_bf16_bits(p[1]) << 16);
-          w.y = (uint32_t)f32_to_bf16_bits(p[2]) | ((uint32_t)f32_to_bf16_bits(p[3]) << 16);
-          *reinterpret_cast<uint2*>((uint16_t*)out + o) = w;
+      for (int i = 0; i < 4; ++i) lg[g][i] = (g < G) ? expf(lg[g][i] - mx[g]) / sm[g] : 0.f;   // now probabilities
+    if (parts == 0) {
+      // reference layout [B,Hq,L,R]
+#pragma unroll
+      for (int g = 0; g < kSHMaxG; ++g) {
+        if (g < G) {
+          const int64_t o = (((int64_t)b * Hq + kvh * G + g) * L + l) * R + r0;
+          if (out_dtype == SOCKET_F32) {
+            *reinterpret_cast<float4*>((float*)out + o) = make_float4(lg[g][0], lg[g][1], lg[g][2], lg[g][3]);
+          } else {
+            uint2 w;
+            w.x = (uint32_t)f32_to_bf16_bits(lg[g][0]) | ((uint32_t)f32_to_bf16_bits(lg[g][1]) << 16);
+            w.y = (uint32_t)f32_to_bf16_bits(lg[g][2]) | ((uint32_t)f32_to_bf16_bits(lg[g][3]) << 16);
+            *reinterpret_cast<uint2*>((uint16_t*)out + o) = w;
+          }
+        }
+      }
+    } else {
+      // grouped layout [B*Hkv*parts, L, R, width]: the scorer's LDS image
+      for (int part = 0; part < parts; ++part) {
+        const int64_t o = ((((int64_t)pair * parts + part) * L + l) * R + r0) * width;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+          for (int g = 0; g < kSHMaxG; ++g) {
+            const int gg = g - part * width;      // position inside this part
+            if (gg >= 0 && gg < width) {
+              if (out_dtype == SOCKET_F32) ((float*)out)[o + i * width + gg] = lg[g][i];
+              else ((uint16_t*)out)[o + i * width + gg] = f32_to_bf16_bits(lg[g][i]);
+            }
+          }
         }
       }
     }
@@ -161,10 +181,11 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
 
 }  // namespace
 
-extern "C" int socket_soft_hash(const void* q, int dtype, int64_t q_stride_b, int64_t q_stride_h,
-                                const void* planes, const void* protos_T, void* out, int out_dtype,
-                                int B, int Hq, int Hkv, int D, int L, int K, int R,
-                                float tanh_scale, float inv_temperature, void* stream) {
+namespace {
+
+int soft_hash_entry(const void* q, int dtype, int64_t q_stride_b, int64_t q_stride_h, const void* planes,
+                    const void* protos_T, void* out, int out_dtype, int B, int Hq, int Hkv, int D, int L, int K,
+                    int R, float tanh_scale, float inv_temperature, void* stream, int grouped) {
   SOCKET_REQUIRE(q && planes && protos_T && out, SOCKET_ERR_NULL);
   SOCKET_REQUIRE(socket_dtype_bytes(dtype) != 0, SOCKET_ERR_UNSUPPORTED);
   SOCKET_REQUIRE(out_dtype == SOCKET_F32 || out_dtype == SOCKET_BF16, SOCKET_ERR_UNSUPPORTED);
@@ -174,16 +195,39 @@ extern "C" int socket_soft_hash(const void* q, int dtype, int64_t q_stride_b, in
   SOCKET_REQUIRE(R >= 4 && R % 4 == 0, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE((int64_t)B * Hkv <= 65535, SOCKET_ERR_SHAPE);
   SOCKET_REQUIRE(socket_aligned16(out), SOCKET_ERR_ALIGN);
+  int parts = 0, width = 0;
+  if (grouped) {
+    const int st = socket_group_shape(Hq, Hkv, &parts, &width);
+    if (st != SOCKET_OK) return st;
+  }
   const dim3 grid(L, B * Hkv);
   hipStream_t s = (hipStream_t)stream;
 #define SOCKET_SH(DT)                                                                               \
   hipLaunchKernelGGL((soft_hash_kernel<DT>), grid, dim3(kSHThreads), 0, s, q, q_stride_b, q_stride_h, \
                      planes, protos_T, out, out_dtype, Hq, Hkv, Hq / Hkv, D, L, K, R, tanh_scale,     \
-                     inv_temperature)
+                     inv_temperature, parts, width)
   if (dtype == SOCKET_F32) SOCKET_SH(DType_f32);
   else if (dtype == SOCKET_BF16) SOCKET_SH(DType_bf16);
   else SOCKET_SH(DType_f16);
 #undef SOCKET_SH
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
+}
+
+}  // namespace
+
+extern "C" int socket_soft_hash(const void* q, int dtype, int64_t q_stride_b, int64_t q_stride_h,
+                                const void* planes, const void* protos_T, void* out, int out_dtype,
+                                int B, int Hq, int Hkv, int D, int L, int K, int R,
+                                float tanh_scale, float inv_temperature, void* stream) {
+  return soft_hash_entry(q, dtype, q_stride_b, q_stride_h, planes, protos_T, out, out_dtype, B, Hq, Hkv, D, L,
+                         K, R, tanh_scale, inv_temperature, stream, 0);
+}
+
+extern "C" int socket_soft_hash_grouped(const void* q, int dtype, int64_t q_stride_b, int64_t q_stride_h,
+                                        const void* planes, const void* protos_T, void* q_table,
+                                        int out_dtype, int B, int Hq, int Hkv, int D, int L, int K, int R,
+                                        float tanh_scale, float inv_temperature, void* stream) {
+  return soft_hash_entry(q, dtype, q_stride_b, q_stride_h, planes, protos_T, q_table, out_dtype, B, Hq, Hkv, D,
+                         L, K, R, tanh_scale, inv_temperature, stream, 1);
 }

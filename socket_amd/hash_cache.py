@@ -110,15 +110,44 @@ def pack_codes_into(codes_i16_bhlt: torch.Tensor, codes: torch.Tensor, P: int, t
             int(t0), T, codes.shape[3], stream_ptr(codes.device)))
 
 
+def group_shape(n_heads: int, n_kv_heads: int) -> Tuple[int, int]:
+    """(parts, width) of the grouped table layout for this head geometry."""
+    import ctypes
+    parts, width = ctypes.c_int(0), ctypes.c_int(0)
+    check("socket_group_shape", lib().socket_group_shape(int(n_heads), int(n_kv_heads), ctypes.byref(parts),
+                                                         ctypes.byref(width)))
+    return parts.value, width.value
+
+
+@torch.no_grad()
+def group_q_probs(q_probs: torch.Tensor, n_kv_heads: int) -> torch.Tensor:
+    """[B,Hq,L,R] (float32 / bfloat16) -> grouped table [B, Hkv*parts, L, R, width]:
+    the query heads of a KV head interleaved per bucket, which is how the scorer
+    keeps the table in LDS."""
+    assert q_probs.is_cuda and q_probs.dim() == 4
+    if q_probs.dtype not in (torch.float32, torch.bfloat16):
+        q_probs = q_probs.float()
+    q_probs = q_probs.contiguous()
+    B, Hq, L, R = q_probs.shape
+    parts, width = group_shape(Hq, n_kv_heads)
+    out = torch.empty((B, n_kv_heads * parts, L, R, width), dtype=q_probs.dtype, device=q_probs.device)
+    check("socket_group_q_probs", lib().socket_group_q_probs(
+        ptr(q_probs), dtype_enum(q_probs.dtype), ptr(out), B, Hq, int(n_kv_heads), L, R,
+        stream_ptr(q_probs.device)))
+    return out
+
+
 @torch.no_grad()
 def soft_hash(queries_bhd: torch.Tensor, planes_lkd: torch.Tensor, protos_T: torch.Tensor,
               temperature: float = 1.0, n_kv_heads: Optional[int] = None,
-              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+              out_dtype: Optional[torch.dtype] = None, grouped: bool = False) -> torch.Tensor:
     """Query soft bucket probabilities [B,Hq,L,R] in one launch:
     softmax_r((tanh(q . planes) / sqrt(D)) @ protos_T / temperature)
     (GPT-FAST/model.py:392-401 with temperature 1; modeling_llama.py:618-638 with
     0.3).  fp32 arithmetic on the stored inputs, one rounding to `out_dtype`
-    (bfloat16 for bfloat16 queries, else float32)."""
+    (bfloat16 for bfloat16 queries, else float32).  `grouped=True` writes the
+    scorer's grouped table layout [B, Hkv*parts, L, R, width] instead (same values;
+    `n_kv_heads` is then required)."""
     assert queries_bhd.is_cuda and queries_bhd.dim() == 3 and queries_bhd.stride(-1) == 1
     B, Hq, D = queries_bhd.shape
     L, K, D2 = planes_lkd.shape
@@ -129,21 +158,28 @@ def soft_hash(queries_bhd: torch.Tensor, planes_lkd: torch.Tensor, protos_T: tor
     protos_T = protos_T.to(dt).contiguous()
     if out_dtype is None:
         out_dtype = torch.bfloat16 if dt == torch.bfloat16 else torch.float32
+    args = lambda out, Hkv: (
+        ptr(queries_bhd), dtype_enum(dt), queries_bhd.stride(0), queries_bhd.stride(1), ptr(planes_lkd),
+        ptr(protos_T), ptr(out), dtype_enum(out_dtype), B, Hq, Hkv, D, L, K, R,
+        1.0 / max(math.sqrt(D), 1e-6), 1.0 / float(temperature), stream_ptr(queries_bhd.device))
+    if grouped:
+        assert n_kv_heads, "the grouped layout is defined by the number of KV heads"
+        parts, width = group_shape(Hq, n_kv_heads)
+        out = torch.empty((B, n_kv_heads * parts, L, R, width), dtype=out_dtype, device=queries_bhd.device)
+        check("socket_soft_hash_grouped", lib().socket_soft_hash_grouped(*args(out, int(n_kv_heads))))
+        return out
     Hkv = n_kv_heads if n_kv_heads else Hq
     if Hq % Hkv != 0 or Hq // Hkv > 8:
         Hkv = Hq
     out = torch.empty((B, Hq, L, R), dtype=out_dtype, device=queries_bhd.device)
-    check("socket_soft_hash", lib().socket_soft_hash(
-        ptr(queries_bhd), dtype_enum(dt), queries_bhd.stride(0), queries_bhd.stride(1), ptr(planes_lkd),
-        ptr(protos_T), ptr(out), dtype_enum(out_dtype), B, Hq, Hkv, D, L, K, R,
-        1.0 / max(math.sqrt(D), 1e-6), 1.0 / float(temperature), stream_ptr(queries_bhd.device)))
+    check("socket_soft_hash", lib().socket_soft_hash(*args(out, Hkv)))
     return out
 
 
 @torch.no_grad()
 def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
                  lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                 with_range: bool = False):
+                 with_range: bool = False, n_heads: Optional[int] = None):
     """Soft-collision scores [B,Hq,T] fp32 (row pitch padded to a multiple of 4)
     from q_probs [B,Hq,L,R] and the packed cache.  q_probs may be float32 or
     bfloat16; a bfloat16 table is read as is (the reference widens it with
@@ -151,12 +187,21 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
     the LDS bytes per gather.  float16 is widened to float32 first.
     with_range=True also returns the per-tile key ranges of every row (int32
     [B,Hq,parts,2]) for `select_list(..., row_range=...)`."""
-    assert q_probs.is_cuda and q_probs.dim() == 4
+    assert q_probs.is_cuda and q_probs.dim() in (4, 5)
     if q_probs.dtype not in (torch.float32, torch.bfloat16):
         q_probs = q_probs.float()
     q_probs = q_probs.contiguous()
-    B, Hq, L, R = q_probs.shape
     _, Hkv, NW, Tcap = codes.shape
+    grouped = q_probs.dim() == 5
+    if grouped:       # [B, Hkv*parts, L, R, width] as written by soft_hash(grouped=True) / group_q_probs
+        assert n_heads is not None, "a grouped table does not carry the number of query heads: pass n_heads"
+        Hq = int(n_heads)
+        B = codes.shape[0]
+        parts, width = group_shape(Hq, Hkv)
+        assert q_probs.shape[0] == B and q_probs.shape[1] == Hkv * parts and q_probs.shape[4] == width
+        L, R = q_probs.shape[2], q_probs.shape[3]
+    else:
+        B, Hq, L, R = q_probs.shape
     assert codes.dtype == torch.int32 and codes.is_contiguous() and codes.shape[0] == B
     assert v_norm.dtype == torch.float16 and v_norm.is_contiguous() and tuple(v_norm.shape) == (B, Hkv, Tcap)
     assert NW == words_per_key(L, P), "codes were packed for a different (L, P)"
@@ -169,9 +214,13 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
         assert lens.dtype == torch.int32 and lens.is_cuda and lens.numel() == B
     rng, parts = None, 0
     if with_range:
-        parts = lib().socket_score_range_parts(B, Hq, Hkv, int(T))
+        if grouped:
+            parts = lib().socket_score_range_parts_grouped(B, Hq, Hkv, int(T), dtype_enum(q_probs.dtype), int(P), R)
+        else:
+            parts = lib().socket_score_range_parts(B, Hq, Hkv, int(T))
         rng = torch.empty((B, Hq, parts, 2), dtype=torch.int32, device=q_probs.device)
-    check("socket_score_packed", lib().socket_score_packed(
+    entry = lib().socket_score_packed_grouped if grouped else lib().socket_score_packed
+    check("socket_score_packed", entry(
         ptr(q_probs), dtype_enum(q_probs.dtype), ptr(codes), ptr(v_norm), ptr(lens), ptr(out),
         ptr(rng), parts, B, Hq, Hkv, L, int(P), R, int(T), Tcap, pitch, stream_ptr(q_probs.device)))
     if with_range:
@@ -191,7 +240,7 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     q [B,Hq,D]; q_probs [B,Hq,L,R]; T = number of cached tokens to consider (an
     upper bound when `lens` gives per-sequence lengths).  Returns out [B,Hq,D].
     """
-    scores, rng = score_packed(q_probs, codes, v_norm, T, P, lens=lens, with_range=True)
+    scores, rng = score_packed(q_probs, codes, v_norm, T, P, lens=lens, with_range=True, n_heads=q.shape[1])
     sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets, row_range=rng)
     out = sparse_attention_fwd(q, k_cache, v_cache, sparse_list, sparse_len)
     if return_details:

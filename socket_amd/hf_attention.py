@@ -255,7 +255,7 @@ def _hash_rows(st: dict, k_new, v_new, t0: int) -> None:
 
 
 def _soft_hash(q_bhd, planes, protos_T, n_kv_heads: int):
-    return hash_cache.soft_hash(q_bhd, planes, protos_T, 0.3, n_kv_heads)
+    return hash_cache.soft_hash(q_bhd, planes, protos_T, 0.3, n_kv_heads, grouped=True)
 
 
 def _sparse_step(q_bhd, q_probs, k, v, st: dict, T_k: int, sink: int, window: int, M: int):

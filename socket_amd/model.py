@@ -197,8 +197,8 @@ def _dense_step(q_bhd: Tensor, cache: KVCache) -> Tensor:
     return dense_decode_fwd(q_bhd, cache.k_cache, cache.v_cache, cache.lens)
 
 
-def _soft_hash(q_bhd: Tensor, planes: Tensor, protos_T: Tensor, n_kv_heads: int) -> Tensor:
-    return hash_cache.soft_hash(q_bhd, planes, protos_T, 1.0, n_kv_heads)
+def _soft_hash(q_bhd: Tensor, planes: Tensor, protos_T: Tensor, n_kv_heads: int, grouped: bool = False) -> Tensor:
+    return hash_cache.soft_hash(q_bhd, planes, protos_T, 1.0, n_kv_heads, grouped=grouped)
 
 
 def _planes_to_words(planes: Tensor) -> Tensor:
@@ -385,8 +385,11 @@ class Attention(nn.Module):
         if sparse:
             T = cache.k_cache.size(2)       # upper bound; the kernels stop at cache.lens
             cfg = self.config
-            out_bhd = _sparse_step(q_bhd, self.soft_hash(q_bhd), cache, T, int(cfg.sink_size),
-                                   int(cfg.window_size), int(self.heavy_const))
+            # on the device the table is written in the scorer's grouped layout (same values)
+            q_probs = (_soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, grouped=True)
+                       if q_bhd.is_cuda else self.soft_hash(q_bhd))
+            out_bhd = _sparse_step(q_bhd, q_probs, cache, T, int(cfg.sink_size), int(cfg.window_size),
+                                   int(self.heavy_const))
         else:
             out_bhd = _dense_step(q_bhd, cache)
         return self.wo(out_bhd.reshape(bsz, 1, self.dim))

@@ -29,11 +29,23 @@ def hash_rows(cache, k_bshd, v_bshd, t0=0, pos_b=None):
         cache.v_norm[b, :, p0:p0 + S] = vn[b]
 
 
+def ungroup(q_table, H, Hkv):
+    """Grouped table [B, Hkv*parts, L, R, width] -> [B,H,L,R]."""
+    if q_table.dim() == 4:
+        return q_table
+    B, _, L, R, width = q_table.shape
+    G = H // Hkv
+    parts = q_table.shape[1] // Hkv
+    t = q_table.view(B, Hkv, parts, L, R, width).permute(0, 1, 2, 5, 3, 4).reshape(B, Hkv, parts * width, L, R)
+    return t[:, :, :G].reshape(B, H, L, R)
+
+
 def sparse_step(q_bhd, q_probs, cache, T, sink, window, M):
     dev, dt = q_bhd.device, q_bhd.dtype
     B, H, D = q_bhd.shape
     Hkv = cache.k_cache.shape[1]
     G = H // Hkv
+    q_probs = ungroup(q_probs, H, Hkv)
     out = torch.empty((B, H, D), dtype=dt)
     for b in range(B):
         n = min(int(cache.lens[b]), T)

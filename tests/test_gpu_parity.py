@@ -533,6 +533,55 @@ def test_soft_hash_matches_oracle(dev, dtype, B, Hq, Hkv, D, L, K, R, temp, cube
         assert torch.equal(have32.argmax(-1)[clear], hard[clear])
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,L,P,T,dtype", [
+    (2, 8, 2, 20, 10, 5000, torch.bfloat16),     # G=4
+    (1, 14, 2, 12, 10, 3000, torch.bfloat16),    # G=7: two parts of width 4
+    (2, 6, 2, 9, 8, 2000, torch.float32),        # G=3 padded to 4
+    (1, 4, 4, 7, 10, 1500, torch.float32),       # G=1
+    (1, 4, 2, 6, 10, 1500, torch.bfloat16),      # G=2
+    (4, 32, 8, 60, 10, 20000, torch.bfloat16),   # large tile
+    (8, 32, 8, 60, 10, 70000, torch.bfloat16),   # a tile for every CU: slices go straight from global memory to LDS
+    (8, 56, 8, 20, 10, 33000, torch.float32),    # the same with fp32 entries and split head groups
+    (16, 16, 16, 7, 8, 9000, torch.bfloat16),    # ... and one head per group, P = 8
+])
+def test_grouped_table_layout_gives_identical_scores(dev, B, Hq, Hkv, L, P, T, dtype):
+    """The grouped table (converter and fused producer) is a relayout only: the
+    scorer returns bit-identical scores from it."""
+    g = torch.Generator().manual_seed(Hq * 100 + L)
+    R, G = 1 << P, Hq // Hkv
+    q_probs = torch.softmax(torch.randn(B, Hq, L, R, generator=g) * 3, -1).to(dtype).to(dev)
+    parts, width = hash_cache.group_shape(Hq, Hkv)
+    assert width == (1 if G == 1 else 2 if G == 2 else 4) and parts == (G + width - 1) // width
+    table = hash_cache.group_q_probs(q_probs, Hkv)
+    assert tuple(table.shape) == (B, Hkv * parts, L, R, width) and table.dtype == dtype
+    # the layout itself
+    want = torch.zeros(B, Hkv, parts * width, L, R, dtype=dtype)
+    want[:, :, :G] = q_probs.cpu().view(B, Hkv, G, L, R)
+    want = want.view(B, Hkv, parts, width, L, R).permute(0, 1, 2, 4, 5, 3).reshape(B, Hkv * parts, L, R, width)
+    assert torch.equal(table.cpu(), want)
+    codes = _rand_codes(g, B, Hkv, L, T, P)
+    Tcap = (T + 7) // 8 * 8
+    vn = torch.zeros(B, Hkv, Tcap, dtype=torch.float16)
+    vn[..., :T] = (torch.rand(B, Hkv, T, generator=g) * 5).to(torch.float16)
+    lens = torch.randint(T // 2, T + 1, (B,), generator=g, dtype=torch.int32).to(dev)
+    packed = _packed_cache(codes, P, Tcap, dev)
+    a, ra = hash_cache.score_packed(q_probs, packed, vn.to(dev), T, P, lens=lens, with_range=True)
+    b, rb = hash_cache.score_packed(table, packed, vn.to(dev), T, P, lens=lens, with_range=True, n_heads=Hq)
+    assert torch.equal(a, b) and torch.equal(ra, rb)
+
+
+def test_soft_hash_grouped_output_is_the_grouped_relayout(dev):
+    g = torch.Generator().manual_seed(77)
+    for Hq, Hkv in ((8, 2), (14, 2), (6, 2), (4, 4)):
+        q = torch.randn(2, Hq, 128, generator=g).to(torch.bfloat16).to(dev)
+        planes = (torch.randn(7, 10, 128, generator=g) * 0.3).to(torch.bfloat16).to(dev)
+        protos = (torch.randn(10, 1024, generator=g) * 3).to(torch.bfloat16).to(dev)
+        for out_dtype in (torch.bfloat16, torch.float32):
+            std = hash_cache.soft_hash(q, planes, protos, 1.0, Hkv, out_dtype=out_dtype)
+            grp = hash_cache.soft_hash(q, planes, protos, 1.0, Hkv, out_dtype=out_dtype, grouped=True)
+            assert torch.equal(grp, hash_cache.group_q_probs(std, Hkv))
+
+
 def test_soft_hash_strided_queries_and_argument_checks(dev):
     g = torch.Generator().manual_seed(9)
     qkv = torch.randn(2, 1, 12, 128, generator=g).to(torch.bfloat16).to(dev)      # queries are heads 0..7 of a wider row
