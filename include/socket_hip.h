@@ -288,6 +288,39 @@ int socket_dense_decode(const void* q, const void* k, const void* v, int dtype,
                         void* workspace, size_t workspace_bytes,
                         int B, int Hq, int Hkv, int D, int T, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Decode-step helpers around the attention hook
+ * ---------------------------------------------------------------------- */
+
+/* Rotary embedding of the new token's q and k and the append of k / v to the
+ * cache, from the fused projection qkv [B, (Hq + 2*Hkv) * D] (row stride
+ * qkv_stride_b): q_out [B,Hq,D] contiguous; rotated k and v are written at
+ * row pos of k_cache / v_cache (element strides b, h, s; unit-stride last dim),
+ * and lens[b] (may be NULL) is raised to pos + 1.  pos: int64 on the device,
+ * one for all sequences (pos_stride 0) or one each (pos_stride 1); a position
+ * outside [0, min(Tcap, n_pos)) writes nothing.  freqs_cis [n_pos, D/2, 2] holds
+ * (cos, sin) in bf16 or f32.  k_new / v_new (may be NULL): [B,Hkv,D] contiguous
+ * copies of the rotated key and the value, for the hashing kernel.  Pairs (2i, 2i+1) are rotated in fp32 with separately
+ * rounded products, then rounded to `dtype`.
+ * Replaces apply_rotary_emb on q and k (GPT-FAST/model.py:443-444, :626-639) and the
+ * K/V writes and length update of KVCache.update (:215-217, :228) for one token. */
+int socket_rope_append(const void* qkv, int dtype, int64_t qkv_stride_b, const void* freqs_cis,
+                       int freqs_dtype, int64_t n_pos, const int64_t* pos, int pos_stride, void* q_out,
+                       void* k_cache, void* v_cache, int64_t cache_stride_b, int64_t cache_stride_h,
+                       int64_t cache_stride_s, int32_t* lens, void* k_new, void* v_new, int B, int Hq, int Hkv,
+                       int D, int64_t Tcap, void* stream);
+
+/* h = x + residual (residual may be NULL: h = x), rounded to `dtype`;
+ * y = round(h * rsqrt(mean(h^2) + eps)) * weight.  x, residual, h_out (may be
+ * NULL), y_out: [rows, dim] contiguous; weight [dim].
+ * Replaces RMSNorm.forward (GPT-FAST/model.py:603-614) and the residual add in front
+ * of it (TransformerBlock, :340-342). */
+int socket_add_rmsnorm(const void* x, const void* residual, const void* weight, void* h_out, void* y_out,
+                       int dtype, int64_t rows, int dim, float eps, void* stream);
+
+/* out = round(silu(a)) * b elementwise over n elements (FeedForward, GPT-FAST/model.py:599-600). */
+int socket_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,205 @@
+// Decode-step helpers around the attention hook: each replaces a chain of small
+// elementwise launches of the reference's decode step by one launch, with the
+// same arithmetic (fp32 inside, the same roundings to the storage type).
+//
+//  * rope_append_kernel: rotary embedding of the new token's q and k, and the
+//    append of k / v to the cache at the token's position, read from the fused
+//    qkv projection (GPT-FAST/model.py:433-444 apply_rotary_emb :626-639, and the
+//    K/V part of KVCache.update :215-217); also raises the cache's device-side
+//    lengths.  The position comes from device memory, nothing is read back.
+//  * add_rmsnorm_kernel: optional residual add + RMSNorm (model.py:603-614 and
+//    the `x + ...` of TransformerBlock :340-342).
+//  * silu_mul_kernel: silu(a) * b of the feed-forward (model.py:599-600).
+#include "socket_common.h"
+
+namespace {
+
+template <class DT>
+__device__ __forceinline__ float ld(const void* p, int64_t i);
+template <>
+__device__ __forceinline__ float ld<DType_f32>(const void* p, int64_t i) { return ((const float*)p)[i]; }
+template <>
+__device__ __forceinline__ float ld<DType_bf16>(const void* p, int64_t i) {
+  return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+template <>
+__device__ __forceinline__ float ld<DType_f16>(const void* p, int64_t i) {
+  return f16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+
+// round to the storage type and back (what a torch op on that dtype leaves behind)
+template <class DT>
+__device__ __forceinline__ float rnd(float x);
+template <>
+__device__ __forceinline__ float rnd<DType_f32>(float x) { return x; }
+template <>
+__device__ __forceinline__ float rnd<DType_bf16>(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+template <>
+__device__ __forceinline__ float rnd<DType_f16>(float x) { return f16_bits_to_f32(f32_to_f16_bits(x)); }
+
+// (x0 + i x1) * (c + i s) with separately rounded products, as the reference's
+// elementwise multiplies, subtraction and addition round: no contraction into
+// fused multiply-adds here.
+__device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s, float& re, float& im) {
+#pragma clang fp contract(off)
+  const float a = x0 * c, b = x1 * s, cc = x1 * c, d = x0 * s;
+  re = a - b;
+  im = cc + d;
+}
+
+// One workgroup per (head of the fused projection, sequence); lane i owns the
+// pair (2i, 2i+1).  Heads [0,Hq) are queries, [Hq,Hq+Hkv) keys, the rest values.
+template <class DT, class FT>
+__global__ void rope_append_kernel(const void* __restrict__ qkv, int64_t qkv_sb, const void* __restrict__ freqs,
+                                   const int64_t* __restrict__ pos, int pos_stride, void* __restrict__ q_out,
+                                   void* __restrict__ k_cache, void* __restrict__ v_cache, int64_t c_sb,
+                                   int64_t c_sh, int64_t c_ss, int32_t* __restrict__ lens,
+                                   void* __restrict__ k_new, void* __restrict__ v_new, int Hq, int Hkv, int D,
+                                   int64_t Tcap, int64_t n_pos) {
+  const int hh = blockIdx.x, b = blockIdx.y, i = threadIdx.x;
+  const int64_t p = pos[(int64_t)b * pos_stride];
+  const bool ok = p >= 0 && p < Tcap && p < n_pos;   // a position outside the cache or the table writes nothing
+  if (hh == 0 && i == 0 && ok && lens) lens[b] = max(lens[b], (int32_t)p + 1);
+  const int64_t src = (int64_t)b * qkv_sb + (int64_t)hh * D + 2 * i;
+  const float x0 = ld<DT>(qkv, src), x1 = ld<DT>(qkv, src + 1);
+  if (hh >= Hq + Hkv) {  // value: plain copy
+    if (v_new) {
+      const int64_t o = ((int64_t)b * Hkv + (hh - Hq - Hkv)) * D + 2 * i;
+      store_elem<DT>(v_new, o, x0);
+      store_elem<DT>(v_new, o + 1, x1);
+    }
+    if (ok) {
+      const int64_t o = b * c_sb + (int64_t)(hh - Hq - Hkv) * c_sh + p * c_ss + 2 * i;
+      store_elem<DT>(v_cache, o, x0);
+      store_elem<DT>(v_cache, o + 1, x1);
+    }
+    return;
+  }
+  float re = x0, im = x1;
+  if (p >= 0 && p < n_pos) {
+    const float c = ld<FT>(freqs, (p * (D / 2) + i) * 2), s = ld<FT>(freqs, (p * (D / 2) + i) * 2 + 1);
+    rotate_pair(x0, x1, c, s, re, im);
+  }
+  if (hh < Hq) {
+    const int64_t o = ((int64_t)b * Hq + hh) * D + 2 * i;
+    store_elem<DT>(q_out, o, re);
+    store_elem<DT>(q_out, o + 1, im);
+  } else {
+    if (k_new) {
+      const int64_t o = ((int64_t)b * Hkv + (hh - Hq)) * D + 2 * i;
+      store_elem<DT>(k_new, o, re);
+      store_elem<DT>(k_new, o + 1, im);
+    }
+    if (ok) {
+      const int64_t o = b * c_sb + (int64_t)(hh - Hq) * c_sh + p * c_ss + 2 * i;
+      store_elem<DT>(k_cache, o, re);
+      store_elem<DT>(k_cache, o + 1, im);
+    }
+  }
+}
+
+constexpr int kNormThreads = 256;
+
+// One workgroup per row.  h = x + r (rounded to the storage type) when r is
+// given, y = round(h * rsqrt(mean(h^2) + eps)) * w, rounded again.
+template <class DT>
+__global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(
+    const void* __restrict__ x, const void* __restrict__ r, const void* __restrict__ w,
+    void* __restrict__ h_out, void* __restrict__ y_out, int dim, float eps) {
+  __shared__ float red[kNormThreads / SOCKET_WAVE];
+  const int64_t row = (int64_t)blockIdx.x * dim;
+  const int tid = threadIdx.x;
+  float ss = 0.f;
+  for (int i = tid; i < dim; i += kNormThreads) {
+    float h = ld<DT>(x, row + i);
+    if (r) h = rnd<DT>(h + ld<DT>(r, row + i));
+    ss += h * h;
+  }
+#pragma unroll
+  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) ss += __shfl_xor(ss, d, SOCKET_WAVE);
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int k = 0; k < kNormThreads / SOCKET_WAVE; ++k) tot += red[k];
+  const float rs = rsqrtf(tot / (float)dim + eps);
+  for (int i = tid; i < dim; i += kNormThreads) {
+    float h = ld<DT>(x, row + i);
+    if (r) h = rnd<DT>(h + ld<DT>(r, row + i));
+    if (h_out) store_elem<DT>(h_out, row + i, h);
+    store_elem<DT>(y_out, row + i, rnd<DT>(h * rs) * ld<DT>(w, i));
+  }
+}
+
+template <class DT>
+__global__ void silu_mul_kernel(const void* __restrict__ a, const void* __restrict__ b, void* __restrict__ out,
+                                int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float x = ld<DT>(a, i);
+  const float s = rnd<DT>(x / (1.f + expf(-x)));
+  store_elem<DT>(out, i, s * ld<DT>(b, i));
+}
+
+}  // namespace
+
+extern "C" int socket_rope_append(const void* qkv, int dtype, int64_t qkv_stride_b, const void* freqs_cis,
+                                  int freqs_dtype, int64_t n_pos, const int64_t* pos, int pos_stride, void* q_out,
+                                  void* k_cache, void* v_cache, int64_t cache_stride_b, int64_t cache_stride_h,
+                                  int64_t cache_stride_s, int32_t* lens, void* k_new, void* v_new, int B, int Hq,
+                                  int Hkv, int D, int64_t Tcap, void* stream) {
+  SOCKET_REQUIRE(qkv && freqs_cis && pos && q_out && k_cache && v_cache, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(socket_dtype_bytes(dtype) != 0, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(freqs_dtype == SOCKET_F32 || freqs_dtype == SOCKET_BF16, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(B > 0 && B <= 65535 && Hq > 0 && Hkv > 0 && Tcap > 0 && n_pos > 0, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(D >= 2 && D % 2 == 0 && D <= 2048, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(pos_stride == 0 || pos_stride == 1, SOCKET_ERR_SHAPE);
+  const dim3 grid(Hq + 2 * Hkv, B), block(D / 2);
+  hipStream_t s = (hipStream_t)stream;
+#define SOCKET_RA(DT, FT)                                                                                  \
+  hipLaunchKernelGGL((rope_append_kernel<DT, FT>), grid, block, 0, s, qkv, qkv_stride_b, freqs_cis, pos,   \
+                     pos_stride, q_out, k_cache, v_cache, cache_stride_b, cache_stride_h, cache_stride_s,  \
+                     lens, k_new, v_new, Hq, Hkv, D, Tcap, n_pos)
+#define SOCKET_RA_F(DT)                                      \
+  do {                                                       \
+    if (freqs_dtype == SOCKET_F32) SOCKET_RA(DT, DType_f32); \
+    else SOCKET_RA(DT, DType_bf16);                          \
+  } while (0)
+  if (dtype == SOCKET_F32) SOCKET_RA_F(DType_f32);
+  else if (dtype == SOCKET_BF16) SOCKET_RA_F(DType_bf16);
+  else SOCKET_RA_F(DType_f16);
+#undef SOCKET_RA_F
+#undef SOCKET_RA
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}
+
+extern "C" int socket_add_rmsnorm(const void* x, const void* residual, const void* weight, void* h_out,
+                                  void* y_out, int dtype, int64_t rows, int dim, float eps, void* stream) {
+  SOCKET_REQUIRE(x && weight && y_out, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(socket_dtype_bytes(dtype) != 0, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(rows > 0 && rows < (1LL << 31) && dim > 0, SOCKET_ERR_SHAPE);
+  hipStream_t s = (hipStream_t)stream;
+#define SOCKET_RN(DT)                                                                                     \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<DT>), dim3((unsigned)rows), dim3(kNormThreads), 0, s, x, residual, \
+                     weight, h_out, y_out, dim, eps)
+  if (dtype == SOCKET_F32) SOCKET_RN(DType_f32);
+  else if (dtype == SOCKET_BF16) SOCKET_RN(DType_bf16);
+  else SOCKET_RN(DType_f16);
+#undef SOCKET_RN
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}
+
+extern "C" int socket_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n, void* stream) {
+  SOCKET_REQUIRE(a && b && out, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(socket_dtype_bytes(dtype) != 0, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(n > 0 && (n + 255) / 256 < (1LL << 31), SOCKET_ERR_SHAPE);
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (dtype == SOCKET_F32) hipLaunchKernelGGL((silu_mul_kernel<DType_f32>), grid, block, 0, s, a, b, out, n);
+  else if (dtype == SOCKET_BF16) hipLaunchKernelGGL((silu_mul_kernel<DType_bf16>), grid, block, 0, s, a, b, out, n);
+  else hipLaunchKernelGGL((silu_mul_kernel<DType_f16>), grid, block, 0, s, a, b, out, n);
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}

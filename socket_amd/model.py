@@ -32,7 +32,7 @@ import torch.nn as nn
 from torch import Tensor
 from torch.nn import functional as F
 
-from . import hash_cache
+from . import decode_ops, hash_cache
 from .socket_kernels import dense_decode_fwd
 
 
@@ -205,6 +205,15 @@ def _planes_to_words(planes: Tensor) -> Tensor:
     return hash_cache.permute_planes(planes)
 
 
+class DecodeStep:
+    """What the layers of one fused single-token step share: the rotary table and
+    the token position as int32 per sequence."""
+    __slots__ = ("freqs_table", "pos_b")
+
+    def __init__(self, freqs_table: Tensor, pos_b: Tensor):
+        self.freqs_table, self.pos_b = freqs_table, pos_b
+
+
 class Transformer(nn.Module):
     def __init__(self, config: ModelArgs) -> None:
         super().__init__()
@@ -216,6 +225,7 @@ class Transformer(nn.Module):
         self.register_buffer("freqs_cis", None, persistent=False)
         self.max_batch_size = -1
         self.max_seq_length = -1
+        self.fused_decode = True     # single-token steps on the device use the fused helper kernels
 
     def setup_caches(self, max_batch_size, max_seq_length):
         if self.max_seq_length >= max_seq_length and self.max_batch_size >= max_batch_size:
@@ -252,8 +262,16 @@ class Transformer(nn.Module):
         input_pos, pos0 = self._positions(idx, input_pos, pos0)
         if idx.dtype != torch.long:
             idx = idx.long()
-        freqs_cis = self.freqs_cis[input_pos]
         x = self.tok_embeddings(idx)
+        if self.fused_decode and x.is_cuda and idx.shape[1] == 1 and pos0 is None and self.layers[0].attention.kv_cache is not None:
+            # one token on the device: rotary + append, norms and the SiLU product are
+            # single launches; the position is handed on as it is (and once as int32
+            # per sequence for the hashing kernel)
+            step = DecodeStep(self.freqs_cis, input_pos.to(torch.int32).expand(idx.shape[0]).contiguous())
+            for layer in self.layers:
+                x = layer._run_fused(x, input_pos, sparse, step)
+            return self.output(decode_ops.add_rmsnorm(x, self.norm.weight, self.norm.eps)[1])
+        freqs_cis = self.freqs_cis[input_pos]
         for layer in self.layers:
             x = layer._run(x, input_pos, freqs_cis, sparse, pos0)
         if last_only:
@@ -287,6 +305,13 @@ class TransformerBlock(nn.Module):
     def _run(self, x, input_pos, freqs_cis, sparse: bool, pos0):
         h = x + self.attention._run(self.attention_norm(x), freqs_cis, input_pos, sparse, pos0)
         return h + self.feed_forward(self.ffn_norm(h))
+
+    def _run_fused(self, x, input_pos, sparse: bool, step: "DecodeStep"):
+        an, fn, ff = self.attention_norm, self.ffn_norm, self.feed_forward
+        _, y = decode_ops.add_rmsnorm(x, an.weight, an.eps)
+        a = self.attention._run_fused(y, input_pos, sparse, step)
+        h, y = decode_ops.add_rmsnorm(x, fn.weight, fn.eps, residual=a)
+        return h + ff.w2(decode_ops.silu_mul(ff.w1(y), ff.w3(y)))
 
     def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Tensor = None) -> Tensor:
         return self._run(x, input_pos, freqs_cis, False, None)
@@ -391,6 +416,27 @@ class Attention(nn.Module):
             out_bhd = _sparse_step(q_bhd, q_probs, cache, T, int(cfg.sink_size), int(cfg.window_size),
                                    int(self.heavy_const))
         else:
+            out_bhd = _dense_step(q_bhd, cache)
+        return self.wo(out_bhd.reshape(bsz, 1, self.dim))
+
+    def _run_fused(self, x: Tensor, input_pos: Tensor, sparse: bool, step: "DecodeStep") -> Tensor:
+        """The decode step of `_run` with rotary embedding, K/V append and length
+        update in one launch (same values)."""
+        bsz = x.shape[0]
+        cache = self.kv_cache
+        qkv = self.wqkv(x)
+        if sparse:
+            q_bhd, k_new, v_new = decode_ops.rope_append(qkv, step.freqs_table, input_pos, cache.k_cache,
+                                                         cache.v_cache, cache.lens, self.n_head,
+                                                         self.n_local_heads, return_new=True)
+            _hash_rows(cache, k_new, v_new, pos_b=step.pos_b)
+            cfg = self.config
+            q_probs = _soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, grouped=True)
+            out_bhd = _sparse_step(q_bhd, q_probs, cache, cache.k_cache.size(2), int(cfg.sink_size),
+                                   int(cfg.window_size), int(self.heavy_const))
+        else:
+            q_bhd = decode_ops.rope_append(qkv, step.freqs_table, input_pos, cache.k_cache, cache.v_cache,
+                                           cache.lens, self.n_head, self.n_local_heads)
             out_bhd = _dense_step(q_bhd, cache)
         return self.wo(out_bhd.reshape(bsz, 1, self.dim))
 

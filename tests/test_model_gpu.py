@@ -149,3 +149,81 @@ def test_load_random_model_and_warmup(dev):
     assert 0.015 < float(model.output.weight.float().std()) < 0.025
     model.setup_caches(1, 512)
     gen.warmup_sparse_decode(model, dev, T=300)
+
+
+# ---------------------------------------------------------------- fused single-token helpers
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_rope_append_equals_the_torch_chain(dev, dtype):
+    g = torch.Generator().manual_seed(11)
+    B, Hq, Hkv, D, Tcap = 3, 4, 2, 128, 64
+    from socket_amd import decode_ops
+    qkv = torch.randn(B, 1, (Hq + 2 * Hkv) * D, generator=g).to(dtype).to(dev)
+    table = M.precompute_freqs_cis(80, D, 10000).to(dev)
+    for pos in (0, 5, 63):
+        kc = torch.zeros(B, Hkv, Tcap, D, dtype=dtype, device=dev)
+        vc = torch.zeros_like(kc)
+        lens = torch.tensor([3, 10, 70], dtype=torch.int32, device=dev)
+        ip = torch.tensor([pos], device=dev)
+        q, kn, vn = decode_ops.rope_append(qkv, table, ip, kc, vc, lens, Hq, Hkv, return_new=True)
+        qs, ks, vs = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        want_q = M.apply_rotary_emb(qs.view(B, 1, Hq, D), table[ip])
+        want_k = M.apply_rotary_emb(ks.view(B, 1, Hkv, D), table[ip])
+        assert torch.equal(q, want_q[:, 0]) and torch.equal(kn, want_k) and torch.equal(vn, vs.view(B, 1, Hkv, D))
+        assert torch.equal(kc[:, :, pos], want_k[:, 0]) and torch.equal(vc[:, :, pos], vs.view(B, Hkv, D))
+        kc[:, :, pos] = 0
+        vc[:, :, pos] = 0
+        assert not kc.any() and not vc.any()                                   # nothing else was touched
+        assert lens.tolist() == [max(3, pos + 1), max(10, pos + 1), 70]
+    # per-sequence positions; one of them outside the cache writes nothing
+    kc = torch.zeros(B, Hkv, Tcap, D, dtype=dtype, device=dev)
+    vc = torch.zeros_like(kc)
+    lens = torch.zeros(B, dtype=torch.int32, device=dev)
+    ip = torch.tensor([2, 64, 9], device=dev)
+    decode_ops.rope_append(qkv, table, ip, kc, vc, lens, Hq, Hkv)
+    assert lens.tolist() == [3, 0, 10] and not kc[1].any() and kc[0, :, 2].any() and kc[2, :, 9].any()
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 1e-2), (torch.float32, 1e-6)])
+def test_add_rmsnorm_and_silu_mul_equal_the_torch_chain(dev, dtype, tol):
+    from socket_amd import decode_ops
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(5, 1, 4096, generator=g).to(dtype).to(dev)
+    r = torch.randn(5, 1, 4096, generator=g).to(dtype).to(dev)
+    norm = M.RMSNorm(4096, 1e-5).to(dev).to(dtype)
+    with torch.no_grad():
+        norm.weight.copy_(torch.randn(4096, generator=g).to(dtype))
+        h, y = decode_ops.add_rmsnorm(x, norm.weight, norm.eps, residual=r)
+        assert torch.equal(h, x + r)
+        want = norm(x + r)
+        # the mean is summed in another order, so the scale can differ in its last bit:
+        # in bf16 that shows in a few outputs, in fp32 in whole rows, by one ulp
+        few = 0.02 if dtype == torch.bfloat16 else 1.0
+        assert float((y.float() - want.float()).abs().max()) <= tol * float(want.float().abs().max())
+        assert float((y != want).float().mean()) <= few
+        h2, y2 = decode_ops.add_rmsnorm(x, norm.weight, norm.eps)
+        assert h2 is x and float((y2 != norm(x)).float().mean()) <= few
+        assert float((y2.float() - norm(x).float()).abs().max()) <= tol * float(want.float().abs().max())
+        a = torch.randn(3, 1, 14336, generator=g).to(dtype).to(dev) * 3
+        b = torch.randn(3, 1, 14336, generator=g).to(dtype).to(dev)
+        got, want = decode_ops.silu_mul(a, b), torch.nn.functional.silu(a) * b
+        assert float((got.float() - want.float()).abs().max()) <= tol * float(want.float().abs().max())
+        assert float((got != want).float().mean()) <= few
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("sparse", [True, False])
+def test_fused_decode_step_equals_the_plain_one(dev, dtype, tol, sparse):
+    model = toy_model(dev, dtype, seed=8)
+    g = torch.Generator().manual_seed(13)
+    ids = torch.randint(0, 331, (2, 60), generator=g).to(dev)
+    model.setup_caches(2, 64)
+    model.fused_decode = True
+    fused = _run_steps(model, ids, 50, sparse=sparse)
+    codes_fused = model.layers[1].attention.kv_cache.codes.clone()
+    _reset(model)
+    model.fused_decode = False
+    plain = _run_steps(model, ids, 50, sparse=sparse)
+    scale = float(plain.abs().max())
+    assert float((fused - plain).abs().max()) <= tol * max(scale, 1.0)
+    if sparse and dtype == torch.float32:
+        assert torch.equal(codes_fused, model.layers[1].attention.kv_cache.codes)
