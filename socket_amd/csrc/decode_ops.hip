@@ -37,6 +37,32 @@ __device__ __forceinline__ float rnd<DType_bf16>(float x) { return bf16_bits_to_
 template <>
 __device__ __forceinline__ float rnd<DType_f16>(float x) { return f16_bits_to_f32(f32_to_f16_bits(x)); }
 
+// One 16-byte vector of elements from floats (rounded to the storage type).
+template <class DT>
+__device__ __forceinline__ void store16(void* base, int64_t idx, const float* v);
+template <>
+__device__ __forceinline__ void store16<DType_f32>(void* base, int64_t idx, const float* v) {
+  *reinterpret_cast<float4*>((float*)base + idx) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <>
+__device__ __forceinline__ void store16<DType_bf16>(void* base, int64_t idx, const float* v) {
+  uint4 w;
+  w.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+  w.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+  w.z = (uint32_t)f32_to_bf16_bits(v[4]) | ((uint32_t)f32_to_bf16_bits(v[5]) << 16);
+  w.w = (uint32_t)f32_to_bf16_bits(v[6]) | ((uint32_t)f32_to_bf16_bits(v[7]) << 16);
+  *reinterpret_cast<uint4*>((uint16_t*)base + idx) = w;
+}
+template <>
+__device__ __forceinline__ void store16<DType_f16>(void* base, int64_t idx, const float* v) {
+  uint4 w;
+  w.x = (uint32_t)f32_to_f16_bits(v[0]) | ((uint32_t)f32_to_f16_bits(v[1]) << 16);
+  w.y = (uint32_t)f32_to_f16_bits(v[2]) | ((uint32_t)f32_to_f16_bits(v[3]) << 16);
+  w.z = (uint32_t)f32_to_f16_bits(v[4]) | ((uint32_t)f32_to_f16_bits(v[5]) << 16);
+  w.w = (uint32_t)f32_to_f16_bits(v[6]) | ((uint32_t)f32_to_f16_bits(v[7]) << 16);
+  *reinterpret_cast<uint4*>((uint16_t*)base + idx) = w;
+}
+
 // (x0 + i x1) * (c + i s) with separately rounded products, as the reference's
 // elementwise multiplies, subtraction and addition round: no contraction into
 // fused multiply-adds here.
@@ -99,21 +125,45 @@ __global__ void rope_append_kernel(const void* __restrict__ qkv, int64_t qkv_sb,
 }
 
 constexpr int kNormThreads = 256;
+constexpr int kNormVecs = 4;  // 16-byte vectors a lane keeps between the two sweeps
 
 // One workgroup per row.  h = x + r (rounded to the storage type) when r is
-// given, y = round(h * rsqrt(mean(h^2) + eps)) * w, rounded again.
+// given, y = round(h * rsqrt(mean(h^2) + eps)) * w, rounded again.  Rows of up to
+// 256 * 4 vectors (8192 bf16 / 4096 fp32 elements, 16-byte aligned) are read once,
+// 16 bytes per lane, and kept in registers for the second sweep.
 template <class DT>
 __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(
     const void* __restrict__ x, const void* __restrict__ r, const void* __restrict__ w,
-    void* __restrict__ h_out, void* __restrict__ y_out, int dim, float eps) {
+    void* __restrict__ h_out, void* __restrict__ y_out, int dim, float eps, int vec_ok) {
+  constexpr int E = DT::kPer16B;
   __shared__ float red[kNormThreads / SOCKET_WAVE];
   const int64_t row = (int64_t)blockIdx.x * dim;
   const int tid = threadIdx.x;
   float ss = 0.f;
-  for (int i = tid; i < dim; i += kNormThreads) {
-    float h = ld<DT>(x, row + i);
-    if (r) h = rnd<DT>(h + ld<DT>(r, row + i));
-    ss += h * h;
+  float hreg[kNormVecs][E];
+  const int nvec = dim / E;
+  if (vec_ok) {
+#pragma unroll
+    for (int k = 0; k < kNormVecs; ++k) {
+      const int v = tid + k * kNormThreads;
+      if (v < nvec) {
+        unpack16<DT>(*reinterpret_cast<const uint4*>((const typename DT::storage*)x + row + (int64_t)v * E), hreg[k]);
+        if (r) {
+          float rr[E];
+          unpack16<DT>(*reinterpret_cast<const uint4*>((const typename DT::storage*)r + row + (int64_t)v * E), rr);
+#pragma unroll
+          for (int e = 0; e < E; ++e) hreg[k][e] = rnd<DT>(hreg[k][e] + rr[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) ss += hreg[k][e] * hreg[k][e];
+      }
+    }
+  } else {
+    for (int i = tid; i < dim; i += kNormThreads) {
+      float h = ld<DT>(x, row + i);
+      if (r) h = rnd<DT>(h + ld<DT>(r, row + i));
+      ss += h * h;
+    }
   }
 #pragma unroll
   for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) ss += __shfl_xor(ss, d, SOCKET_WAVE);
@@ -123,22 +173,50 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(
 #pragma unroll
   for (int k = 0; k < kNormThreads / SOCKET_WAVE; ++k) tot += red[k];
   const float rs = rsqrtf(tot / (float)dim + eps);
-  for (int i = tid; i < dim; i += kNormThreads) {
-    float h = ld<DT>(x, row + i);
-    if (r) h = rnd<DT>(h + ld<DT>(r, row + i));
-    if (h_out) store_elem<DT>(h_out, row + i, h);
-    store_elem<DT>(y_out, row + i, rnd<DT>(h * rs) * ld<DT>(w, i));
+  if (vec_ok) {
+#pragma unroll
+    for (int k = 0; k < kNormVecs; ++k) {
+      const int v = tid + k * kNormThreads;
+      if (v < nvec) {
+        float ww[E];
+        unpack16<DT>(*reinterpret_cast<const uint4*>((const typename DT::storage*)w + (int64_t)v * E), ww);
+        float y[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) y[e] = rnd<DT>(hreg[k][e] * rs) * ww[e];
+        if (h_out) store16<DT>(h_out, row + (int64_t)v * E, hreg[k]);
+        store16<DT>(y_out, row + (int64_t)v * E, y);
+      }
+    }
+  } else {
+    for (int i = tid; i < dim; i += kNormThreads) {
+      float h = ld<DT>(x, row + i);
+      if (r) h = rnd<DT>(h + ld<DT>(r, row + i));
+      if (h_out) store_elem<DT>(h_out, row + i, h);
+      store_elem<DT>(y_out, row + i, rnd<DT>(h * rs) * ld<DT>(w, i));
+    }
   }
 }
 
 template <class DT>
 __global__ void silu_mul_kernel(const void* __restrict__ a, const void* __restrict__ b, void* __restrict__ out,
-                                int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const float x = ld<DT>(a, i);
-  const float s = rnd<DT>(x / (1.f + expf(-x)));
-  store_elem<DT>(out, i, s * ld<DT>(b, i));
+                                int64_t n, int vec_ok) {
+  constexpr int E = DT::kPer16B;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (vec_ok) {
+    const int64_t i = t * E;
+    if (i >= n) return;
+    float x[E], y[E], o[E];
+    unpack16<DT>(*reinterpret_cast<const uint4*>((const typename DT::storage*)a + i), x);
+    unpack16<DT>(*reinterpret_cast<const uint4*>((const typename DT::storage*)b + i), y);
+#pragma unroll
+    for (int e = 0; e < E; ++e) o[e] = rnd<DT>(x[e] / (1.f + expf(-x[e]))) * y[e];
+    store16<DT>(out, i, o);
+    return;
+  }
+  for (int64_t i = t * E; i < min(n, (t + 1) * E); ++i) {
+    const float x = ld<DT>(a, i);
+    store_elem<DT>(out, i, rnd<DT>(x / (1.f + expf(-x))) * ld<DT>(b, i));
+  }
 }
 
 }  // namespace
@@ -180,9 +258,14 @@ extern "C" int socket_add_rmsnorm(const void* x, const void* residual, const voi
   SOCKET_REQUIRE(socket_dtype_bytes(dtype) != 0, SOCKET_ERR_UNSUPPORTED);
   SOCKET_REQUIRE(rows > 0 && rows < (1LL << 31) && dim > 0, SOCKET_ERR_SHAPE);
   hipStream_t s = (hipStream_t)stream;
+  const int per16 = 16 / socket_dtype_bytes(dtype);
+  const int vec_ok = dim % per16 == 0 && dim / per16 <= kNormThreads * kNormVecs && socket_aligned16(x) &&
+                     socket_aligned16(weight) && socket_aligned16(y_out) &&
+                     (residual == nullptr || socket_aligned16(residual)) &&
+                     (h_out == nullptr || socket_aligned16(h_out));
 #define SOCKET_RN(DT)                                                                                     \
   hipLaunchKernelGGL((add_rmsnorm_kernel<DT>), dim3((unsigned)rows), dim3(kNormThreads), 0, s, x, residual, \
-                     weight, h_out, y_out, dim, eps)
+                     weight, h_out, y_out, dim, eps, vec_ok)
   if (dtype == SOCKET_F32) SOCKET_RN(DType_f32);
   else if (dtype == SOCKET_BF16) SOCKET_RN(DType_bf16);
   else SOCKET_RN(DType_f16);
@@ -194,12 +277,15 @@ extern "C" int socket_add_rmsnorm(const void* x, const void* residual, const voi
 extern "C" int socket_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n, void* stream) {
   SOCKET_REQUIRE(a && b && out, SOCKET_ERR_NULL);
   SOCKET_REQUIRE(socket_dtype_bytes(dtype) != 0, SOCKET_ERR_UNSUPPORTED);
-  SOCKET_REQUIRE(n > 0 && (n + 255) / 256 < (1LL << 31), SOCKET_ERR_SHAPE);
+  const int per16 = 16 / socket_dtype_bytes(dtype);
+  const int64_t nthreads = (n + per16 - 1) / per16;
+  SOCKET_REQUIRE(n > 0 && (nthreads + 255) / 256 < (1LL << 31), SOCKET_ERR_SHAPE);
+  const int vec_ok = n % per16 == 0 && socket_aligned16(a) && socket_aligned16(b) && socket_aligned16(out);
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid((unsigned)((n + 255) / 256)), block(256);
-  if (dtype == SOCKET_F32) hipLaunchKernelGGL((silu_mul_kernel<DType_f32>), grid, block, 0, s, a, b, out, n);
-  else if (dtype == SOCKET_BF16) hipLaunchKernelGGL((silu_mul_kernel<DType_bf16>), grid, block, 0, s, a, b, out, n);
-  else hipLaunchKernelGGL((silu_mul_kernel<DType_f16>), grid, block, 0, s, a, b, out, n);
+  const dim3 grid((unsigned)((nthreads + 255) / 256)), block(256);
+  if (dtype == SOCKET_F32) hipLaunchKernelGGL((silu_mul_kernel<DType_f32>), grid, block, 0, s, a, b, out, n, vec_ok);
+  else if (dtype == SOCKET_BF16) hipLaunchKernelGGL((silu_mul_kernel<DType_bf16>), grid, block, 0, s, a, b, out, n, vec_ok);
+  else hipLaunchKernelGGL((silu_mul_kernel<DType_f16>), grid, block, 0, s, a, b, out, n, vec_ok);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }

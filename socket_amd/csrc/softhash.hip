@@ -46,11 +46,13 @@ template <class DT>
 __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
     const void* __restrict__ q, int64_t q_sb, int64_t q_sh, const void* __restrict__ planes,
     const void* __restrict__ protos_T, void* __restrict__ out, int out_dtype, int Hq, int Hkv, int G,
-    int D, int L, int K, int R, float tanh_scale, float inv_temperature, int parts, int width) {
+    int D, int L, int K, int R, float tanh_scale, float inv_temperature, int parts, int width,
+    int protos_in_lds) {
   __shared__ float qs[kSHMaxG][kSHMaxD];
   __shared__ float ps[kSHMaxK][kSHMaxD + 1];
   __shared__ float ts[kSHMaxG][kSHMaxK];
   __shared__ float red[kSHWaves][kSHMaxG];
+  extern __shared__ __attribute__((aligned(16))) float protos_lds[];   // [K][R] when protos_in_lds
   const int l = blockIdx.x, pair = blockIdx.y;
   const int b = pair / Hkv, kvh = pair % Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -60,12 +62,20 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
     qs[g][d] = sh_load<DT>(q, b * q_sb + (int64_t)(kvh * G + g) * q_sh + d);
   }
   for (int i = tid; i < K * D; i += kSHThreads) ps[i / D][i % D] = sh_load<DT>(planes, (int64_t)l * K * D + i);
+  if (protos_in_lds)
+    for (int i = tid; i < K * R; i += kSHThreads) protos_lds[i] = sh_load<DT>(protos_T, i);
   __syncthreads();
-  if (tid < G * K) {
-    const int g = tid / K, k = tid % K;
+  // projections: four lanes per (head, plane) pair, a quarter of the dimension each
+  for (int p0 = 0; p0 < G * K; p0 += kSHThreads / 4) {
+    const int p = p0 + tid / 4, part = tid % 4;
     float s = 0.f;
-    for (int d = 0; d < D; ++d) s += qs[g][d] * ps[k][d];
-    ts[g][k] = tanhf(s) * tanh_scale * inv_temperature;
+    if (p < G * K) {
+      const int g = p / K, k = p % K;
+      for (int d = part; d < D; d += 4) s += qs[g][d] * ps[k][d];
+    }
+    s += __shfl_xor(s, 1, SOCKET_WAVE);
+    s += __shfl_xor(s, 2, SOCKET_WAVE);
+    if (p < G * K && part == 0) ts[p / K][p % K] = tanhf(s) * tanh_scale * inv_temperature;
   }
   __syncthreads();
 
@@ -77,8 +87,16 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
       for (int i = 0; i < 4; ++i) lg[g][i] = 0.f;
     for (int k = 0; k < K; ++k) {
       float pr[4];
+      if (protos_in_lds) {
+        const float4 v = *reinterpret_cast<const float4*>(protos_lds + (size_t)k * R + r0);
+        pr[0] = v.x;
+        pr[1] = v.y;
+        pr[2] = v.z;
+        pr[3] = v.w;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) pr[i] = sh_load<DT>(protos_T, (int64_t)k * R + r0 + i);
+        for (int i = 0; i < 4; ++i) pr[i] = sh_load<DT>(protos_T, (int64_t)k * R + r0 + i);
+      }
 #pragma unroll
       for (int g = 0; g < kSHMaxG; ++g) {
         if (g < G) {
@@ -114,6 +132,9 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
     }
   };
 
+  // With R <= 1024 a lane owns a single run of four buckets: its logits are
+  // computed once and kept; otherwise each sweep recomputes them.
+  const bool keep = R <= kSHThreads * 4;
   float lg[kSHMaxG][4];
   float mx[kSHMaxG], sm[kSHMaxG];
 #pragma unroll
@@ -130,7 +151,7 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
   }
   reduce(mx, true);
   for (int r0 = tid * 4; r0 < R; r0 += kSHThreads * 4) {
-    logits4(r0, lg);
+    if (!keep) logits4(r0, lg);
 #pragma unroll
     for (int g = 0; g < kSHMaxG; ++g)
 #pragma unroll
@@ -138,7 +159,7 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
   }
   reduce(sm, false);
   for (int r0 = tid * 4; r0 < R; r0 += kSHThreads * 4) {
-    logits4(r0, lg);
+    if (!keep) logits4(r0, lg);
 #pragma unroll
     for (int g = 0; g < kSHMaxG; ++g)
 #pragma unroll
@@ -163,15 +184,30 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
       // grouped layout [B*Hkv*parts, L, R, width]: the scorer's LDS image
       for (int part = 0; part < parts; ++part) {
         const int64_t o = ((((int64_t)pair * parts + part) * L + l) * R + r0) * width;
+        float v[16];  // [bucket][head of this part]: 4 * width consecutive elements of the table
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int g = 0; g < kSHMaxG; ++g) {
-            const int gg = g - part * width;      // position inside this part
-            if (gg >= 0 && gg < width) {
-              if (out_dtype == SOCKET_F32) ((float*)out)[o + i * width + gg] = lg[g][i];
-              else ((uint16_t*)out)[o + i * width + gg] = f32_to_bf16_bits(lg[g][i]);
-            }
+            const int gg = g - part * width;
+            if (gg >= 0 && gg < width) v[i * width + gg] = lg[g][i];
+          }
+        if (out_dtype == SOCKET_F32) {
+          for (int c = 0; c < width; ++c)
+            *reinterpret_cast<float4*>((float*)out + o + 4 * c) = make_float4(v[4 * c], v[4 * c + 1], v[4 * c + 2], v[4 * c + 3]);
+        } else {
+          uint32_t w[8];
+#pragma unroll
+          for (int c = 0; c < 8; ++c)
+            w[c] = (uint32_t)f32_to_bf16_bits(v[2 * c]) | ((uint32_t)f32_to_bf16_bits(v[2 * c + 1]) << 16);
+          uint16_t* dst = (uint16_t*)out + o;
+          if (width == 4) {
+            *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+            *reinterpret_cast<uint4*>(dst + 8) = make_uint4(w[4], w[5], w[6], w[7]);
+          } else if (width == 2) {
+            *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+          } else {
+            *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
           }
         }
       }
@@ -202,10 +238,21 @@ int soft_hash_entry(const void* q, int dtype, int64_t q_stride_b, int64_t q_stri
   }
   const dim3 grid(L, B * Hkv);
   hipStream_t s = (hipStream_t)stream;
-#define SOCKET_SH(DT)                                                                               \
-  hipLaunchKernelGGL((soft_hash_kernel<DT>), grid, dim3(kSHThreads), 0, s, q, q_stride_b, q_stride_h, \
-                     planes, protos_T, out, out_dtype, Hq, Hkv, Hq / Hkv, D, L, K, R, tanh_scale,     \
-                     inv_temperature, parts, width)
+  // the prototypes go to LDS as fp32 when they fit in 64 KB (K = 10, R = 1024: 40 KB)
+  const size_t protos_bytes = (size_t)K * R * sizeof(float);
+  const int protos_in_lds = protos_bytes <= 64 * 1024 ? 1 : 0;
+  const size_t dyn_lds = protos_in_lds ? protos_bytes : 0;
+#define SOCKET_SH(DT)                                                                                      \
+  do {                                                                                                     \
+    auto kern = soft_hash_kernel<DT>;                                                                      \
+    if (dyn_lds > 16 * 1024 &&                                                                             \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)dyn_lds) != hipSuccess)                                                   \
+      return SOCKET_ERR_LAUNCH;                                                                            \
+    hipLaunchKernelGGL(kern, grid, dim3(kSHThreads), dyn_lds, s, q, q_stride_b, q_stride_h, planes,        \
+                       protos_T, out, out_dtype, Hq, Hkv, Hq / Hkv, D, L, K, R, tanh_scale, inv_temperature, \
+                       parts, width, protos_in_lds);                                                       \
+  } while (0)
   if (dtype == SOCKET_F32) SOCKET_SH(DType_f32);
   else if (dtype == SOCKET_BF16) SOCKET_SH(DType_bf16);
   else SOCKET_SH(DType_f16);
