@@ -226,14 +226,18 @@ __device__ __forceinline__ void interleave_heads(const uint4 (&x)[GP], uint4 (&o
 // The table slice of the tables held by `chunk_words` packed words sits in LDS;
 // with two LDS buffers the next slice is fetched into registers while the
 // current one is being gathered from, and there is one barrier per slice.
-template <int GP, class TT, int KT4, int THREADS, int PT, bool DMA>
+template <int GP, class TT, int KT4, int THREADS, int PT, int MODE>
 __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     const typename TT::elem* __restrict__ q_probs, const uint32_t* __restrict__ codes,
     const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens,
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
     int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
-    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit,
-    int grouped) {
+    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit) {
+  // MODE: 0 = table in the reference layout [B,Hq,L,R], interleaved while staged;
+  // 1 = grouped table, copied through registers; 2 = grouped table, copied from
+  // global memory straight into LDS
+  constexpr bool grouped = MODE != 0;
+  constexpr bool DMA = MODE == 2;
   typedef typename TT::elem TE;
   const Bf16Select sel = make_bf16_select(bf16_one);
   constexpr int EPV = 16 / (int)sizeof(TE);   // table elements per 16-byte vector
@@ -601,7 +605,7 @@ struct ScoreArgs {
   int grouped;  // table layout: 0 = [B,Hq,L,R], 1 = [B*Hkv*parts, L, R, group width]
 };
 
-template <int GP, class TT, int KT4, int THREADS, int PT, bool DMA>
+template <int GP, class TT, int KT4, int THREADS, int PT, int MODE>
 int launch_score_packed(const ScoreArgs& a) {
   typedef typename TT::elem TE;
   const SocketDeviceLimits& lim = socket_device_limits();
@@ -611,6 +615,7 @@ int launch_score_packed(const ScoreArgs& a) {
   constexpr int EPV = 16 / (int)sizeof(TE);
   const size_t bytes_per_word = (size_t)cpw * a.R * GP * sizeof(TE);
   const size_t slots_per_word = (size_t)cpw * a.R / EPV;
+  constexpr bool DMA = MODE == 2;
   int nbuf = 2, chunk_words = 1;
   if (DMA) {
     // two buffers, as many words per slice as LDS holds (no register staging to fit)
@@ -629,7 +634,7 @@ int launch_score_packed(const ScoreArgs& a) {
   }
   const size_t lds_bytes = bytes_per_word * chunk_words * nbuf;
 
-  auto kern = score_packed_kernel<GP, TT, KT4, THREADS, PT, DMA>;
+  auto kern = score_packed_kernel<GP, TT, KT4, THREADS, PT, MODE>;
   if (lds_bytes > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
@@ -645,16 +650,21 @@ int launch_score_packed(const ScoreArgs& a) {
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
                      a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
                      a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, xcd_remap, 0x3f80u,
-                     a.row_range, hsplit, a.grouped);
+                     a.row_range, hsplit);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }
 
-template <int GP, class TT, int KT4, int THREADS, bool DMA = false>
+template <int GP, class TT, int KT4, int THREADS, int MODE>
 int dispatch_p(const ScoreArgs& a) {
-  if (a.P == 10) return launch_score_packed<GP, TT, KT4, THREADS, 10, DMA>(a);
-  if (a.P == 8) return launch_score_packed<GP, TT, KT4, THREADS, 8, DMA>(a);
-  return launch_score_packed<GP, TT, KT4, THREADS, 0, DMA>(a);
+  if (a.P == 10) return launch_score_packed<GP, TT, KT4, THREADS, 10, MODE>(a);
+  if (a.P == 8) return launch_score_packed<GP, TT, KT4, THREADS, 8, MODE>(a);
+  return launch_score_packed<GP, TT, KT4, THREADS, 0, MODE>(a);
+}
+
+template <int GP, class TT, int KT4, int THREADS>
+int dispatch_layout(const ScoreArgs& a) {
+  return a.grouped ? dispatch_p<GP, TT, KT4, THREADS, 1>(a) : dispatch_p<GP, TT, KT4, THREADS, 0>(a);
 }
 
 constexpr int kDmaKT4 = 2;  // token groups of four per lane in the direct-to-LDS variant
@@ -682,11 +692,11 @@ int tile_tokens(int B, int Hkv, int G, int T, int grouped, size_t table_elem_byt
 template <int GP, class TT>
 int dispatch_tile(const ScoreArgs& a) {
   const int tw = tile_tokens(a.B, a.Hkv, a.Hq / a.Hkv, a.T, a.grouped, sizeof(typename TT::elem), a.P, a.R);
-  if (tw == kDmaTile) return dispatch_p<GP, TT, kDmaKT4, 1024, true>(a);
-  if (tw == 8192) return dispatch_p<GP, TT, 2, 1024>(a);
-  if (tw == 4096) return dispatch_p<GP, TT, 2, 512>(a);
-  if (tw == 2048) return dispatch_p<GP, TT, 1, 512>(a);
-  return dispatch_p<GP, TT, 1, 256>(a);
+  if (tw == kDmaTile) return dispatch_p<GP, TT, kDmaKT4, 1024, 2>(a);
+  if (tw == 8192) return dispatch_layout<GP, TT, 2, 1024>(a);
+  if (tw == 4096) return dispatch_layout<GP, TT, 2, 512>(a);
+  if (tw == 2048) return dispatch_layout<GP, TT, 1, 512>(a);
+  return dispatch_layout<GP, TT, 1, 256>(a);
 }
 
 template <class TT>
