@@ -16,10 +16,11 @@
 //    kCandCap entries.  Because the composites are distinct, ties need no special
 //    case.  The pool is the whole row when that fits; otherwise everything at or
 //    above a threshold estimated from a fixed sample of the row and aimed at
-//    about 2m entries.  For long rows select_local_kernel applies the threshold
-//    beforehand, one 256-lane workgroup per slice of 16384 scores held in
-//    registers (one HBM read of the scores in all), and the row kernel only
-//    gathers the slices' lists.  A pool that comes out shorter than m or longer
+//    about 2m entries.  For long rows select_tau_kernel finds the thresholds (one
+//    workgroup per row, only the sample is read) and select_local_kernel applies
+//    them, one 256-lane workgroup per slice of 16384 scores held in registers
+//    (one HBM read of the scores in all); the row kernel only gathers the slices'
+//    lists.  A pool that comes out shorter than m or longer
 //    than kPoolCap (the sample misjudged the row, or one key value is massively
 //    repeated) is dropped and the row redone from scratch: the result is always
 //    exact, only the time differs.
@@ -515,75 +516,101 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
 // ---------------------------------------------------------------------------
 // slices: everything at or above the row's sampled threshold
 // ---------------------------------------------------------------------------
+constexpr uint32_t kNoThreshold = 0xffffffffu;  // row is not filtered by slices (the row kernel does it all)
+
+// One workgroup per row: the sampled threshold of the row for the slice filter.
 template <bool VEC>
-__global__ __launch_bounds__(kLocThreads) void select_local_kernel(
+__global__ __launch_bounds__(kThreads) void select_tau_kernel(
     const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
     const int32_t* __restrict__ budgets, int Hq, int T, int M, int sink, int window, int write_base,
-    int list_width, int S, int k_cap, u64* __restrict__ loc, int32_t* __restrict__ loc_count) {
+    int list_width, uint32_t* __restrict__ tau_out) {
   __shared__ uint32_t hist[kBins];
   __shared__ SelectShared sh;
-  const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int rowi = blockIdx.x, tid = threadIdx.x;
   int n, m, nbase;
   row_shape(lens, budgets, rowi / Hq, T, M, sink, window, write_base, list_width, n, m, nbase);
-  const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
-  const int64_t slot = (int64_t)rowi * S + s;
   // short rows are pooled whole by the row kernel; it also takes over when no
   // threshold can be relied on
-  if (m == 0 || n <= kPoolCap || end <= begin || !sampling_ok(m)) {
+  if (m == 0 || n <= kPoolCap || !sampling_ok(m)) {
+    if (tid == 0) tau_out[rowi] = kNoThreshold;
+    return;
+  }
+  const uint32_t tau = sample_threshold<kThreads, VEC>(scores + (int64_t)rowi * score_stride, n, m, hist, sh, tid);
+  // (a key of 0xffffffff is a NaN score; a threshold that high is as good as none)
+  if (tid == 0) tau_out[rowi] = tau;
+}
+
+// One workgroup of 256 lanes per slice of 16384 scores, in two halves of 32 keys
+// per lane held in registers between counting and writing.
+template <bool VEC>
+__global__ __launch_bounds__(kLocThreads) void select_local_kernel(
+    const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens, int Hq, int T,
+    int S, int k_cap, const uint32_t* __restrict__ tau_in, u64* __restrict__ loc,
+    int32_t* __restrict__ loc_count) {
+  __shared__ int wsum[kLocWaves];
+  const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int n = lens ? max(0, min(lens[rowi / Hq], T)) : T;
+  const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
+  const int64_t slot = (int64_t)rowi * S + s;
+  const uint32_t tau = tau_in[rowi];
+  if (tau == kNoThreshold || end <= begin) {
     if (tid == 0) loc_count[slot] = 0;
     return;
   }
   const float* row = scores + (int64_t)rowi * score_stride;
-  const uint32_t tau = sample_threshold<kLocThreads, VEC>(row, n, m, hist, sh, tid);
-
-  // the slice's keys, 64 per lane: element e of lane t is index
-  // begin + ((e / 4) * 256 + t) * 4 + e % 4; places past the row's end get key 0
-  // and are excluded by their index
-  uint32_t key[kLocPerLane];
+  u64* my = loc + slot * k_cap;
+  constexpr int kHalf = kLocPerLane / 2;
+  int written = 0;  // entries of the earlier half (uniform)
+  for (int half = 0; half < 2; ++half) {
+    // element e of lane t is index hbase + ((e / 4) * 256 + t) * 4 + e % 4; places past
+    // the row's end get key 0 and are excluded by their index
+    const int hbase = begin + half * (kSliceLen / 2);
+    uint32_t key[kHalf];
 #pragma unroll
-  for (int u = 0; u < kLocPerLane / 4; ++u) {
-    const int i0 = begin + (u * kLocThreads + tid) * 4;
-    float x[4] = {0.f, 0.f, 0.f, 0.f};
-    if (VEC && i0 + 4 <= end) {
-      const float4 v = *reinterpret_cast<const float4*>(row + i0);
-      x[0] = v.x;
-      x[1] = v.y;
-      x[2] = v.z;
-      x[3] = v.w;
-    } else {
+    for (int u = 0; u < kHalf / 4; ++u) {
+      const int i0 = hbase + (u * kLocThreads + tid) * 4;
+      float x[4] = {0.f, 0.f, 0.f, 0.f};
+      if (VEC && i0 + 4 <= end) {
+        const float4 v = *reinterpret_cast<const float4*>(row + i0);
+        x[0] = v.x;
+        x[1] = v.y;
+        x[2] = v.z;
+        x[3] = v.w;
+      } else {
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (i0 + c < end) x[c] = row[i0 + c];
+        for (int c = 0; c < 4; ++c)
+          if (i0 + c < end) x[c] = row[i0 + c];
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) key[u * 4 + c] = score_to_key(x[c]);
+    }
+    auto index_of = [&](int e) { return hbase + ((e >> 2) * kLocThreads + tid) * 4 + (e & 3); };
+    int cnt = 0;
+#pragma unroll
+    for (int e = 0; e < kHalf; ++e) cnt += (key[e] >= tau && index_of(e) < end) ? 1 : 0;
+    const int incl = wave_incl_scan(cnt, lane);
+    __syncthreads();  // the earlier half's readers of wsum are done
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    int at = written + incl - cnt, total = 0;
+#pragma unroll
+    for (int w = 0; w < kLocWaves; ++w) {
+      if (w < wave) at += wsum[w];
+      total += wsum[w];
+    }
+    written += total;
+    if (written > k_cap) {  // more than the slice's share of the pool: the row kernel starts over
+      if (tid == 0) loc_count[slot] = k_cap + 1;
+      return;
     }
 #pragma unroll
-    for (int c = 0; c < 4; ++c) key[u * 4 + c] = score_to_key(x[c]);
+    for (int e = 0; e < kHalf; ++e) {
+      const int i = index_of(e);
+      if (key[e] >= tau && i < end) my[at++] = composite(key[e], i);
+    }
   }
-  auto index_of = [&](int e) { return begin + ((e >> 2) * kLocThreads + tid) * 4 + (e & 3); };
-
-  int cnt = 0;
-#pragma unroll
-  for (int e = 0; e < kLocPerLane; ++e) cnt += (key[e] >= tau && index_of(e) < end) ? 1 : 0;
-  const int incl = wave_incl_scan(cnt, lane);
-  if (lane == 63) sh.wsum[wave] = incl;
-  __syncthreads();
-  int at = incl - cnt, total = 0;
-#pragma unroll
-  for (int w = 0; w < kLocWaves; ++w) {
-    if (w < wave) at += sh.wsum[w];
-    total += sh.wsum[w];
-  }
-  if (total > k_cap) {  // more than the slice's share of the pool: the row kernel starts over
-    if (tid == 0) loc_count[slot] = k_cap + 1;
-    return;
-  }
-  u64* my = loc + slot * k_cap;
-#pragma unroll
-  for (int e = 0; e < kLocPerLane; ++e) {
-    const int i = index_of(e);
-    if (key[e] >= tau && i < end) my[at++] = composite(key[e], i);
-  }
-  if (tid == 0) loc_count[slot] = total;
+  if (tid == 0) loc_count[slot] = written;
 }
 
 // ---------------------------------------------------------------------------
@@ -879,7 +906,7 @@ int slice_cap(int T, int m_max, int* S_out) {
 }
 
 struct SplitLayout {
-  size_t off_loc, off_count, total;
+  size_t off_loc, off_count, off_tau, total;
 };
 
 SplitLayout split_layout(int rows, int S, int k_cap) {
@@ -892,6 +919,7 @@ SplitLayout split_layout(int rows, int S, int k_cap) {
   };
   l.off_loc = take((size_t)rows * S * k_cap * sizeof(u64));
   l.off_count = take((size_t)rows * S * sizeof(int32_t));
+  l.off_tau = take((size_t)rows * sizeof(uint32_t));
   l.total = o;
   return l;
 }
@@ -952,15 +980,19 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
     char* ws = (char*)workspace;
     u64* loc_w = (u64*)(ws + l.off_loc);
     int32_t* count_w = (int32_t*)(ws + l.off_count);
+    uint32_t* tau_w = (uint32_t*)(ws + l.off_tau);
     const dim3 sgrid(S, rows);
-    if (vec)
-      hipLaunchKernelGGL(select_local_kernel<true>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride,
-                         lens, budgets, Hq, T, M, sink, window, write_base, list_width, S, k_cap, loc_w,
-                         count_w);
-    else
-      hipLaunchKernelGGL(select_local_kernel<false>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride,
-                         lens, budgets, Hq, T, M, sink, window, write_base, list_width, S, k_cap, loc_w,
-                         count_w);
+    if (vec) {
+      hipLaunchKernelGGL(select_tau_kernel<true>, dim3(rows), dim3(kThreads), 0, s, scores, score_stride, lens,
+                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w);
+      hipLaunchKernelGGL(select_local_kernel<true>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride, lens,
+                         Hq, T, S, k_cap, tau_w, loc_w, count_w);
+    } else {
+      hipLaunchKernelGGL(select_tau_kernel<false>, dim3(rows), dim3(kThreads), 0, s, scores, score_stride, lens,
+                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w);
+      hipLaunchKernelGGL(select_local_kernel<false>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride, lens,
+                         Hq, T, S, k_cap, tau_w, loc_w, count_w);
+    }
     SOCKET_LAUNCH_CHECK();
     loc = loc_w;
     loc_count = count_w;
