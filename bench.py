@@ -165,7 +165,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--only", default=None,
-                    choices=["score", "score_f32", "score_grouped", "select", "attend", "hash", "dense", "copy"])
+                    choices=["score", "score_f32", "score_grouped", "select", "attend", "hash", "prefill_hash", "dense", "copy"])
     ap.add_argument("--reference-table-layout", action="store_true",
                     help="feed the scorer q_probs as [B,Hq,L,R] instead of the grouped layout the soft-hash kernel writes")
     ap.add_argument("--no-cpu", action="store_true")
@@ -204,6 +204,12 @@ def main():
     def prefill_hash():
         hash_cache.hash_keys_into(inp.k, inp.v, planes_words, codes, v_norm, w.L, w.P, t0=0, layout="bhsd")
 
+    if args.only == "prefill_hash":
+        us = time_launches(prefill_hash, max(args.steps, 1), warmup=args.warmup)
+        rows = B * Hkv * T
+        print(json.dumps({"only": "prefill_hash", "workload": w.name, "us": round(us, 1), "rows": rows,
+                          "mfma_tflops": round(2.0 * rows * D * NW * 32 / us / 1e6, 1)}))
+        return
     prefill_us = time_launches(prefill_hash, 3, warmup=1)
     rows = B * Hkv * T
     prefill_flops = 2.0 * rows * D * NW * 32          # columns actually contracted (incl. pad bits)

@@ -2,20 +2,24 @@
 //
 // Replaces hard_hash_keys + pack_bits (GPT-FAST/model.py:403-413): the einsum
 // that materialises [B,S,Hkv,L,P] projections, the bool compare and the int16
-// weighted sum become one MFMA contraction whose epilogue is a wave ballot.
+// weighted sum become one MFMA contraction with a sign-bit epilogue.
 //
 // The hyperplanes are pre-ordered (socket_permute_planes) so that column
 // w*32 + p of the contraction is the plane whose sign is bit p of packed word w.
-// With keys as the M operand and planes as the N operand of
-// v_mfma_f32_32x32x16_bf16, accumulator register r of lane x holds
-//   key row 8*(r/4) + 4*(x/32) + r%4,  column x%32,
-// so ballot(acc[r] >= 0) is, in its low and high halves, the complete packed
-// word w of two keys: no bit shuffling, no LDS round trip.  The words of 32
-// consecutive keys are gathered into lanes 0..31 and stored as one 128-byte
-// run of the table-major code cache.
+// With planes as the M operand and keys as the N operand of
+// v_mfma_f32_16x16x32_bf16, accumulator register r of lane x holds
+//   plane row 4*(x/16) + r of a 16-plane block,  key x%16,
+// so each lane has sign bits of ITS key in its own registers: they are shifted
+// into a byte one v_alignbit per register, the four lane quarters are OR-ed into
+// the 32-bit word, and lane x ends up with the packed word of key x of the
+// 64-key tile, stored as one 256-byte run of the table-major code cache.  No
+// compares, no ballots, no LDS round trip.  The 16x16x32 shape is chosen for the
+// key loads: its N operand wants 64 consecutive bytes of a row from four lanes,
+// so a load instruction touches 16 rows x one 64-byte sector (the 32x32x16 shape
+// touches 64 lines for 16 bytes each, eight times over).
 //
-// A wave owns 64 consecutive keys of one (b, kv head) (two 32-row M tiles) at a
-// time and keeps their A fragments in registers for the whole column sweep; the
+// A wave owns 64 consecutive keys of one (b, kv head) (four 16-key blocks) at a
+// time and keeps their fragments in registers for the whole column sweep; the
 // planes sit in LDS (all NW words when NW*8 KB fits, which L=60 x P=10 exactly
 // does at 160 KB) and workgroups are persistent, so the planes are fetched once
 // per CU, not once per tile.
@@ -24,13 +28,14 @@
 namespace {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
-typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 constexpr int kHashThreads = 512;
 constexpr int kHashWaves = kHashThreads / SOCKET_WAVE;
 constexpr int kKeysPerWave = 64;
 constexpr int kD = 128;
-constexpr int kKSteps = kD / 16;  // MFMA k-steps
+constexpr int kKSteps = kD / 32;      // MFMA k-steps (16x16x32)
+constexpr int kKeyBlocks = kKeysPerWave / 16;
 
 union Frag {
   uint4 u;
@@ -67,6 +72,12 @@ __device__ __forceinline__ uint4 load_frag8<DType_f16>(const uint16_t* p) {
   r.w = (uint32_t)f32_to_bf16_bits(f[6]) | ((uint32_t)f32_to_bf16_bits(f[7]) << 16);
   return r;
 }
+
+// LDS placement of the planes: row `col` is 16 groups of 16 bytes, group g stored
+// at slot g ^ plane_swizzle(col).  A fragment read has sixteen lanes on sixteen
+// columns {4..7} + 8j (or {0..3} + 8j) at one group; the swizzle sends those to
+// sixteen different slots, i.e. all 64 banks once.
+__device__ __forceinline__ int plane_swizzle(int col) { return (col & 3) | (((col >> 3) & 3) << 2); }
 
 // Sum of squares of 8 consecutive elements starting at p (fp32).
 template <class DT>
@@ -133,87 +144,168 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
         for (int u = 0; u < U; ++u) {
           const int i = i0 + u * kHashThreads;
           const int col = i >> 4, grp = i & 15;
-          plds[col * 16 + (grp ^ (col & 15))] = x[u];
+          plds[col * 16 + (grp ^ plane_swizzle(col))] = x[u];
         }
       }
       for (; i0 < total; i0 += kHashThreads) {
         const int col = i0 >> 4, grp = i0 & 15;
-        plds[col * 16 + (grp ^ (col & 15))] = src[i0];
+        plds[col * 16 + (grp ^ plane_swizzle(col))] = src[i0];
       }
     }
     __syncthreads();
+
+    // Key fragments (the N operand of v_mfma_f32_16x16x32_bf16): for key block nb
+    // and k-step ks, lane x holds key nb*16 + x%16, elements 32*ks + 8*(x/16) .. +7,
+    // so the four lanes x, x+16, x+32, x+48 read 64 consecutive bytes of one row:
+    // a load instruction touches 16 rows x one 64-byte sector each.
+    auto load_rows = [&](const void* base_, int64_t sb, int64_t sh, int64_t ss, int tile,
+                         Frag (&dst)[kKeyBlocks][kKSteps]) {
+      const int pair = tile / tiles_per_row;
+      const int s0 = (tile % tiles_per_row) * kKeysPerWave;
+      const ST* base = (const ST*)base_ + (pair / Hkv) * sb + (pair % Hkv) * sh;
+#pragma unroll
+      for (int nb = 0; nb < kKeyBlocks; ++nb) {
+        const int srow = s0 + nb * 16 + (lane & 15);
+        const bool ok = srow < S;
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks) {
+          dst[nb][ks].u = ok ? load_frag8<DT>(base + (int64_t)srow * ss + ks * 32 + (lane >> 4) * 8)
+                             : make_uint4(0, 0, 0, 0);
+        }
+      }
+    };
+    // bf16 values: their norms come from the matrix core too (see below), from
+    // fragments requested together with the keys'
+    constexpr bool kNormByMfma = DT::kEnum == SOCKET_BF16;
+    const bool want_norm = v_ != nullptr && w0 == 0;  // only the workgroups that own word 0
+    Frag kfrag[kKeyBlocks][kKSteps];
 
     for (int tile = first_tile; tile < n_tiles; tile += tile_stride) {
       const int pair = tile / tiles_per_row;
       const int s0 = (tile % tiles_per_row) * kKeysPerWave;
       const int b = pair / Hkv, h = pair % Hkv;
       const int pos0 = pos_b ? pos_b[b] : t0;
+      load_rows(k_, k_sb, k_sh, k_ss, tile, kfrag);
+      Frag vfrag[kKeyBlocks][kKSteps];
+      if (kNormByMfma && want_norm) load_rows(v_, v_sb, v_sh, v_ss, tile, vfrag);
 
-      // A fragments: lane x holds row x%32, elements 64*(x/32) + 8*kk .. +7, so a
-      // lane reads one contiguous half row over the 8 k-steps.  (The contraction
-      // only needs A and B to agree on which k each slot holds.)
-      Frag afrag[2][kKSteps];
-      const ST* kbase = (const ST*)k_ + b * k_sb + h * k_sh;
+      const int prow = lane & 15, quarter = lane >> 4;
+      // fused value norm, bf16 values (once per tile; done first so that the value
+      // fragments are not live across the contraction)
+      if (kNormByMfma) {
+        // ||v||^2 is the diagonal of V V^T: the value fragments against themselves.
+        // Element (i, i) of a 16 x 16 block sits in register i % 4 of lane
+        // 16 * (i / 4) + i, so sixteen lanes of the wave hold the sixteen norms and
+        // store them; no cross-lane reduction.  (bf16 products are exact in fp32.)
+        if (want_norm) {
+          uint16_t* vn = v_norm + (int64_t)pair * Tcap + pos0;
+          const int r = prow - 4 * quarter;
 #pragma unroll
-      for (int mt = 0; mt < 2; ++mt) {
-        const int srow = s0 + mt * 32 + (lane & 31);
-        const bool ok = srow < S;
+          for (int nb = 0; nb < kKeyBlocks; ++nb) {
+            f32x4 g = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kk = 0; kk < kKSteps; ++kk) {
-          afrag[mt][kk].u = ok ? load_frag8<DT>(kbase + (int64_t)srow * k_ss + (lane >> 5) * 64 + kk * 8)
-                               : make_uint4(0, 0, 0, 0);
+            for (int ks = 0; ks < kKSteps; ++ks)
+              g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfrag[nb][ks].v, vfrag[nb][ks].v, g, 0, 0, 0);
+            const float d = r == 0 ? g[0] : r == 1 ? g[1] : r == 2 ? g[2] : g[3];
+            const int srow = s0 + nb * 16 + prow;
+            if (r >= 0 && r < 4 && srow < S) vn[srow] = f32_to_f16_bits(sqrtf(d));
+          }
         }
       }
-      const bool second = s0 + 32 < S;  // the tile's second 32 rows hold keys at all
 
       uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
-      for (int ww = 0; ww < nw; ++ww) {
-        f32x16 acc0 = {0}, acc1 = {0};
-        const int col = ww * 32 + (lane & 31);
+      // Planes are the M operand: accumulator register r of lane x is plane row
+      // 4*(x/16) + r of its 16-plane block against key x%16.  A lane shifts the sign
+      // bits of its eight accumulators (two plane blocks x four registers) into a
+      // byte, one v_alignbit each; byte q of the word comes from lane quarter q.
+      // Block mb, register r, quarter q therefore lands at bit 8q + 7 - 4mb - r, and
+      // the lane fetches for plane row i of block mb the plane column that belongs
+      // at that bit, so the word comes out in the packed order.
+      const int pbit0 = 8 * (prow >> 2) + 7 - (prow & 3);  // block 0; block 1 is 4 lower
+      // Byte q of a key's word is made in lane quarter q, and a lane makes one byte
+      // for each of the four key blocks: a 4 x 4 byte transpose between the quarters,
+      // done on whole words in two exchanges (lanes x ^ 16, then x ^ 32) with a
+      // byte-select each.  Afterwards lane x holds the word of key s0 + x.
+      const uint32_t sel1 = (quarter & 1) ? 0x03070105u : 0x06020400u;
+      const uint32_t sel2 = (quarter & 2) ? 0x03020706u : 0x05040100u;
+      // plane fragments of one packed word: [k-step][plane block], straight from LDS
+      auto load_planes = [&](int ww, Frag (&pf)[kKSteps][2]) {
 #pragma unroll
-        for (int kk = 0; kk < kKSteps; ++kk) {
-          Frag bf;
-          const int grp = (lane >> 5) * 8 + kk;
-          bf.u = plds[col * 16 + (grp ^ (col & 15))];
-          acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[0][kk].v, bf.v, acc0, 0, 0, 0);
-          if (second) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afrag[1][kk].v, bf.v, acc1, 0, 0, 0);
+        for (int ks = 0; ks < kKSteps; ++ks) {
+          const int grp = ks * 4 + quarter;
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb) {
+            const int col = ww * 32 + pbit0 - 4 * mb;
+            pf[ks][mb].u = plds[col * 16 + (grp ^ plane_swizzle(col))];
+          }
         }
+      };
+      auto do_word = [&](int ww, const Frag (&pf)[kKSteps][2]) {
+        f32x4 acc[2][kKeyBlocks];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int nb = 0; nb < kKeyBlocks; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks)
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < kKeyBlocks; ++nb)  // (blocks past the last key hold zeros: no branch here)
+              acc[mb][nb] =
+                  __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[ks][mb].v, kfrag[nb][ks].v, acc[mb][nb], 0, 0, 0);
         const int w = w0 + ww;
         const int nbits = min(cpw, L - w * cpw) * P;
         const uint32_t valid = nbits >= 32 ? 0xffffffffu : ((1u << nbits) - 1u);
-        uint32_t word0 = 0, word1 = 0;  // lane x < 32: packed word of key row x in M tile 0 / 1
+        // sign bits (set = negative projection; an accumulator that starts at +0 never
+        // becomes -0, so "sign clear" is exactly "projection >= 0"); byte nb of `neg`
+        // is this quarter's byte for key block nb
+        uint32_t neg = 0;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row_lo = 8 * (r / 4) + (r % 4);  // lanes 0..31 of the ballot
-          const unsigned long long b0 = __ballot(acc0[r] >= 0.f);
-          const unsigned long long b1 = __ballot(acc1[r] >= 0.f);
-          if (lane == row_lo) {
-            word0 = (uint32_t)b0;
-            word1 = (uint32_t)b1;
-          } else if (lane == row_lo + 4) {
-            word0 = (uint32_t)(b0 >> 32);
-            word1 = (uint32_t)(b1 >> 32);
-          }
-        }
-        if (lane < 32) {
-          uint32_t* dst = codes_pair + (int64_t)w * Tcap + pos0 + s0;
-          if (s0 + lane < S) dst[lane] = word0 & valid;
-          if (s0 + 32 + lane < S) dst[32 + lane] = word1 & valid;
+        for (int nb = kKeyBlocks - 1; nb >= 0; --nb)
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) neg = __builtin_amdgcn_alignbit(neg, __float_as_uint(acc[mb][nb][r]), 31);
+        const uint32_t t = (uint32_t)__shfl_xor((int)neg, 16, SOCKET_WAVE);
+        const uint32_t x = __builtin_amdgcn_perm(t, neg, sel1);   // two blocks x this pair of quarters
+        const uint32_t u = (uint32_t)__shfl_xor((int)x, 32, SOCKET_WAVE);
+        const uint32_t word = __builtin_amdgcn_perm(u, x, sel2);  // block `quarter` x all four quarters
+        if (s0 + lane < S) codes_pair[(int64_t)w * Tcap + pos0 + s0 + lane] = ~word & valid;
+      };
+      // two fragment sets: the next word's LDS reads are in flight during the
+      // current word's contraction
+      Frag pfa[kKSteps][2], pfb[kKSteps][2];
+      load_planes(0, pfa);
+      for (int ww = 0; ww < nw; ww += 2) {
+        if (ww + 1 < nw) load_planes(ww + 1, pfb);
+        do_word(ww, pfa);
+        if (ww + 1 < nw) {
+          if (ww + 2 < nw) load_planes(ww + 2, pfa);
+          do_word(ww + 1, pfb);
         }
       }
 
-      // fused value norm: 16 lanes per row, 4 rows per pass (once per tile)
-      if (v_ != nullptr && w0 == 0) {  // only the workgroups that own word 0
+      // fused value norm for the other element types (once per tile)
+      if (!kNormByMfma && want_norm) {
+        // they keep their precision: 16 lanes per row, 4 rows per pass
         const ST* vbase = (const ST*)v_ + b * v_sb + h * v_sh;
         uint16_t* vn = v_norm + (int64_t)pair * Tcap + pos0;
         const int sub = lane >> 4, part = lane & 15;
-        const int rows_here = min(kKeysPerWave, S - s0);
-        for (int r0 = 0; r0 < rows_here; r0 += 4) {
-          const int srow = s0 + r0 + sub;
-          float ss = (srow < S) ? sumsq8<DT>(vbase + (int64_t)srow * v_ss + part * 8) : 0.f;
+        // all sixteen row groups' loads are issued before the first is reduced
+        float ss[kKeysPerWave / 4];
 #pragma unroll
-          for (int x = 1; x < 16; x <<= 1) ss += __shfl_xor(ss, x, SOCKET_WAVE);
-          if (part == 0 && srow < S) vn[srow] = f32_to_f16_bits(sqrtf(ss));
+        for (int g = 0; g < kKeysPerWave / 4; ++g) {
+          const int srow = s0 + g * 4 + sub;
+          ss[g] = (srow < S) ? sumsq8<DT>(vbase + (int64_t)srow * v_ss + part * 8) : 0.f;
+        }
+#pragma unroll
+        for (int g = 0; g < kKeysPerWave / 4; ++g) {
+          const int srow = s0 + g * 4 + sub;
+          float t = ss[g];
+#pragma unroll
+          for (int x = 1; x < 16; x <<= 1) t += __shfl_xor(t, x, SOCKET_WAVE);
+          if (part == 0 && srow < S) vn[srow] = f32_to_f16_bits(sqrtf(t));
         }
       }
     }
