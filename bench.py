@@ -247,7 +247,10 @@ def main():
     # ... and in the layout the fused soft-hash kernel writes it in (heads of a KV head
     # interleaved per bucket: the scorer's LDS image); same values
     q_table_grouped = hash_cache.group_q_probs(q_table, Hkv)
-    use_grouped = not args.reference_table_layout
+    # the step uses the layout the library asks its producers for at this shape
+    use_grouped = (not args.reference_table_layout and
+                   hash_cache._prefers_grouped(B, Hq, Hkv, T, 1 if q_table.dtype == torch.bfloat16 else 0,
+                                               w.L, w.P, q_table.shape[-1]))
 
     def k_score_grouped():
         return hash_cache.score_packed(q_table_grouped, codes, v_norm, T, w.P, lens=lens, out=scores_buf,

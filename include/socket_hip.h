@@ -122,10 +122,16 @@ int socket_pack_codes(const int16_t* in, int64_t in_stride_b, int64_t in_stride_
  * row_range (optional, may be NULL): uint32 [B*Hq, range_parts, 2]; for every row
  * and token tile the minimum and maximum order-preserving key of the tile's
  * scores at t < len(b) (0xffffffff / 0 for a tile without such a token).
- * range_parts must equal socket_score_range_parts(B, Hq, Hkv, T).  Passing the
- * array on to socket_select_list saves that kernel a pass over the scores for the
- * rows it has to select without its sampled threshold. */
-int socket_score_range_parts(int B, int Hq, int Hkv, int T);
+ * range_parts must equal socket_score_range_parts(...) of the same call (the
+ * tile size follows from the shape; 0 = invalid shape).  Passing the array on to
+ * socket_select_list saves that kernel a pass over the scores for the rows it has
+ * to select without its sampled threshold.
+ *
+ * With few (b, kv head) pairs and a context too short to give every CU a tile,
+ * and a table of one head (L*R elements) that fits LDS, a workgroup serves one
+ * query head with its whole table resident instead of a head group with table
+ * slices; results are the same. */
+int socket_score_range_parts(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);
 int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
                         const uint16_t* v_norm, const int32_t* lens, float* scores,
                         uint32_t* row_range, int range_parts,
@@ -142,9 +148,15 @@ int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
  * socket_group_q_probs converts a [B,Hq,L,R] table; socket_soft_hash_grouped
  * produces the layout directly.  socket_score_packed_grouped is socket_score_packed
  * on such a table: same arguments, same results, except that its row_range has
- * socket_score_range_parts_grouped(...) parts (its tiles can be of another size). */
+ * socket_score_range_parts_grouped(...) parts (its tiles can be of another size),
+ * and bf16 scores may differ in the last place (within the bound above).
+ * socket_score_prefers_grouped: which layout a producer should write for this
+ * shape (T = the context length the scorer will be called with): 1 = grouped,
+ * 0 = [B,Hq,L,R] (the shapes the scorer serves one head per workgroup, see
+ * socket_score_packed), -1 = invalid shape.  Either layout is always accepted. */
 int socket_group_shape(int Hq, int Hkv, int* parts, int* width);
-int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int P, int R);
+int socket_score_prefers_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);
+int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);
 int socket_group_q_probs(const void* q_probs, int q_dtype, void* q_table, int B, int Hq, int Hkv,
                          int L, int R, void* stream);
 int socket_score_packed_grouped(const void* q_table, int q_dtype, const uint32_t* codes,

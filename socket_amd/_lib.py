@@ -42,12 +42,13 @@ SIGNATURES = {
                               _I, _I, _I, _I, _I, _I, _L, _P]),
     "socket_unpack_codes": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _P]),
     "socket_pack_codes": (_I, [_P, _L, _L, _L, _L, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
-    "socket_score_range_parts": (_I, [_I, _I, _I, _I]),
+    "socket_score_range_parts": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "socket_score_packed": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
     "socket_soft_hash_collision": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "socket_soft_hash_score_f16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "socket_group_shape": (_I, [_I, _I, POINTER(c_int), POINTER(c_int)]),
-    "socket_score_range_parts_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I]),
+    "socket_score_prefers_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
+    "socket_score_range_parts_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "socket_group_q_probs": (_I, [_P, _I, _P, _I, _I, _I, _I, _I, _P]),
     "socket_score_packed_grouped": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
     "socket_soft_hash_grouped": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),

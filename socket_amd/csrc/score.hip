@@ -254,15 +254,19 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   constexpr int TW = CT * 4 * KT4;
 
   // Workgroup -> (pair, tile).  Workgroups are dealt to the 8 XCDs round-robin
-  // by linear id; with the remap all tiles of one (b, kv head) land on one XCD,
-  // so its L2 serves that pair's table slices to every tile.
+  // by linear id; with the remap all tiles of one (b, kv head), and all the
+  // workgroups that share its query heads out between them, land on one XCD: its
+  // L2 serves that pair's table slices to every tile, and the pair's code stream
+  // comes from HBM once however many workgroups read it.
   int pair, tile;
   {
     const int n = blockIdx.x;
     if (xcd_remap) {
       const int xcd = n & 7, slot = n >> 3;
-      pair = (slot / n_tiles) * 8 + xcd;
-      tile = slot % n_tiles;
+      const int per_kv = n_tiles * hsplit;
+      const int rem = slot % per_kv;
+      pair = ((slot / per_kv) * 8 + xcd) * hsplit + rem % hsplit;
+      tile = rem / hsplit;
     } else {
       pair = n / n_tiles;
       tile = n % n_tiles;
@@ -618,9 +622,18 @@ int launch_score_packed(const ScoreArgs& a) {
   constexpr bool DMA = MODE == 2;
   int nbuf = 2, chunk_words = 1;
   if (DMA) {
-    // two buffers, as many words per slice as LDS holds (no register staging to fit)
-    if (!a.grouped || 2 * bytes_per_word > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
-    while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= (size_t)lim.max_lds_per_block) ++chunk_words;
+    // The slice copy needs the table block of a workgroup contiguous: the grouped
+    // layout, or any layout when a workgroup serves one head.
+    if (!(a.grouped || GP == 1) || (a.grouped && GP == 1 && G != 1)) return SOCKET_ERR_UNSUPPORTED;
+    if (bytes_per_word * NW <= (size_t)lim.max_lds_per_block) {
+      // the whole table at once: one copy, no slices
+      nbuf = 1;
+      chunk_words = NW;
+    } else {
+      // two buffers, as many words per slice as LDS holds (no register staging to fit)
+      if (2 * bytes_per_word > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
+      while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= (size_t)lim.max_lds_per_block) ++chunk_words;
+    }
   } else if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && slots_per_word <= 1024) {
     // Double-buffered when one word's tables fit twice in LDS and in the staging
     // registers (1024 vector slots per workgroup); as many words per slice as that
@@ -645,7 +658,7 @@ int launch_score_packed(const ScoreArgs& a) {
   if (a.row_range && a.range_parts != n_tiles) return SOCKET_ERR_SHAPE;
   const int hsplit = (G + GP - 1) / GP;
   const int n_pairs = a.B * a.Hkv * hsplit;
-  const int xcd_remap = (n_pairs % 8 == 0) ? 1 : 0;
+  const int xcd_remap = ((a.B * a.Hkv) % 8 == 0) ? 1 : 0;
   const int n_wg = n_pairs * n_tiles;
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
                      a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
@@ -668,43 +681,70 @@ int dispatch_layout(const ScoreArgs& a) {
 }
 
 constexpr int kDmaKT4 = 2;  // token groups of four per lane in the direct-to-LDS variant
-constexpr int kDmaTile = 1024 * 4 * kDmaKT4 + 1;  // 8192-token tiles; the odd value only tags the variant
+
+// How a scorer launch is shaped.
+struct ScorePlan {
+  int tile;   // tokens per workgroup
+  bool dma;   // table slices copied global -> LDS directly
+  bool solo;  // one query head per workgroup, its whole table resident in LDS
+};
 
 // Tile size: the largest of 8192 / 4096 / 2048 / 1024 tokens per workgroup that
 // still gives every CU a workgroup.  With a grouped table the largest tile uses
 // the direct-to-LDS variant.
-int tile_tokens(int B, int Hkv, int G, int T, int grouped, size_t table_elem_bytes, int P, int R) {
+//
+// Few (b, kv head) pairs and a short context leave most CUs without a workgroup
+// at any useful tile size, and every workgroup still has to pull the pair's whole
+// table through LDS slice by slice, one exposed load latency per slice.  There a
+// workgroup takes ONE query head instead: that head's table (L*R elements) fits
+// LDS whole, is copied in once, and the tile runs with no barriers; the G
+// workgroups of a pair share its code stream through the XCD's L2.
+ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_elem_bytes, int L, int P, int R) {
   const SocketDeviceLimits& lim = socket_device_limits();
   const int width = G == 1 ? 1 : G == 2 ? 2 : 4;
   const int64_t pairs = (int64_t)B * Hkv * ((G + width - 1) / width);  // groups of 5..8 heads go as two workgroups
+  auto tiles = [&](int tw) { return (int64_t)((T + tw - 1) / tw); };
+  if (P > 0 && G > 1 && !grouped && pairs * tiles(8192) < lim.cu_count &&
+      (size_t)L * R * table_elem_bytes <= (size_t)lim.max_lds_per_block) {
+    const int64_t heads = (int64_t)B * Hkv * G;
+    for (int tw = 8192; tw > 1024; tw >>= 1)
+      if (heads * tiles(tw) >= lim.cu_count) return {tw, true, true};
+    return {1024, true, true};
+  }
   if (grouped && P > 0) {
     const size_t bytes_per_word = (size_t)(32 / P) * R * width * table_elem_bytes;
-    constexpr int tw = 1024 * 4 * kDmaKT4;
-    if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && pairs * ((T + tw - 1) / tw) >= lim.cu_count)
-      return kDmaTile;
+    if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && pairs * tiles(1024 * 4 * kDmaKT4) >= lim.cu_count)
+      return {1024 * 4 * kDmaKT4, true, false};
   }
-  if (pairs * ((T + 8191) / 8192) >= lim.cu_count) return 8192;
-  if (pairs * ((T + 4095) / 4096) >= lim.cu_count) return 4096;
-  if (pairs * ((T + 2047) / 2048) >= lim.cu_count) return 2048;
-  return 1024;
+  for (int tw = 8192; tw > 1024; tw >>= 1)
+    if (pairs * tiles(tw) >= lim.cu_count) return {tw, false, false};
+  return {1024, false, false};
 }
 
 template <int GP, class TT>
-int dispatch_tile(const ScoreArgs& a) {
-  const int tw = tile_tokens(a.B, a.Hkv, a.Hq / a.Hkv, a.T, a.grouped, sizeof(typename TT::elem), a.P, a.R);
-  if (tw == kDmaTile) return dispatch_p<GP, TT, kDmaKT4, 1024, 2>(a);
-  if (tw == 8192) return dispatch_layout<GP, TT, 2, 1024>(a);
-  if (tw == 4096) return dispatch_layout<GP, TT, 2, 512>(a);
-  if (tw == 2048) return dispatch_layout<GP, TT, 1, 512>(a);
+int dispatch_tile(const ScoreArgs& a, const ScorePlan& plan) {
+  if (plan.dma) {
+    if (plan.tile == 8192) return dispatch_p<GP, TT, 2, 1024, 2>(a);
+    if (GP == 1) {
+      if (plan.tile == 4096) return dispatch_p<1, TT, 1, 1024, 2>(a);
+      if (plan.tile == 2048) return dispatch_p<1, TT, 1, 512, 2>(a);
+      return dispatch_p<1, TT, 1, 256, 2>(a);
+    }
+    return SOCKET_ERR_UNSUPPORTED;
+  }
+  if (plan.tile == 8192) return dispatch_layout<GP, TT, 2, 1024>(a);
+  if (plan.tile == 4096) return dispatch_layout<GP, TT, 2, 512>(a);
+  if (plan.tile == 2048) return dispatch_layout<GP, TT, 1, 512>(a);
   return dispatch_layout<GP, TT, 1, 256>(a);
 }
 
 template <class TT>
 int dispatch_g(const ScoreArgs& a) {
   const int G = a.Hq / a.Hkv;
-  if (G == 1) return dispatch_tile<1, TT>(a);
-  if (G == 2) return dispatch_tile<2, TT>(a);
-  return dispatch_tile<4, TT>(a);
+  const ScorePlan plan = score_plan(a.B, a.Hkv, G, a.T, a.grouped, sizeof(typename TT::elem), a.L, a.P, a.R);
+  if (G == 1 || plan.solo) return dispatch_tile<1, TT>(a, plan);
+  if (G == 2) return dispatch_tile<2, TT>(a, plan);
+  return dispatch_tile<4, TT>(a, plan);
 }
 
 // ---------------------------------------------------------------------------
@@ -773,17 +813,26 @@ int launch_collision_i16(const QT* q_probs, const int16_t* key_buckets, const ui
 
 }  // namespace
 
-extern "C" int socket_score_range_parts(int B, int Hq, int Hkv, int T) {
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv != 0) return 0;
-  const int tw = tile_tokens(B, Hkv, Hq / Hkv, T, 0, 0, 0, 0);
-  return (T + tw - 1) / tw;
+namespace {
+int range_parts_of(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R, int grouped) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv != 0 || L <= 0 || P < 1 || P > 16 || R <= 0) return 0;
+  if (q_dtype != SOCKET_F32 && q_dtype != SOCKET_BF16) return 0;
+  const ScorePlan plan = score_plan(B, Hkv, Hq / Hkv, T, grouped, q_dtype == SOCKET_F32 ? 4 : 2, L, P, R);
+  return (T + plan.tile - 1) / plan.tile;
+}
+}  // namespace
+
+extern "C" int socket_score_range_parts(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {
+  return range_parts_of(B, Hq, Hkv, T, q_dtype, L, P, R, 0);
 }
 
-extern "C" int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int P, int R) {
-  if (B <= 0 || Hq <= 0 || Hkv <= 0 || T <= 0 || Hq % Hkv != 0 || P < 1 || P > 16 || R <= 0) return 0;
-  int tw = tile_tokens(B, Hkv, Hq / Hkv, T, 1, q_dtype == SOCKET_F32 ? 4 : 2, P, R);
-  if (tw == kDmaTile) tw = 1024 * 4 * kDmaKT4;
-  return (T + tw - 1) / tw;
+extern "C" int socket_score_prefers_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {
+  if (range_parts_of(B, Hq, Hkv, T, q_dtype, L, P, R, 0) == 0) return -1;
+  return score_plan(B, Hkv, Hq / Hkv, T, 0, q_dtype == SOCKET_F32 ? 4 : 2, L, P, R).solo ? 0 : 1;
+}
+
+extern "C" int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {
+  return range_parts_of(B, Hq, Hkv, T, q_dtype, L, P, R, 1);
 }
 
 namespace {

@@ -16,6 +16,7 @@ Nothing on the step path reads a length back to the host.
 """
 from __future__ import annotations
 
+import functools
 import math
 from typing import Optional, Tuple
 
@@ -119,6 +120,27 @@ def group_shape(n_heads: int, n_kv_heads: int) -> Tuple[int, int]:
     return parts.value, width.value
 
 
+@functools.lru_cache(maxsize=None)
+def _prefers_grouped(B: int, Hq: int, Hkv: int, T: int, dtype_code: int, L: int, P: int, R: int) -> bool:
+    r = lib().socket_score_prefers_grouped(B, Hq, Hkv, T, dtype_code, L, P, R)
+    if r < 0:
+        raise ValueError(f"socket_score_prefers_grouped: invalid shape B={B} Hq={Hq} Hkv={Hkv} T={T} L={L} P={P} R={R}")
+    return bool(r)
+
+
+def prefers_grouped(q_bhd: torch.Tensor, planes: torch.Tensor, protos_T: torch.Tensor, n_kv_heads: int,
+                    context_len: int, out_dtype: Optional[torch.dtype] = None) -> bool:
+    """Which table layout `soft_hash` should write for a scorer call over
+    `context_len` cached tokens: True = grouped, False = [B,Hq,L,R] (short
+    contexts with few kv heads, which the scorer serves one head per workgroup)."""
+    B, Hq = int(q_bhd.shape[0]), int(q_bhd.shape[1])
+    L, P = int(planes.shape[0]), int(planes.shape[1])
+    if out_dtype is None:
+        out_dtype = torch.bfloat16 if q_bhd.dtype == torch.bfloat16 else torch.float32
+    return _prefers_grouped(B, Hq, int(n_kv_heads), int(context_len), dtype_enum(out_dtype), L, P,
+                            int(protos_T.shape[1]))
+
+
 @torch.no_grad()
 def group_q_probs(q_probs: torch.Tensor, n_kv_heads: int) -> torch.Tensor:
     """[B,Hq,L,R] (float32 / bfloat16) -> grouped table [B, Hkv*parts, L, R, width]:
@@ -214,10 +236,8 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
         assert lens.dtype == torch.int32 and lens.is_cuda and lens.numel() == B
     rng, parts = None, 0
     if with_range:
-        if grouped:
-            parts = lib().socket_score_range_parts_grouped(B, Hq, Hkv, int(T), dtype_enum(q_probs.dtype), int(P), R)
-        else:
-            parts = lib().socket_score_range_parts(B, Hq, Hkv, int(T))
+        count = lib().socket_score_range_parts_grouped if grouped else lib().socket_score_range_parts
+        parts = count(B, Hq, Hkv, int(T), dtype_enum(q_probs.dtype), L, int(P), R)
         rng = torch.empty((B, Hq, parts, 2), dtype=torch.int32, device=q_probs.device)
     entry = lib().socket_score_packed_grouped if grouped else lib().socket_score_packed
     check("socket_score_packed", entry(

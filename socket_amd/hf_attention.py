@@ -237,7 +237,7 @@ class SocketLlamaAttention(nn.Module):
         M = max(0, min(self._effective_size(M_cfg, T_k), T_k))
         protos_T = self.get_protos_T(self._protos_cache, P, device, k.dtype)
         q_bhd = q[:, :, 0]
-        q_probs = _soft_hash(q_bhd, st["planes"], protos_T, Hkv)
+        q_probs = _soft_hash(q_bhd, st["planes"], protos_T, Hkv, T_k)
         out_bhd = _sparse_step(q_bhd, q_probs, k, v, st, T_k, sink, window, M)
         out = self.o_proj(out_bhd.reshape(B, 1, -1))
         return out, None, {"bucket_sparse": True, "mode": "cra_sparse", "T_k": int(T_k), "P": P, "R": R,
@@ -254,8 +254,9 @@ def _hash_rows(st: dict, k_new, v_new, t0: int) -> None:
     hash_cache.hash_keys_into(k_new, v_new, st["planes_words"], st["codes"], st["v_norm"], st["L"], st["P"], t0=t0)
 
 
-def _soft_hash(q_bhd, planes, protos_T, n_kv_heads: int):
-    return hash_cache.soft_hash(q_bhd, planes, protos_T, 0.3, n_kv_heads, grouped=True)
+def _soft_hash(q_bhd, planes, protos_T, n_kv_heads: int, context_len: int):
+    grouped = hash_cache.prefers_grouped(q_bhd, planes, protos_T, n_kv_heads, context_len)
+    return hash_cache.soft_hash(q_bhd, planes, protos_T, 0.3, n_kv_heads, grouped=grouped)
 
 
 def _sparse_step(q_bhd, q_probs, k, v, st: dict, T_k: int, sink: int, window: int, M: int):

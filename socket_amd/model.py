@@ -197,7 +197,10 @@ def _dense_step(q_bhd: Tensor, cache: KVCache) -> Tensor:
     return dense_decode_fwd(q_bhd, cache.k_cache, cache.v_cache, cache.lens)
 
 
-def _soft_hash(q_bhd: Tensor, planes: Tensor, protos_T: Tensor, n_kv_heads: int, grouped: bool = False) -> Tensor:
+def _soft_hash(q_bhd: Tensor, planes: Tensor, protos_T: Tensor, n_kv_heads: int, context_len: int = 0) -> Tensor:
+    """The query's bucket probabilities, in the table layout the scorer wants for a
+    context of `context_len` tokens (0: the reference's [B,H,L,R])."""
+    grouped = context_len > 0 and hash_cache.prefers_grouped(q_bhd, planes, protos_T, n_kv_heads, context_len)
     return hash_cache.soft_hash(q_bhd, planes, protos_T, 1.0, n_kv_heads, grouped=grouped)
 
 
@@ -410,8 +413,8 @@ class Attention(nn.Module):
         if sparse:
             T = cache.k_cache.size(2)       # upper bound; the kernels stop at cache.lens
             cfg = self.config
-            # on the device the table is written in the scorer's grouped layout (same values)
-            q_probs = (_soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, grouped=True)
+            # on the device the table is written in the layout the scorer prefers (same values)
+            q_probs = (_soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, T)
                        if q_bhd.is_cuda else self.soft_hash(q_bhd))
             out_bhd = _sparse_step(q_bhd, q_probs, cache, T, int(cfg.sink_size), int(cfg.window_size),
                                    int(self.heavy_const))
@@ -431,7 +434,7 @@ class Attention(nn.Module):
                                                          self.n_local_heads, return_new=True)
             _hash_rows(cache, k_new, v_new, pos_b=step.pos_b)
             cfg = self.config
-            q_probs = _soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, grouped=True)
+            q_probs = _soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, cache.k_cache.size(2))
             out_bhd = _sparse_step(q_bhd, q_probs, cache, cache.k_cache.size(2), int(cfg.sink_size),
                                    int(cfg.window_size), int(self.heavy_const))
         else:

@@ -567,7 +567,22 @@ def test_grouped_table_layout_gives_identical_scores(dev, B, Hq, Hkv, L, P, T, d
     packed = _packed_cache(codes, P, Tcap, dev)
     a, ra = hash_cache.score_packed(q_probs, packed, vn.to(dev), T, P, lens=lens, with_range=True)
     b, rb = hash_cache.score_packed(table, packed, vn.to(dev), T, P, lens=lens, with_range=True, n_heads=Hq)
-    assert torch.equal(a, b) and torch.equal(ra, rb)
+    # A short context with few kv heads is scored from the [B,Hq,L,R] table one
+    # head per workgroup, with plain fp32 adds; the grouped table always goes
+    # through the several-heads-at-once accumulate, whose last-place rounding can
+    # differ for bf16 entries.  fp32 entries: identical either way.
+    if dtype == torch.float32:
+        assert torch.equal(a, b)
+    else:
+        rel = ((a - b).abs() / b.abs().clamp_min(1e-30)).nan_to_num(0).max()
+        assert rel <= 2e-6, f"max rel diff {rel}"
+    if True:
+        for r, sc in ((ra, a), (rb, b)):   # each range array against its own scores
+            u, keys = r.cpu().numpy().view(np.uint32), _score_keys(sc.cpu())
+            for bb in range(B):
+                kk = keys[bb, :, :int(lens[bb])]
+                assert np.array_equal(u[bb, ..., 0].min(-1), kk.min(-1))
+                assert np.array_equal(u[bb, ..., 1].max(-1), kk.max(-1))
 
 
 def test_soft_hash_grouped_output_is_the_grouped_relayout(dev):

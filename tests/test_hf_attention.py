@@ -50,7 +50,7 @@ def _o_hash_rows(st, k_new, v_new, t0):
     st["v_norm"][:, :, t0:t0 + S] = orc.value_norm(v_new.detach().float().cpu())
 
 
-def _o_soft_hash(q_bhd, planes, protos_T, n_kv_heads):
+def _o_soft_hash(q_bhd, planes, protos_T, n_kv_heads, context_len):
     return orc.soft_hash(q_bhd.detach().float().cpu(), planes.float().cpu(), protos_T.float().cpu(), 0.3)
 
 

@@ -98,8 +98,9 @@ def test_sizes_helpers(lib):
     assert lib.socket_sparse_attention_workspace_bytes(4, 32, 128, 2308) == 4 * 32 * ns * 129 * 4
     assert lib.socket_select_workspace_bytes(4, 32, 4096, 128) == 0        # short rows: one workgroup per row
     assert lib.socket_select_workspace_bytes(4, 32, 131072, 2048) > 0
-    assert lib.socket_score_range_parts(4, 32, 8, 131072) * 8192 >= 131072
-    assert lib.socket_score_range_parts(1, 5, 2, 100) == 0
+    assert lib.socket_score_range_parts(4, 32, 8, 131072, 1, 60, 10, 1024) * 8192 >= 131072
+    assert lib.socket_score_range_parts_grouped(4, 32, 8, 131072, 1, 60, 10, 1024) == 16
+    assert lib.socket_score_range_parts(1, 5, 2, 100, 1, 60, 10, 1024) == 0
 
 
 def test_python_api_keeps_reference_signatures():
