@@ -25,6 +25,8 @@
 // per CU, not once per tile.
 #include "socket_common.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -71,6 +73,18 @@ __device__ __forceinline__ uint4 load_frag8<DType_f16>(const uint16_t* p) {
   r.z = (uint32_t)f32_to_bf16_bits(f[4]) | ((uint32_t)f32_to_bf16_bits(f[5]) << 16);
   r.w = (uint32_t)f32_to_bf16_bits(f[6]) | ((uint32_t)f32_to_bf16_bits(f[7]) << 16);
   return r;
+}
+
+// v of lane x ^ 16 / x ^ 32, without the LDS crossbar: v_permlane16_swap exchanges
+// the odd 16-lane rows of its first operand with the even rows of its second,
+// v_permlane32_swap the upper half of the first with the lower half of the second.
+__device__ __forceinline__ uint32_t lane_xor16(uint32_t v, bool odd_row) {
+  const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return odd_row ? r[0] : r[1];
+}
+__device__ __forceinline__ uint32_t lane_xor32(uint32_t v, bool upper_half) {
+  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return upper_half ? r[0] : r[1];
 }
 
 // LDS placement of the planes: row `col` is 16 groups of 16 bytes, group g stored
@@ -267,9 +281,9 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
           for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int r = 0; r < 4; ++r) neg = __builtin_amdgcn_alignbit(neg, __float_as_uint(acc[mb][nb][r]), 31);
-        const uint32_t t = (uint32_t)__shfl_xor((int)neg, 16, SOCKET_WAVE);
+        const uint32_t t = lane_xor16(neg, quarter & 1);
         const uint32_t x = __builtin_amdgcn_perm(t, neg, sel1);   // two blocks x this pair of quarters
-        const uint32_t u = (uint32_t)__shfl_xor((int)x, 32, SOCKET_WAVE);
+        const uint32_t u = lane_xor32(x, quarter & 2);
         const uint32_t word = __builtin_amdgcn_perm(u, x, sel2);  // block `quarter` x all four quarters
         if (s0 + lane < S) codes_pair[(int64_t)w * Tcap + pos0 + s0 + lane] = ~word & valid;
       };
@@ -309,6 +323,190 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
         }
       }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Streamed variant for large bf16 launches (prefill).
+//
+// The roles are turned round: the PLANES are stationary in registers and the
+// keys stream through LDS.  Wave i of the eight owns packed words i, i + 8 and
+// i + 16 (96 plane rows = 96 registers per lane, loaded once per kernel), and all
+// eight waves read the same 128-key tile, which arrives by direct global -> LDS
+// loads (no registers, no LDS store instructions) one tile ahead of the
+// contraction: the memory latency that the register-staged kernel above exposes
+// once per tile is hidden behind a whole tile of MFMA work.  Values come the same
+// way; wave i takes the norms of key block i of the tile from the Gram diagonal.
+//
+// LDS image of a tile: row r (256 bytes) holds its sixteen 16-byte chunks at slot
+// chunk ^ (r & 15); the lane that fetches slot s of row r asks global memory for
+// chunk s ^ (r & 15), so the image needs no pass of its own, and the sixteen
+// lanes of a fragment read (sixteen consecutive rows, one chunk) hit sixteen
+// different slots.
+constexpr int kStreamTile = 128;                       // keys per tile
+constexpr int kStreamTileBytes = kStreamTile * kD * 2;  // 32 KB
+constexpr int kStreamStageBytes = 2 * kStreamTileBytes; // keys | values
+constexpr int kStreamWordsPerWave = 3;
+constexpr int kStreamMaxWords = kStreamWordsPerWave * kHashWaves;
+
+__global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void hash_keys_stream_kernel(
+    const uint16_t* __restrict__ k_, const uint16_t* __restrict__ v_, int64_t k_sb, int64_t k_sh,
+    int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+    const uint16_t* __restrict__ planes_words,  // bf16 [NW*32, 128]
+    uint32_t* __restrict__ codes, uint16_t* __restrict__ v_norm,
+    const int32_t* __restrict__ pos_b, int t0, int Hkv, int S, int L, int P, int NW, int64_t Tcap,
+    int tiles_per_row, int n_tiles) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int prow = lane & 15, quarter = lane >> 4;
+  const int cpw = 32 / P;
+  const bool with_values = v_ != nullptr;
+
+  // this wave's plane rows, in the operand order of the sign-bit epilogue (see
+  // hash_keys_kernel): register set [j][k-step][plane block]
+  const int pbit0 = 8 * (prow >> 2) + 7 - (prow & 3);
+  Frag preg[kStreamWordsPerWave][kKSteps][2];
+  {
+    const uint4* planes16 = reinterpret_cast<const uint4*>(planes_words);
+#pragma unroll
+    for (int j = 0; j < kStreamWordsPerWave; ++j) {
+      const int w = wave + kHashWaves * j;
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+          const int col = w * 32 + pbit0 - 4 * mb;
+          preg[j][ks][mb].u = w < NW ? planes16[(int64_t)col * 16 + ks * 4 + quarter] : make_uint4(0, 0, 0, 0);
+        }
+    }
+  }
+  const uint32_t sel1 = (quarter & 1) ? 0x03070105u : 0x06020400u;
+  const uint32_t sel2 = (quarter & 2) ? 0x03020706u : 0x05040100u;
+
+  // this wave's four 1 KB pieces of a tile (rows 4p .. 4p+3 of piece p), keys and values
+  auto issue_tile = [&](int tile, int stage) {
+    const int pair = tile / tiles_per_row;
+    const int s0 = (tile % tiles_per_row) * kStreamTile;
+    const int b = pair / Hkv, h = pair % Hkv;
+    const uint16_t* kbase = k_ + b * k_sb + h * k_sh;
+    const uint16_t* vbase = with_values ? v_ + b * v_sb + h * v_sh : nullptr;
+    unsigned char* dst = lds_raw + (size_t)stage * kStreamStageBytes;
+#pragma unroll
+    for (int q = 0; q < kStreamTile / 4 / kHashWaves; ++q) {
+      const int p = wave + kHashWaves * q;
+      const int row = 4 * p + quarter;
+      const int srow = min(s0 + row, S - 1);  // rows past the end re-read the last one; never stored
+      const int chunk = prow ^ (row & 15);
+      lds_dma16(kbase + (int64_t)srow * k_ss + chunk * 8, dst + p * 1024);
+      if (with_values) lds_dma16(vbase + (int64_t)srow * v_ss + chunk * 8, dst + kStreamTileBytes + p * 1024);
+    }
+  };
+
+  int tile = blockIdx.x;
+  if (tile < n_tiles) issue_tile(tile, 0);
+  for (int it = 0; tile < n_tiles; tile += gridDim.x, ++it) {
+    const int stage = it & 1;
+    const int next = tile + gridDim.x;
+    // One barrier per tile: behind it every wave's pieces of this tile are in place
+    // AND every wave is done with the previous tile, whose stage the next tile's
+    // loads may therefore overwrite while this one is contracted.
+    wait_vmcnt(0);
+    __syncthreads();
+    if (next < n_tiles) issue_tile(next, stage ^ 1);
+
+    const int pair = tile / tiles_per_row;
+    const int s0 = (tile % tiles_per_row) * kStreamTile;
+    const int pos0 = pos_b ? pos_b[pair / Hkv] : t0;
+    const uint4* ktile = reinterpret_cast<const uint4*>(lds_raw + (size_t)stage * kStreamStageBytes);
+    const uint4* vtile = ktile + kStreamTileBytes / 16;
+    // chunk c of row r of a tile (r & 15 == prow for every row this lane reads)
+    auto frag_at = [&](const uint4* t, int r, int c) { return t[r * 16 + (c ^ prow)]; };
+
+    if (with_values) {
+      // ||v||^2 = diagonal of V V^T (see hash_keys_kernel), key block `wave` of the tile
+      Frag vf[kKSteps];
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) vf[ks].u = frag_at(vtile, wave * 16 + prow, ks * 4 + quarter);
+      f32x4 g = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[ks].v, vf[ks].v, g, 0, 0, 0);
+      const int r = prow - 4 * quarter;
+      const float d = r == 0 ? g[0] : r == 1 ? g[1] : r == 2 ? g[2] : g[3];
+      const int srow = s0 + wave * 16 + prow;
+      if (r >= 0 && r < 4 && srow < S) v_norm[(int64_t)pair * Tcap + pos0 + srow] = f32_to_f16_bits(sqrtf(d));
+    }
+
+    uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
+    // The tile's eight 16-key blocks go through in pairs, the next pair's
+    // fragments on their way from LDS while the current pair is contracted.  A
+    // 64-key group is taken high blocks first, (3,2) then (1,0), so that the sign
+    // bits shift into `neg` in the byte order the transpose expects.
+    auto pair_block = [](int pp) { return (pp >> 1) * 4 + ((pp & 1) ? 0 : 2); };  // lower block of pair pp
+    auto load_pair = [&](int pp, Frag (&kf)[2][kKSteps]) {
+      const int nb0 = pair_block(pp);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int ks = 0; ks < kKSteps; ++ks)
+          kf[i][ks].u = frag_at(ktile, (nb0 + i) * 16 + prow, ks * 4 + quarter);
+    };
+    auto tile_body = [&](auto nwords_c) {
+      constexpr int NWD = decltype(nwords_c)::value;
+      uint32_t neg[NWD];
+#pragma unroll
+      for (int j = 0; j < NWD; ++j) neg[j] = 0;
+      auto do_pair = [&](int pp, const Frag (&kf)[2][kKSteps]) {
+#pragma unroll
+        for (int j = 0; j < NWD; ++j) {
+          f32x4 acc[2][2];
+#pragma unroll
+          for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) acc[mb][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < kKSteps; ++ks)
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+              for (int i = 0; i < 2; ++i)
+                acc[mb][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(preg[j][ks][mb].v, kf[i][ks].v, acc[mb][i], 0, 0, 0);
+          // sign bits -> this quarter's byte per key block (higher block first)
+#pragma unroll
+          for (int i = 1; i >= 0; --i)
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) neg[j] = __builtin_amdgcn_alignbit(neg[j], __float_as_uint(acc[mb][i][r]), 31);
+          if (pp & 1) {
+            // all four blocks of the 64-key group are in: 4 x 4 byte transpose between
+            // the quarters (as in hash_keys_kernel), lane x gets key x's word
+            const int w = wave + kHashWaves * j;
+            const int nbits = min(cpw, L - w * cpw) * P;
+            const uint32_t valid = nbits >= 32 ? 0xffffffffu : ((1u << nbits) - 1u);
+            const uint32_t t = lane_xor16(neg[j], quarter & 1);
+            const uint32_t x = __builtin_amdgcn_perm(t, neg[j], sel1);
+            const uint32_t u = lane_xor32(x, quarter & 2);
+            const uint32_t word = __builtin_amdgcn_perm(u, x, sel2);
+            const int key = s0 + (pp >> 1) * kKeysPerWave + lane;
+            if (key < S) codes_pair[(int64_t)w * Tcap + pos0 + key] = ~word & valid;
+          }
+        }
+      };
+      Frag kfa[2][kKSteps], kfb[2][kKSteps];
+      load_pair(0, kfa);
+#pragma unroll
+      for (int pp = 0; pp < kStreamTile / 32; pp += 2) {
+        load_pair(pp + 1, kfb);
+        do_pair(pp, kfa);
+        if (pp + 2 < kStreamTile / 32) load_pair(pp + 2, kfa);
+        do_pair(pp + 1, kfb);
+      }
+    };
+    // (uniform per wave: waves 0 .. NW % 8 - 1 own one word more than the others)
+    const int my_words = wave < NW ? (NW - wave + kHashWaves - 1) / kHashWaves : 0;
+    if (my_words == 3) tile_body(std::integral_constant<int, 3>{});
+    else if (my_words == 2) tile_body(std::integral_constant<int, 2>{});
+    else if (my_words == 1) tile_body(std::integral_constant<int, 1>{});
   }
 }
 
@@ -428,11 +626,33 @@ extern "C" int socket_hash_keys(const void* k, const void* v, int dtype, int64_t
                        v_stride_s % per16 == 0,
                    SOCKET_ERR_ALIGN);
   }
+  const SocketDeviceLimits& lim = socket_device_limits();
+  hipStream_t s = (hipStream_t)stream;
+  {
+    // enough 128-key tiles to keep every CU streaming: the variant with the planes in registers
+    const int tiles_per_row = (S + kStreamTile - 1) / kStreamTile;
+    const int64_t n_tiles64 = (int64_t)B * Hkv * tiles_per_row;
+    SOCKET_REQUIRE(n_tiles64 < (1LL << 30), SOCKET_ERR_SHAPE);  // tile + grid size stays an int
+    if (dtype == SOCKET_BF16 && NW <= kStreamMaxWords && n_tiles64 >= lim.cu_count &&
+        2 * kStreamStageBytes <= lim.max_lds_per_block) {
+      const size_t lds = 2 * (size_t)kStreamStageBytes;
+      auto kern = hash_keys_stream_kernel;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds) != hipSuccess)
+        return SOCKET_ERR_LAUNCH;
+      const int n_wg = (int)(n_tiles64 < lim.cu_count ? n_tiles64 : lim.cu_count);
+      hipLaunchKernelGGL(kern, dim3(n_wg), dim3(kHashThreads), lds, s, (const uint16_t*)k, (const uint16_t*)v,
+                         k_stride_b, k_stride_h, k_stride_s, v_stride_b, v_stride_h, v_stride_s,
+                         (const uint16_t*)planes_words, codes, v_norm, pos_b, t0, Hkv, S, L, P, NW, Tcap,
+                         tiles_per_row, (int)n_tiles64);
+      SOCKET_LAUNCH_CHECK();
+      return SOCKET_OK;
+    }
+  }
   const int tiles_per_row = (S + kKeysPerWave - 1) / kKeysPerWave;
   const int64_t n_tiles64 = (int64_t)B * Hkv * tiles_per_row;
   SOCKET_REQUIRE(n_tiles64 < (1LL << 31), SOCKET_ERR_SHAPE);
   const int n_tiles = (int)n_tiles64;
-  const SocketDeviceLimits& lim = socket_device_limits();
   // plane slice: every word when they all fit in LDS (one slice, loaded once per
   // workgroup), else as many as fit; one persistent workgroup per CU
   int wc = lim.max_lds_per_block / (32 * kD * 2);
@@ -448,7 +668,6 @@ extern "C" int socket_hash_keys(const void* k, const void* v, int dtype, int64_t
   if (wc > words_per_wg) wc = words_per_wg;
   const size_t lds = (size_t)wc * 32 * kD * 2;
   const dim3 grid(n_wg, wsplit);
-  hipStream_t s = (hipStream_t)stream;
 #define SOCKET_HASH_LAUNCH(DT)                                                                     \
   do {                                                                                             \
     auto kern = hash_keys_kernel<DT>;                                                              \

@@ -121,6 +121,37 @@ __device__ __forceinline__ void store_elem<DType_f16>(void* base, int64_t idx, f
   ((uint16_t*)base)[idx] = f32_to_f16_bits(v);
 }
 
+// 16 bytes per lane from global memory straight into LDS: lane i's bytes land at
+// lds_dst + 16 * i (lds_dst is the same for the whole wave).  Written as assembly
+// so that the compiler does not serialise later LDS reads behind it; M0, which
+// carries the LDS address, is saved and restored.  Completion: vmcnt.
+__device__ __forceinline__ void lds_dma16(const void* src_lane, void* lds_dst) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_dst);
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src_lane), "s"(base)
+      : "memory");
+}
+
+// s_waitcnt vmcnt(n) only (n <= 15 here; larger requests wait for 15)
+__device__ __forceinline__ void wait_vmcnt(int n) {
+#define SOCKET_VM(k) \
+  case k: __builtin_amdgcn_s_waitcnt((k) | (7 << 4) | (15 << 8)); break;
+  switch (n) {
+    SOCKET_VM(0) SOCKET_VM(1) SOCKET_VM(2) SOCKET_VM(3) SOCKET_VM(4) SOCKET_VM(5) SOCKET_VM(6) SOCKET_VM(7)
+    SOCKET_VM(8) SOCKET_VM(9) SOCKET_VM(10) SOCKET_VM(11) SOCKET_VM(12) SOCKET_VM(13) SOCKET_VM(14)
+    default: __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (15 << 8)); break;
+  }
+#undef SOCKET_VM
+}
+
 // Cached device limits (read once per process; the library keeps no other state).
 struct SocketDeviceLimits {
   int cu_count;

@@ -462,6 +462,54 @@ def test_hash_keys_vs_oracle(dev, dtype, L, P, S):
     assert torch.allclose(got_vn.float(), want_vn.float(), rtol=1e-3, atol=0)
 
 
+def test_hash_keys_streamed_variant_equals_the_staged_one(dev):
+    """A launch with a 128-key tile for every CU takes the variant that keeps the
+    planes in registers and streams the keys through LDS.  Same contraction order,
+    so codes and norms must equal, bit for bit, those of the same rows hashed in
+    pieces small enough for the register-staged kernel; plus the oracle check."""
+    g = torch.Generator().manual_seed(60)
+    B, Hkv, D, L, P, S, t0 = 2, 8, 128, 60, 10, 2100, 40          # 17 tiles x 16 pairs, ragged last tile
+    Tcap = 2160
+    k = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+    v = (torch.randn(B, S, Hkv, D, generator=g) * 2).to(torch.bfloat16)
+    planes = torch.randn(L, P, D, generator=g)
+    NW = orc.words_per_key(L, P)
+    pw = hash_cache.permute_planes(planes.to(dev))
+    kd, vd = k.to(dev), v.to(dev)
+
+    def fresh():
+        return (torch.full((B, Hkv, NW, Tcap), -1, dtype=torch.int32, device=dev),
+                torch.full((B, Hkv, Tcap), -1.0, dtype=torch.float16, device=dev))
+
+    codes, vn = fresh()
+    hash_cache.hash_keys_into(kd, vd, pw, codes, vn, L, P, t0=t0, layout="bshd")
+    codes_p, vn_p = fresh()
+    for a in range(0, S, 700):
+        hash_cache.hash_keys_into(kd[:, a:a + 700], vd[:, a:a + 700], pw, codes_p, vn_p, L, P, t0=t0 + a, layout="bshd")
+    assert torch.equal(codes, codes_p) and torch.equal(vn, vn_p)
+    assert (codes[..., :t0] == -1).all() and (codes[..., t0 + S:] == -1).all()
+    assert (vn[..., :t0] == -1).all() and (vn[..., t0 + S:] == -1).all()
+    # per-sequence positions, no values
+    pos = torch.tensor([3, 57], dtype=torch.int32, device=dev)
+    codes_q, vn_q = fresh()
+    hash_cache.hash_keys_into(kd, None, pw, codes_q, None, L, P, pos_b=pos, layout="bshd")
+    for b in range(B):
+        p0 = int(pos[b])
+        assert torch.equal(codes_q[b, :, :, p0:p0 + S], codes[b, :, :, t0:t0 + S])
+        assert (codes_q[b, :, :, :p0] == -1).all() and (codes_q[b, :, :, p0 + S:] == -1).all()
+    assert (vn_q == -1).all()
+    # against fp64 projections on the decided bits, and the norms
+    got = hash_cache.unpack_codes(codes, L, P, t0, S, layout="bthl").cpu()
+    pb = planes.to(torch.bfloat16)
+    proj = orc.projections_f64(k, pb)
+    got_bits = ((got.long().unsqueeze(-1) >> torch.arange(P - 1, -1, -1)) & 1).bool()
+    decided = proj.abs() > 1e-3 * k.double().norm(dim=-1)[..., None, None] * pb.double().norm(dim=-1)
+    assert decided.float().mean() > 0.98
+    assert torch.equal(got_bits[decided], (proj >= 0)[decided])
+    want_vn = orc.value_norm(v).permute(0, 2, 1)
+    assert torch.allclose(vn[..., t0:t0 + S].cpu().float(), want_vn.float(), rtol=1e-3, atol=0)
+
+
 def test_hash_identity_planes_and_sign_flip(dev):
     """planes = +-unit vectors -> bits are the sign bits of key coordinates;
     hash(a*k) = hash(k) for a > 0; hash(-k) = ~hash(k) when no projection is 0."""
