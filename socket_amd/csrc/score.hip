@@ -300,79 +300,6 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
 #pragma unroll
       for (int g = 0; g < GP; ++g) acc[j][i][g] = 0.f;
 
-  // Packed words of the lane's token groups, kPrefetch words deep: ring[0] is the
-  // word being consumed, ring[d] the word d steps ahead.  The code stream is the
-  // HBM traffic of this kernel and a CU needs tens of KB of it in flight to cover
-  // the memory latency; one word ahead (16 B x tokens/4 per lane) is not enough.
-  constexpr int kPrefetch = DMA ? 4 : 3;  // the direct-to-LDS variant has the registers for one more
-  uint4 ring[kPrefetch][KT4];
-#pragma unroll
-  for (int d = 0; d < kPrefetch; ++d)
-#pragma unroll
-    for (int j = 0; j < KT4; ++j)
-      ring[d][j] = load_stream16(codes_pair + (int64_t)min(d, NW - 1) * Tcap + tsafe[j]);
-  // group j has consumed its current word: shift the ring and fetch the word
-  // kPrefetch steps ahead (past the end it refetches the last word, unused)
-  auto advance = [&](int j, int w) {
-#pragma unroll
-    for (int d = 0; d + 1 < kPrefetch; ++d) ring[d][j] = ring[d + 1][j];
-    ring[kPrefetch - 1][j] = load_stream16(codes_pair + (int64_t)min(w + kPrefetch, NW - 1) * Tcap + tsafe[j]);
-  };
-
-  // slice staging: slot s covers table elements [s*EPV, (s+1)*EPV) of every head
-  uint4 stage[SL][GP];
-  auto stage_load = [&](int l0) {
-    const int nt = min(chunk_tables, L - l0);
-    const int nslots = (nt * R) / EPV;
-    if (grouped) {  // straight copy: 16-byte vector i of the slice goes to vector i of the buffer
-      const uint4* src = reinterpret_cast<const uint4*>(qp_pair + (int64_t)l0 * R * GP);
-#pragma unroll
-      for (int k = 0; k < SL; ++k)
-#pragma unroll
-        for (int g = 0; g < GP; ++g) {
-          const int i = tid + (k * GP + g) * THREADS;
-          if (i < nslots * GP) stage[k][g] = src[i];
-        }
-      return;
-    }
-    const TE* src = qp_pair + (int64_t)l0 * R;
-#pragma unroll
-    for (int k = 0; k < SL; ++k) {
-      const int s = tid + k * THREADS;
-      if (s < nslots) {
-#pragma unroll
-        for (int g = 0; g < GP; ++g)
-          stage[k][g] = (g < G) ? *reinterpret_cast<const uint4*>(src + (int64_t)g * L * R + (int64_t)s * EPV)
-                                : make_uint4(0, 0, 0, 0);
-      }
-    }
-  };
-  auto stage_store = [&](int l0, int buf) {
-    const int nt = min(chunk_tables, L - l0);
-    const int nslots = (nt * R) / EPV;
-    uint4* dst = reinterpret_cast<uint4*>(lds_raw + (size_t)buf * chunk_elems * sizeof(TE));
-    if (grouped) {
-#pragma unroll
-      for (int k = 0; k < SL; ++k)
-#pragma unroll
-        for (int g = 0; g < GP; ++g) {
-          const int i = tid + (k * GP + g) * THREADS;
-          if (i < nslots * GP) dst[i] = stage[k][g];
-        }
-      return;
-    }
-#pragma unroll
-    for (int k = 0; k < SL; ++k) {
-      const int s = tid + k * THREADS;
-      if (s < nslots) {
-        uint4 o[GP];
-        interleave_heads<GP, TT>(stage[k], o);
-#pragma unroll
-        for (int v = 0; v < GP; ++v) dst[(size_t)s * GP + v] = o[v];
-      }
-    }
-  };
-
   // DMA: this wave's share of the slice that starts at table l0 -> buffer `buf`
   // (every 16th 1 KB piece); returns nothing, completion is awaited with vmcnt
   auto dma_slice = [&](int l0, int buf) {
@@ -385,110 +312,203 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
       if (o + lane * 16 < bytes) lds_dma16(src + o + lane * 16, dst + o);
     }
   };
-  const bool staged = nbuf == 2;
-  if (DMA) {
+  // A wave whose first token lies at or past the cached length has nothing to
+  // gather (a ragged batch; a context that overhangs the last full tile by a
+  // little): it only takes its share of the table copies and meets the barriers.
+  // The test is wave-uniform and made once, outside the gather loop.
+  const bool wave_active = !DMA || tile * TW + (tid >> 6) * 256 < len;
+  if (!wave_active) {
+    const int chunk_tables_ = chunk_words * cpw;
     dma_slice(0, 0);
-    wait_vmcnt(0);    // (the code prefetches above are waited for too; once per workgroup)
-    __syncthreads();  // slice 0 is in place
-  } else if (staged) {
-    stage_load(0);
-    stage_store(0, 0);
+    wait_vmcnt(0);
     __syncthreads();
-  }
+    int chunk_ = 0;
+    for (int w0 = 0; w0 < NW; w0 += chunk_words, ++chunk_) {
+      const int buf = nbuf == 2 ? (chunk_ & 1) : 0;
+      if (w0 + chunk_words < NW) dma_slice(w0 * cpw + chunk_tables_, buf ^ 1);
+      wait_vmcnt(0);
+      __syncthreads();
+    }
+  } else {
+    // Packed words of the lane's token groups, kPrefetch words deep: ring[0] is the
+    // word being consumed, ring[d] the word d steps ahead.  The code stream is the
+    // HBM traffic of this kernel and a CU needs tens of KB of it in flight to cover
+    // the memory latency; one word ahead (16 B x tokens/4 per lane) is not enough.
+    constexpr int kPrefetch = DMA ? 4 : 3;  // the direct-to-LDS variant has the registers for one more
+    uint4 ring[kPrefetch][KT4];
+#pragma unroll
+    for (int d = 0; d < kPrefetch; ++d)
+#pragma unroll
+      for (int j = 0; j < KT4; ++j)
+        ring[d][j] = load_stream16(codes_pair + (int64_t)min(d, NW - 1) * Tcap + tsafe[j]);
+    // group j has consumed its current word: shift the ring and fetch the word
+    // kPrefetch steps ahead (past the end it refetches the last word, unused)
+    auto advance = [&](int j, int w) {
+#pragma unroll
+      for (int d = 0; d + 1 < kPrefetch; ++d) ring[d][j] = ring[d + 1][j];
+      ring[kPrefetch - 1][j] = load_stream16(codes_pair + (int64_t)min(w + kPrefetch, NW - 1) * Tcap + tsafe[j]);
+    };
 
-  int chunk = 0;
-  for (int w0 = 0; w0 < NW; w0 += chunk_words, ++chunk) {
-    const int l0 = w0 * cpw;
-    const int buf = staged ? (chunk & 1) : 0;
-    const bool more = w0 + chunk_words < NW;
-    if (DMA) {
-      if (more) dma_slice(l0 + chunk_tables, buf ^ 1);
-    } else if (staged) {
-      if (more) stage_load(l0 + chunk_tables);
-    } else {
-      __syncthreads();  // gathers of the previous slice are done
+    // slice staging: slot s covers table elements [s*EPV, (s+1)*EPV) of every head
+    uint4 stage[SL][GP];
+    auto stage_load = [&](int l0) {
       const int nt = min(chunk_tables, L - l0);
       const int nslots = (nt * R) / EPV;
+      if (grouped) {  // straight copy: 16-byte vector i of the slice goes to vector i of the buffer
+        const uint4* src = reinterpret_cast<const uint4*>(qp_pair + (int64_t)l0 * R * GP);
+#pragma unroll
+        for (int k = 0; k < SL; ++k)
+#pragma unroll
+          for (int g = 0; g < GP; ++g) {
+            const int i = tid + (k * GP + g) * THREADS;
+            if (i < nslots * GP) stage[k][g] = src[i];
+          }
+        return;
+      }
       const TE* src = qp_pair + (int64_t)l0 * R;
-      uint4* dst = reinterpret_cast<uint4*>(lds_raw);
+#pragma unroll
+      for (int k = 0; k < SL; ++k) {
+        const int s = tid + k * THREADS;
+        if (s < nslots) {
+#pragma unroll
+          for (int g = 0; g < GP; ++g)
+            stage[k][g] = (g < G) ? *reinterpret_cast<const uint4*>(src + (int64_t)g * L * R + (int64_t)s * EPV)
+                                  : make_uint4(0, 0, 0, 0);
+        }
+      }
+    };
+    auto stage_store = [&](int l0, int buf) {
+      const int nt = min(chunk_tables, L - l0);
+      const int nslots = (nt * R) / EPV;
+      uint4* dst = reinterpret_cast<uint4*>(lds_raw + (size_t)buf * chunk_elems * sizeof(TE));
       if (grouped) {
-        const uint4* src16 = reinterpret_cast<const uint4*>(qp_pair + (int64_t)l0 * R * GP);
-        for (int i = tid; i < nslots * GP; i += THREADS) dst[i] = src16[i];
-      }
-      for (int s = tid; s < (grouped ? 0 : nslots); s += THREADS) {
-        uint4 x[GP], o[GP];
 #pragma unroll
-        for (int g = 0; g < GP; ++g)
-          x[g] = (g < G) ? *reinterpret_cast<const uint4*>(src + (int64_t)g * L * R + (int64_t)s * EPV)
-                         : make_uint4(0, 0, 0, 0);
-        interleave_heads<GP, TT>(x, o);
+        for (int k = 0; k < SL; ++k)
 #pragma unroll
-        for (int v = 0; v < GP; ++v) dst[(size_t)s * GP + v] = o[v];
+          for (int g = 0; g < GP; ++g) {
+            const int i = tid + (k * GP + g) * THREADS;
+            if (i < nslots * GP) dst[i] = stage[k][g];
+          }
+        return;
       }
+#pragma unroll
+      for (int k = 0; k < SL; ++k) {
+        const int s = tid + k * THREADS;
+        if (s < nslots) {
+          uint4 o[GP];
+          interleave_heads<GP, TT>(stage[k], o);
+#pragma unroll
+          for (int v = 0; v < GP; ++v) dst[(size_t)s * GP + v] = o[v];
+        }
+      }
+    };
+
+    const bool staged = nbuf == 2;
+    if (DMA) {
+      dma_slice(0, 0);
+      wait_vmcnt(0);    // (the code prefetches above are waited for too; once per workgroup)
+      __syncthreads();  // slice 0 is in place
+    } else if (staged) {
+      stage_load(0);
+      stage_store(0, 0);
       __syncthreads();
     }
 
-    const TE* table = reinterpret_cast<const TE*>(lds_raw) + (size_t)buf * chunk_elems;
-    const int wend = min(w0 + chunk_words, NW);
-    for (int w = w0; w < wend; ++w) {
-      const int ntw = min(cpw, L - w * cpw);
-      const TE* tw = table + (size_t)(w - w0) * cpw * R * GP;
-      constexpr int EB = GP * (int)sizeof(TE);
-      if (PT != 0 && ntw == 32 / (PT ? PT : 1)) {
-        // Every table of the word is real: straight-line code.  The lookups are
-        // cut into batches of four (one table, one group of four tokens) and the
-        // LDS reads of batch k+1 are issued before batch k is accumulated, so the
-        // gather latency overlaps the adds instead of preceding them.
-        constexpr int CPW = PT ? 32 / PT : 1;
-        constexpr int NB = KT4 * CPW;
-        RawEntry<EB> ent[2][4];
-        auto issue = [&](int bi, RawEntry<EB>(&dst)[4]) {
-          const int j = bi / CPW, jj = bi % CPW;
-          const uint32_t wv[4] = {ring[0][j].x, ring[0][j].y, ring[0][j].z, ring[0][j].w};
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const uint32_t code = __builtin_amdgcn_ubfe(wv[i], jj * (PT ? PT : 1), PT ? PT : 1);
-            dst[i] = load_entry<EB>(tw + (size_t)jj * R * GP + (size_t)code * GP);
-          }
-          if (jj == CPW - 1) advance(j, w);  // last use of this group's word
-        };
-        issue(0, ent[0]);
-#pragma unroll
-        for (int bi = 0; bi < NB; ++bi) {
-          if (bi + 1 < NB) issue(bi + 1, ent[(bi + 1) & 1]);
-          const int j = bi / CPW;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) accumulate<GP>(acc[j][i], ent[bi & 1][i], (const TT*)nullptr, sel);
-        }
+    int chunk = 0;
+    for (int w0 = 0; w0 < NW; w0 += chunk_words, ++chunk) {
+      const int l0 = w0 * cpw;
+      const int buf = staged ? (chunk & 1) : 0;
+      const bool more = w0 + chunk_words < NW;
+      if (DMA) {
+        if (more) dma_slice(l0 + chunk_tables, buf ^ 1);
+      } else if (staged) {
+        if (more) stage_load(l0 + chunk_tables);
       } else {
+        __syncthreads();  // gathers of the previous slice are done
+        const int nt = min(chunk_tables, L - l0);
+        const int nslots = (nt * R) / EPV;
+        const TE* src = qp_pair + (int64_t)l0 * R;
+        uint4* dst = reinterpret_cast<uint4*>(lds_raw);
+        if (grouped) {
+          const uint4* src16 = reinterpret_cast<const uint4*>(qp_pair + (int64_t)l0 * R * GP);
+          for (int i = tid; i < nslots * GP; i += THREADS) dst[i] = src16[i];
+        }
+        for (int s = tid; s < (grouped ? 0 : nslots); s += THREADS) {
+          uint4 x[GP], o[GP];
 #pragma unroll
-        for (int j = 0; j < KT4; ++j) {
-          const uint32_t wv[4] = {ring[0][j].x, ring[0][j].y, ring[0][j].z, ring[0][j].w};
-          for (int jj = 0; jj < ntw; ++jj) {
-            const TE* tb = tw + (size_t)jj * R * GP;
-            const int sh = jj * P;
+          for (int g = 0; g < GP; ++g)
+            x[g] = (g < G) ? *reinterpret_cast<const uint4*>(src + (int64_t)g * L * R + (int64_t)s * EPV)
+                           : make_uint4(0, 0, 0, 0);
+          interleave_heads<GP, TT>(x, o);
+#pragma unroll
+          for (int v = 0; v < GP; ++v) dst[(size_t)s * GP + v] = o[v];
+        }
+        __syncthreads();
+      }
+
+      const TE* table = reinterpret_cast<const TE*>(lds_raw) + (size_t)buf * chunk_elems;
+      const int wend = min(w0 + chunk_words, NW);
+      for (int w = w0; w < wend; ++w) {
+        const int ntw = min(cpw, L - w * cpw);
+        const TE* tw = table + (size_t)(w - w0) * cpw * R * GP;
+        constexpr int EB = GP * (int)sizeof(TE);
+        if (PT != 0 && ntw == 32 / (PT ? PT : 1)) {
+          // Every table of the word is real: straight-line code.  The lookups are
+          // cut into batches of four (one table, one group of four tokens) and the
+          // LDS reads of batch k+1 are issued before batch k is accumulated, so the
+          // gather latency overlaps the adds instead of preceding them.
+          constexpr int CPW = PT ? 32 / PT : 1;
+          constexpr int NB = KT4 * CPW;
+          RawEntry<EB> ent[2][4];
+          auto issue = [&](int bi, RawEntry<EB>(&dst)[4]) {
+            const int j = bi / CPW, jj = bi % CPW;
+            const uint32_t wv[4] = {ring[0][j].x, ring[0][j].y, ring[0][j].z, ring[0][j].w};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              const uint32_t code = (wv[i] >> sh) & code_mask;
-              accumulate<GP>(acc[j][i], load_entry<EB>(tb + (size_t)code * GP), (const TT*)nullptr, sel);
+              const uint32_t code = __builtin_amdgcn_ubfe(wv[i], jj * (PT ? PT : 1), PT ? PT : 1);
+              dst[i] = load_entry<EB>(tw + (size_t)jj * R * GP + (size_t)code * GP);
             }
+            if (jj == CPW - 1) advance(j, w);  // last use of this group's word
+          };
+          issue(0, ent[0]);
+#pragma unroll
+          for (int bi = 0; bi < NB; ++bi) {
+            if (bi + 1 < NB) issue(bi + 1, ent[(bi + 1) & 1]);
+            const int j = bi / CPW;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) accumulate<GP>(acc[j][i], ent[bi & 1][i], (const TT*)nullptr, sel);
           }
-          advance(j, w);
+        } else {
+#pragma unroll
+          for (int j = 0; j < KT4; ++j) {
+            const uint32_t wv[4] = {ring[0][j].x, ring[0][j].y, ring[0][j].z, ring[0][j].w};
+            for (int jj = 0; jj < ntw; ++jj) {
+              const TE* tb = tw + (size_t)jj * R * GP;
+              const int sh = jj * P;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                const uint32_t code = (wv[i] >> sh) & code_mask;
+                accumulate<GP>(acc[j][i], load_entry<EB>(tb + (size_t)code * GP), (const TT*)nullptr, sel);
+              }
+            }
+            advance(j, w);
+          }
         }
+      }
+
+      if (DMA) {
+        // The direct loads were issued at the top of the slice; since then this wave
+        // has issued one code prefetch per word and token group.  Loads retire in
+        // order, so allowing that many to be outstanding, less one word's worth as a
+        // margin, means the direct loads have landed.
+        wait_vmcnt(max(0, (min(w0 + chunk_words, NW) - w0 - 1) * KT4));
+        __syncthreads();
+      } else if (staged) {
+        if (more) stage_store(l0 + chunk_tables, buf ^ 1);
+        __syncthreads();
       }
     }
 
-    if (DMA) {
-      // The direct loads were issued at the top of the slice; since then this wave
-      // has issued one code prefetch per word and token group.  Loads retire in
-      // order, so allowing that many to be outstanding, less one word's worth as a
-      // margin, means the direct loads have landed.
-      wait_vmcnt(max(0, (min(w0 + chunk_words, NW) - w0 - 1) * KT4));
-      __syncthreads();
-    } else if (staged) {
-      if (more) stage_store(l0 + chunk_tables, buf ^ 1);
-      __syncthreads();
-    }
   }
 
   // epilogue: multiply by the value norm, mask, store one float4 per head; on
