@@ -19,8 +19,9 @@
 //    about 2m entries.  For long rows select_tau_kernel finds the thresholds (one
 //    workgroup per row, only the sample is read) and select_local_kernel applies
 //    them, one 256-lane workgroup per slice of 16384 scores held in registers
-//    (one HBM read of the scores in all); the row kernel only gathers the slices'
-//    lists.  A pool that comes out shorter than m or longer
+//    (one HBM read of the scores in all) and appending what passes to the row's
+//    list, in a stretch reserved with one atomic add; the row kernel reads that
+//    one compact list.  A pool that comes out shorter than m or longer
 //    than kPoolCap (the sample misjudged the row, or one key value is massively
 //    repeated) is dropped and the row redone from scratch: the result is always
 //    exact, only the time differs.
@@ -36,6 +37,7 @@
 // it); crowded bins fall back to an in-LDS bitonic sort whose short exchange
 // distances stay in registers and wave shuffles.
 #include "socket_common.h"
+
 
 namespace {
 
@@ -65,6 +67,7 @@ struct SelectShared {
   u64 wmin[kWaves], wmax[kWaves];
   int wsum[kWaves];
   int wflag[kWaves];
+  uint32_t kmin, kmax;  // key range of the pool
 };
 
 __device__ __forceinline__ u64 composite(uint32_t key, int idx) {
@@ -523,10 +526,11 @@ template <bool VEC>
 __global__ __launch_bounds__(kThreads) void select_tau_kernel(
     const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
     const int32_t* __restrict__ budgets, int Hq, int T, int M, int sink, int window, int write_base,
-    int list_width, uint32_t* __restrict__ tau_out) {
+    int list_width, uint32_t* __restrict__ tau_out, int32_t* __restrict__ row_count) {
   __shared__ uint32_t hist[kBins];
   __shared__ SelectShared sh;
   const int rowi = blockIdx.x, tid = threadIdx.x;
+  if (tid == 0) row_count[rowi] = 0;  // the slices add to it
   int n, m, nbase;
   row_shape(lens, budgets, rowi / Hq, T, M, sink, window, write_base, list_width, n, m, nbase);
   // short rows are pooled whole by the row kernel; it also takes over when no
@@ -541,27 +545,27 @@ __global__ __launch_bounds__(kThreads) void select_tau_kernel(
 }
 
 // One workgroup of 256 lanes per slice of 16384 scores, in two halves of 32 keys
-// per lane held in registers between counting and writing.
+// per lane held in registers between counting and writing.  What passes the
+// threshold goes to the ROW's list: a half's entries take a contiguous stretch
+// reserved with one atomic add on the row's counter, so the row kernel finds one
+// compact list (in no particular order; its result does not depend on it).  A
+// stretch that would run past the list's capacity is not written: the counter
+// then exceeds the capacity, which tells the row kernel to start from scratch.
 template <bool VEC>
 __global__ __launch_bounds__(kLocThreads) void select_local_kernel(
     const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens, int Hq, int T,
-    int S, int k_cap, const uint32_t* __restrict__ tau_in, u64* __restrict__ loc,
-    int32_t* __restrict__ loc_count) {
+    const uint32_t* __restrict__ tau_in, u64* __restrict__ loc, int32_t* __restrict__ row_count) {
   __shared__ int wsum[kLocWaves];
+  __shared__ int row_base;
   const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int n = lens ? max(0, min(lens[rowi / Hq], T)) : T;
   const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
-  const int64_t slot = (int64_t)rowi * S + s;
   const uint32_t tau = tau_in[rowi];
-  if (tau == kNoThreshold || end <= begin) {
-    if (tid == 0) loc_count[slot] = 0;
-    return;
-  }
+  if (tau == kNoThreshold || end <= begin) return;
   const float* row = scores + (int64_t)rowi * score_stride;
-  u64* my = loc + slot * k_cap;
+  u64* my = loc + (int64_t)rowi * kPoolCap;
   constexpr int kHalf = kLocPerLane / 2;
-  int written = 0;  // entries of the earlier half (uniform)
   for (int half = 0; half < 2; ++half) {
     // element e of lane t is index hbase + ((e / 4) * 256 + t) * 4 + e % 4; places past
     // the row's end get key 0 and are excluded by their index
@@ -590,27 +594,26 @@ __global__ __launch_bounds__(kLocThreads) void select_local_kernel(
 #pragma unroll
     for (int e = 0; e < kHalf; ++e) cnt += (key[e] >= tau && index_of(e) < end) ? 1 : 0;
     const int incl = wave_incl_scan(cnt, lane);
-    __syncthreads();  // the earlier half's readers of wsum are done
+    __syncthreads();  // the earlier half's readers of wsum / row_base are done
     if (lane == 63) wsum[wave] = incl;
     __syncthreads();
-    int at = written + incl - cnt, total = 0;
+    int at = incl - cnt, total = 0;
 #pragma unroll
     for (int w = 0; w < kLocWaves; ++w) {
       if (w < wave) at += wsum[w];
       total += wsum[w];
     }
-    written += total;
-    if (written > k_cap) {  // more than the slice's share of the pool: the row kernel starts over
-      if (tid == 0) loc_count[slot] = k_cap + 1;
-      return;
-    }
+    if (tid == 0) row_base = total ? atomicAdd(&row_count[rowi], total) : 0;
+    __syncthreads();
+    const int base = row_base;
+    if (base + total > kPoolCap) continue;  // (uniform) over capacity: see above
+    at += base;
 #pragma unroll
     for (int e = 0; e < kHalf; ++e) {
       const int i = index_of(e);
       if (key[e] >= tau && i < end) my[at++] = composite(key[e], i);
     }
   }
-  if (tid == 0) loc_count[slot] = written;
 }
 
 // ---------------------------------------------------------------------------
@@ -622,8 +625,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     const int32_t* __restrict__ budgets, const uint32_t* __restrict__ row_range, int range_parts,
     int Hq, int T, int M, int sink, int window, int write_base, int32_t* __restrict__ sparse_list,
     int64_t list_stride, int list_width, int32_t* __restrict__ sparse_len, int cap_above,
-    int counting_ok, int use_pool, const u64* __restrict__ loc, const int32_t* __restrict__ loc_count,
-    int S, int k_cap) {
+    int counting_ok, int use_pool, const u64* __restrict__ loc, const int32_t* __restrict__ row_count) {
   __shared__ uint32_t hist[kBins];
   __shared__ SelectShared sh;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -652,34 +654,48 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
       sh.fill_above = 0;
       sh.fill_cand = 0;
       sh.fill_pool = 0;
+      sh.kmin = 0xffffffffu;
+      sh.kmax = 0u;
     }
     int total = -1;  // uniform; stays -1 when no pool could be formed
+    uint32_t kmin = 0xffffffffu, kmax = 0u;  // key range of what this lane pooled
     if (n <= kPoolCap) {  // the whole row
-      for_each_in<VEC, kThreads>(row, 0, n, tid,
-                                 [&](int i, float x) { pool[i] = composite(score_to_key(x), i); });
+      for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
+        const uint32_t k = score_to_key(x);
+        kmin = min(kmin, k);
+        kmax = max(kmax, k);
+        pool[i] = composite(k, i);
+      });
       total = n;
     } else if (loc) {  // what the slices found above the sampled threshold
-      int sum = 0;
-      bool ok = true;
-      for (int s = 0; s < S; ++s) {
-        const int cnt = loc_count[(int64_t)rowi * S + s];
-        ok = ok && cnt <= k_cap;
-        sum += cnt;
-      }
-      if (ok && sum >= m && sum <= kPoolCap) {
-        int at = 0;
-        for (int s = 0; s < S; ++s) {
-          const int cnt = loc_count[(int64_t)rowi * S + s];
-          const u64* src = loc + ((int64_t)rowi * S + s) * k_cap;
-          for (int i = tid; i < cnt; i += kThreads) pool[at + i] = src[i];
-          at += cnt;
-        }
+      // The row's list is compact; its length and its entries are requested
+      // together (entries past the length are stale and never used), so the
+      // gather costs one memory latency.
+      constexpr int U = kPoolCap / kThreads;
+      const u64* src = loc + (int64_t)rowi * kPoolCap;
+      const int sum = row_count[rowi];
+      u64 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) v[u] = src[tid + u * kThreads];
+      if (sum >= m && sum <= kPoolCap) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (tid + u * kThreads < sum) {
+            const uint32_t k = (uint32_t)(v[u] >> 32);
+            kmin = min(kmin, k);
+            kmax = max(kmax, k);
+            pool[tid + u * kThreads] = v[u];
+          }
         total = sum;
       }
     } else if (sampling_ok(m)) {  // one workgroup: threshold from the sample, one pass
       const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
       for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
         const uint32_t k = score_to_key(x);
+        if (k >= tau) {
+          kmin = min(kmin, k);
+          kmax = max(kmax, k);
+        }
         wave_append(k >= tau, composite(k, i), &sh.fill_pool, pool, kPoolCap);
       });
       __syncthreads();
@@ -688,30 +704,21 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     }
     __syncthreads();
     if (total >= 0) {
-      // range of the pooled composites
-      u64 cmin = ~0ull, cmax = 0ull;
-      for (int i = tid; i < total; i += kThreads) {
-        const u64 v = pool[i];
-        cmin = min(cmin, v);
-        cmax = max(cmax, v);
-      }
+      // range of the pooled composites, from their keys (the high halves, noted
+      // as the pool was filled): any range that holds them all serves the refinement
 #pragma unroll
       for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
-        cmin = min(cmin, shfl_xor_u64(cmin, d));
-        cmax = max(cmax, shfl_xor_u64(cmax, d));
+        kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
+        kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, SOCKET_WAVE));
       }
       if (lane == 0) {
-        sh.wmin[wave] = cmin;
-        sh.wmax[wave] = cmax;
+        atomicMin(&sh.kmin, kmin);
+        atomicMax(&sh.kmax, kmax);
       }
       __syncthreads();
       if (tid == 0) {
-        for (int w = 1; w < kWaves; ++w) {
-          cmin = min(cmin, sh.wmin[w]);
-          cmax = max(cmax, sh.wmax[w]);
-        }
-        sh.lo = cmin;
-        sh.hi = max(cmin, cmax);
+        sh.lo = (u64)sh.kmin << 32;
+        sh.hi = ((u64)sh.kmax << 32) | 0xffffffffull;
         sh.need = m;
         sh.done = 0;
       }
@@ -892,24 +899,20 @@ int next_pow2(int x) {
   return p;
 }
 
-// Slices pay off once a row is several of them long.  Each gets room for k_cap
-// composites, several times an even share of the pool; 0 means "one workgroup
-// per row does everything".
-int slice_cap(int T, int m_max, int* S_out) {
+// Slices pay off once a row is several of them long; otherwise one workgroup per
+// row does everything.
+bool use_slices(int T, int m_max, int* S_out) {
   const int S = (T + kSliceLen - 1) / kSliceLen;
   *S_out = S;
-  if (S < 4 || S > kMaxSlices || m_max <= 0 || !sampling_ok(m_max)) return 0;
-  int k = 4 * kPoolCap / S;
-  if (k > 4096) k = 4096;
-  if (k < 512) k = 512;
-  return k;
+  return S >= 4 && S <= kMaxSlices && m_max > 0 && sampling_ok(m_max);
 }
 
 struct SplitLayout {
   size_t off_loc, off_count, off_tau, total;
 };
 
-SplitLayout split_layout(int rows, int S, int k_cap) {
+// per row: a candidate list of kPoolCap composites, its length, the threshold
+SplitLayout split_layout(int rows) {
   SplitLayout l;
   size_t o = 0;
   auto take = [&](size_t bytes) {
@@ -917,8 +920,8 @@ SplitLayout split_layout(int rows, int S, int k_cap) {
     o += (bytes + 255) / 256 * 256;
     return at;
   };
-  l.off_loc = take((size_t)rows * S * k_cap * sizeof(u64));
-  l.off_count = take((size_t)rows * S * sizeof(int32_t));
+  l.off_loc = take((size_t)rows * kPoolCap * sizeof(u64));
+  l.off_count = take((size_t)rows * sizeof(int32_t));
   l.off_tau = take((size_t)rows * sizeof(uint32_t));
   l.total = o;
   return l;
@@ -929,9 +932,8 @@ SplitLayout split_layout(int rows, int S, int k_cap) {
 extern "C" size_t socket_select_workspace_bytes(int B, int Hq, int T, int M) {
   if (B <= 0 || Hq <= 0 || T <= 0 || M < 0) return 0;
   int S = 0;
-  const int k_cap = slice_cap(T, M < T ? M : T, &S);
-  if (k_cap == 0) return 0;
-  return split_layout(B * Hq, S, k_cap).total;
+  if (!use_slices(T, M < T ? M : T, &S)) return 0;
+  return split_layout(B * Hq).total;
 }
 
 extern "C" int socket_select_list(const float* scores, int64_t score_stride, const int32_t* lens,
@@ -969,12 +971,12 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
     lds += (size_t)2 * cap_above * sizeof(u64);
   }
   int S = 0;
-  const int k_cap = (workspace && use_pool) ? slice_cap(T, m_max, &S) : 0;
+  const bool slices = workspace && use_pool && use_slices(T, m_max, &S);
 
   const u64* loc = nullptr;
   const int32_t* loc_count = nullptr;
-  if (k_cap) {
-    const SplitLayout l = split_layout(rows, S, k_cap);
+  if (slices) {
+    const SplitLayout l = split_layout(rows);
     SOCKET_REQUIRE(workspace_bytes >= l.total, SOCKET_ERR_WORKSPACE);
     SOCKET_REQUIRE(socket_aligned16(workspace), SOCKET_ERR_ALIGN);
     char* ws = (char*)workspace;
@@ -984,14 +986,14 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
     const dim3 sgrid(S, rows);
     if (vec) {
       hipLaunchKernelGGL(select_tau_kernel<true>, dim3(rows), dim3(kThreads), 0, s, scores, score_stride, lens,
-                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w);
+                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w, count_w);
       hipLaunchKernelGGL(select_local_kernel<true>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride, lens,
-                         Hq, T, S, k_cap, tau_w, loc_w, count_w);
+                         Hq, T, tau_w, loc_w, count_w);
     } else {
       hipLaunchKernelGGL(select_tau_kernel<false>, dim3(rows), dim3(kThreads), 0, s, scores, score_stride, lens,
-                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w);
+                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w, count_w);
       hipLaunchKernelGGL(select_local_kernel<false>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride, lens,
-                         Hq, T, S, k_cap, tau_w, loc_w, count_w);
+                         Hq, T, tau_w, loc_w, count_w);
     }
     SOCKET_LAUNCH_CHECK();
     loc = loc_w;
@@ -1006,7 +1008,7 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
   hipLaunchKernelGGL(kern, dim3(rows), dim3(kThreads), lds, s, scores, score_stride, lens, budgets,
                      row_range, range_parts, Hq, T, M, sink, window, write_base, sparse_list,
                      list_stride, list_width, sparse_len, cap_above, counting_ok, use_pool, loc,
-                     loc_count, S, k_cap);
+                     loc_count);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }
