@@ -195,13 +195,18 @@ __device__ __forceinline__ void interleave_heads(const uint4 (&x)[GP], uint4 (&o
 // The table slice of the tables held by `chunk_words` packed words sits in LDS;
 // with two LDS buffers the next slice is fetched into registers while the
 // current one is being gathered from, and there is one barrier per slice.
+// One tile of one workgroup's (b, kv head, head part).  `table_resident`: the whole
+// table is already in LDS from the tile this workgroup did before (single-buffer
+// launches only), so nothing is copied.  `red_off`: byte offset in LDS, past the
+// table buffers, of the small scratch area of the key-range reduction.
 template <int GP, class TT, int KT4, int THREADS, int PT, int MODE>
-__global__ __launch_bounds__(THREADS) void score_packed_kernel(
+__device__ __forceinline__ void score_tile(
     const typename TT::elem* __restrict__ q_probs, const uint32_t* __restrict__ codes,
     const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens,
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
-    int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
-    int n_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit) {
+    int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf,
+    int n_tiles, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit, int pair, int tile,
+    bool table_resident, int red_off) {
   // MODE: 0 = table in the reference layout [B,Hq,L,R], interleaved while staged;
   // 1 = grouped table, copied through registers; 2 = grouped table, copied from
   // global memory straight into LDS
@@ -222,26 +227,6 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   constexpr int CT = THREADS;  // lanes that own tokens
   constexpr int TW = CT * 4 * KT4;
 
-  // Workgroup -> (pair, tile).  Workgroups are dealt to the 8 XCDs round-robin
-  // by linear id; with the remap all tiles of one (b, kv head), and all the
-  // workgroups that share its query heads out between them, land on one XCD: its
-  // L2 serves that pair's table slices to every tile, and the pair's code stream
-  // comes from HBM once however many workgroups read it.
-  int pair, tile;
-  {
-    const int n = blockIdx.x;
-    if (xcd_remap) {
-      const int xcd = n & 7, slot = n >> 3;
-      const int per_kv = n_tiles * hsplit;
-      const int rem = slot % per_kv;
-      pair = ((slot / per_kv) * 8 + xcd) * hsplit + rem % hsplit;
-      tile = rem / hsplit;
-    } else {
-      pair = n / n_tiles;
-      tile = n % n_tiles;
-    }
-  }
-  if (pair >= n_pairs) return;
   // A group of more than GP query heads is shared out over `hsplit` workgroups
   // (each streams the pair's codes): this one takes heads [h0, h0 + G) of it.
   const int vpair = pair;  // (b, kv head, part of the head group)
@@ -319,9 +304,11 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   const bool wave_active = !DMA || tile * TW + (tid >> 6) * 256 < len;
   if (!wave_active) {
     const int chunk_tables_ = chunk_words * cpw;
-    dma_slice(0, 0);
-    wait_vmcnt(0);
-    __syncthreads();
+    if (!table_resident) {
+      dma_slice(0, 0);
+      wait_vmcnt(0);
+      __syncthreads();
+    }
     int chunk_ = 0;
     for (int w0 = 0; w0 < NW; w0 += chunk_words, ++chunk_) {
       const int buf = nbuf == 2 ? (chunk_ & 1) : 0;
@@ -405,9 +392,11 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
 
     const bool staged = nbuf == 2;
     if (DMA) {
-      dma_slice(0, 0);
-      wait_vmcnt(0);    // (the code prefetches above are waited for too; once per workgroup)
-      __syncthreads();  // slice 0 is in place
+      if (!table_resident) {
+        dma_slice(0, 0);
+        wait_vmcnt(0);    // (the code prefetches above are waited for too; once per workgroup)
+        __syncthreads();  // slice 0 is in place
+      }
     } else if (staged) {
       stage_load(0);
       stage_store(0, 0);
@@ -561,8 +550,8 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
         kmax[g] = max(kmax[g], (uint32_t)__shfl_xor((int)kmax[g], d, SOCKET_WAVE));
       }
     }
-    __syncthreads();  // every wave is done with the table slices
-    uint32_t* red = reinterpret_cast<uint32_t*>(lds_raw);
+    __syncthreads();  // an earlier tile's readers of the scratch area are done
+    uint32_t* red = reinterpret_cast<uint32_t*>(lds_raw + red_off);
     if (lane == 0) {
 #pragma unroll
       for (int g = 0; g < GP; ++g) {
@@ -583,6 +572,51 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     }
   }
 }
+
+template <int GP, class TT, int KT4, int THREADS, int PT, int MODE>
+__global__ __launch_bounds__(THREADS) void score_packed_kernel(
+    const typename TT::elem* __restrict__ q_probs, const uint32_t* __restrict__ codes,
+    const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens,
+    float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
+    int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
+    int n_tiles, int n_launch_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range,
+    int hsplit, int red_off) {
+  // Workgroup -> (pair, tile).  Workgroups are dealt to the 8 XCDs round-robin
+  // by linear id; with the remap all tiles of one (b, kv head), and all the
+  // workgroups that share its query heads out between them, land on one XCD: its
+  // L2 serves that pair's table slices to every tile, and the pair's code stream
+  // comes from HBM once however many workgroups read it.
+  int pair, tile;
+  {
+    const int n = blockIdx.x;
+    if (xcd_remap) {
+      const int xcd = n & 7, slot = n >> 3;
+      const int per_kv = n_launch_tiles * hsplit;
+      const int rem = slot % per_kv;
+      pair = ((slot / per_kv) * 8 + xcd) * hsplit + rem % hsplit;
+      tile = rem / hsplit;
+    } else {
+      pair = n / n_launch_tiles;
+      tile = n % n_launch_tiles;
+    }
+  }
+  if (pair >= n_pairs) return;
+  score_tile<GP, TT, KT4, THREADS, PT, MODE>(q_probs, codes, v_norm, lens, scores, Hq, Hkv, G, L, P_rt, R, T, Tcap,
+                                             score_stride, NW, chunk_words, nbuf, n_tiles, bf16_one, row_range,
+                                             hsplit, pair, tile, false, red_off);
+  // A short last tile is not given a workgroup of its own (a whole extra round of
+  // them on a full chip): the workgroup of the tile before it, with the table
+  // still in LDS, does it as well.  Only where one workgroup holds a whole table.
+  if constexpr (GP == 1 && MODE == 2) {
+    if (n_launch_tiles < n_tiles && tile == n_launch_tiles - 1)
+      score_tile<GP, TT, KT4, THREADS, PT, MODE>(q_probs, codes, v_norm, lens, scores, Hq, Hkv, G, L, P_rt, R, T,
+                                                 Tcap, score_stride, NW, chunk_words, nbuf, n_tiles, bf16_one,
+                                                 row_range, hsplit, pair, tile + 1, true, red_off);
+  }
+}
+
+// LDS past the table buffers in every launch: scratch of the key-range reduction
+constexpr size_t kScoreScratchBytes = 1024;
 
 struct ScoreArgs {
   const void* q_probs;
@@ -609,32 +643,34 @@ int launch_score_packed(const ScoreArgs& a) {
   const size_t bytes_per_word = (size_t)cpw * a.R * GP * sizeof(TE);
   const size_t slots_per_word = (size_t)cpw * a.R / EPV;
   constexpr bool DMA = MODE == 2;
+  const size_t lds_budget = (size_t)lim.max_lds_per_block - kScoreScratchBytes;
   int nbuf = 2, chunk_words = 1;
   if (DMA) {
     // The slice copy needs the table block of a workgroup contiguous: the grouped
     // layout, or any layout when a workgroup serves one head.
     if (!(a.grouped || GP == 1) || (a.grouped && GP == 1 && G != 1)) return SOCKET_ERR_UNSUPPORTED;
-    if (bytes_per_word * NW <= (size_t)lim.max_lds_per_block) {
+    if (bytes_per_word * NW <= lds_budget) {
       // the whole table at once: one copy, no slices
       nbuf = 1;
       chunk_words = NW;
     } else {
       // two buffers, as many words per slice as LDS holds (no register staging to fit)
-      if (2 * bytes_per_word > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
-      while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= (size_t)lim.max_lds_per_block) ++chunk_words;
+      if (2 * bytes_per_word > lds_budget) return SOCKET_ERR_UNSUPPORTED;
+      while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= lds_budget) ++chunk_words;
     }
-  } else if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && slots_per_word <= 1024) {
+  } else if (2 * bytes_per_word <= lds_budget && slots_per_word <= 1024) {
     // Double-buffered when one word's tables fit twice in LDS and in the staging
     // registers (1024 vector slots per workgroup); as many words per slice as that
     // allows.  Otherwise a single buffer filled in place.
-    while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= (size_t)lim.max_lds_per_block / 2 &&
+    while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= lds_budget / 2 &&
            slots_per_word * (chunk_words + 1) <= 1024)
       ++chunk_words;
   } else {
     nbuf = 1;
-    if (bytes_per_word > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
+    if (bytes_per_word > lds_budget) return SOCKET_ERR_UNSUPPORTED;
   }
-  const size_t lds_bytes = bytes_per_word * chunk_words * nbuf;
+  const size_t table_bytes = bytes_per_word * chunk_words * nbuf;
+  const size_t lds_bytes = table_bytes + kScoreScratchBytes;
 
   auto kern = score_packed_kernel<GP, TT, KT4, THREADS, PT, MODE>;
   if (lds_bytes > 48 * 1024) {
@@ -648,11 +684,15 @@ int launch_score_packed(const ScoreArgs& a) {
   const int hsplit = (G + GP - 1) / GP;
   const int n_pairs = a.B * a.Hkv * hsplit;
   const int xcd_remap = ((a.B * a.Hkv) % 8 == 0) ? 1 : 0;
-  const int n_wg = n_pairs * n_tiles;
+  // whole table resident (one buffer, one slice) and a last tile of at most a
+  // quarter of a tile's tokens: folded into the workgroup of the tile before it
+  int n_launch_tiles = n_tiles;
+  if (GP == 1 && DMA && nbuf == 1 && n_tiles >= 2 && a.T - (n_tiles - 1) * TW <= TW / 4) n_launch_tiles = n_tiles - 1;
+  const int n_wg = n_pairs * n_launch_tiles;
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
                      a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
-                     a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, xcd_remap, 0x3f80u,
-                     a.row_range, hsplit);
+                     a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, n_launch_tiles, xcd_remap,
+                     0x3f80u, a.row_range, hsplit, (int)table_bytes);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }
@@ -694,7 +734,7 @@ ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_ele
   const int64_t pairs = (int64_t)B * Hkv * ((G + width - 1) / width);  // groups of 5..8 heads go as two workgroups
   auto tiles = [&](int tw) { return (int64_t)((T + tw - 1) / tw); };
   if (P > 0 && G > 1 && !grouped && pairs * tiles(8192) < lim.cu_count &&
-      (size_t)L * R * table_elem_bytes <= (size_t)lim.max_lds_per_block) {
+      (size_t)L * R * table_elem_bytes + kScoreScratchBytes <= (size_t)lim.max_lds_per_block) {
     const int64_t heads = (int64_t)B * Hkv * G;
     for (int tw = 8192; tw > 1024; tw >>= 1)
       if (heads * tiles(tw) >= lim.cu_count) return {tw, true, true};
@@ -702,7 +742,8 @@ ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_ele
   }
   if (grouped && P > 0) {
     const size_t bytes_per_word = (size_t)(32 / P) * R * width * table_elem_bytes;
-    if (2 * bytes_per_word <= (size_t)lim.max_lds_per_block && pairs * tiles(1024 * 4 * kDmaKT4) >= lim.cu_count)
+    if (2 * bytes_per_word + kScoreScratchBytes <= (size_t)lim.max_lds_per_block &&
+        pairs * tiles(1024 * 4 * kDmaKT4) >= lim.cu_count)
       return {1024 * 4 * kDmaKT4, true, false};
   }
   for (int tw = 8192; tw > 1024; tw >>= 1)
