@@ -69,6 +69,8 @@ int socket_permute_planes(const void* planes, int planes_dtype, int L, int P, in
 
 /* Hash S new keys per (b, kv head) and store their packed codes and value
  * norms at cache positions pos0(b)+s, s in [0,S): pos0(b) = pos_b ? pos_b[b] : t0.
+ * t0 + S > Tcap is an error; with pos_b (int32 on the device, not visible to the
+ * host) rows whose position falls outside [0, Tcap) are dropped.
  * k, v address element [0,0,0,0] of the new rows with the given element strides
  * (last dim contiguous); v may be NULL (then v_norm is not written).
  * bit = (k . plane >= 0) from an MFMA bf16 contraction with fp32 accumulation.

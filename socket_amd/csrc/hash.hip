@@ -87,6 +87,10 @@ __device__ __forceinline__ uint32_t lane_xor32(uint32_t v, bool upper_half) {
   return upper_half ? r[0] : r[1];
 }
 
+// A cache position handed over on the device (per-sequence positions) is not
+// checked by the host: rows that would land outside [0, Tcap) are dropped.
+__device__ __forceinline__ bool in_cache(int pos, int64_t Tcap) { return (uint64_t)(int64_t)pos < (uint64_t)Tcap; }
+
 // LDS placement of the planes: row `col` is 16 groups of 16 bytes, group g stored
 // at slot g ^ plane_swizzle(col).  A fragment read has sixteen lanes on sixteen
 // columns {4..7} + 8j (or {0..3} + 8j) at one group; the swizzle sends those to
@@ -222,7 +226,7 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
               g = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vfrag[nb][ks].v, vfrag[nb][ks].v, g, 0, 0, 0);
             const float d = r == 0 ? g[0] : r == 1 ? g[1] : r == 2 ? g[2] : g[3];
             const int srow = s0 + nb * 16 + prow;
-            if (r >= 0 && r < 4 && srow < S) vn[srow] = f32_to_f16_bits(sqrtf(d));
+            if (r >= 0 && r < 4 && srow < S && in_cache(pos0 + srow, Tcap)) vn[srow] = f32_to_f16_bits(sqrtf(d));
           }
         }
       }
@@ -285,7 +289,7 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
         const uint32_t x = __builtin_amdgcn_perm(t, neg, sel1);   // two blocks x this pair of quarters
         const uint32_t u = lane_xor32(x, quarter & 2);
         const uint32_t word = __builtin_amdgcn_perm(u, x, sel2);  // block `quarter` x all four quarters
-        if (s0 + lane < S) codes_pair[(int64_t)w * Tcap + pos0 + s0 + lane] = ~word & valid;
+        if (s0 + lane < S && in_cache(pos0 + s0 + lane, Tcap)) codes_pair[(int64_t)w * Tcap + pos0 + s0 + lane] = ~word & valid;
       };
       // two fragment sets: the next word's LDS reads are in flight during the
       // current word's contraction
@@ -319,7 +323,7 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
           float t = ss[g];
 #pragma unroll
           for (int x = 1; x < 16; x <<= 1) t += __shfl_xor(t, x, SOCKET_WAVE);
-          if (part == 0 && srow < S) vn[srow] = f32_to_f16_bits(sqrtf(t));
+          if (part == 0 && srow < S && in_cache(pos0 + srow, Tcap)) vn[srow] = f32_to_f16_bits(sqrtf(t));
         }
       }
     }
@@ -433,7 +437,8 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
       const int r = prow - 4 * quarter;
       const float d = r == 0 ? g[0] : r == 1 ? g[1] : r == 2 ? g[2] : g[3];
       const int srow = s0 + wave * 16 + prow;
-      if (r >= 0 && r < 4 && srow < S) v_norm[(int64_t)pair * Tcap + pos0 + srow] = f32_to_f16_bits(sqrtf(d));
+      if (r >= 0 && r < 4 && srow < S && in_cache(pos0 + srow, Tcap))
+        v_norm[(int64_t)pair * Tcap + pos0 + srow] = f32_to_f16_bits(sqrtf(d));
     }
 
     uint32_t* codes_pair = codes + (int64_t)pair * NW * Tcap;
@@ -488,7 +493,7 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
             const uint32_t u = lane_xor32(x, quarter & 2);
             const uint32_t word = __builtin_amdgcn_perm(u, x, sel2);
             const int key = s0 + (pp >> 1) * kKeysPerWave + lane;
-            if (key < S) codes_pair[(int64_t)w * Tcap + pos0 + key] = ~word & valid;
+            if (key < S && in_cache(pos0 + key, Tcap)) codes_pair[(int64_t)w * Tcap + pos0 + key] = ~word & valid;
           }
         }
       };

@@ -184,7 +184,12 @@ def generate(model: Transformer, prompt: torch.Tensor, max_new_tokens: int, *, d
     T = prompt.size(1)
     B = prompt.size(0)
     T_new = T + max_new_tokens
-    max_seq_length = min(T_new, model.config.block_size)
+    if T_new > model.config.block_size:
+        # (GPT-FAST/generate.py:262-268 clamps the cache to block_size and then decodes
+        # past its end; here the request is refused before anything is launched)
+        raise ValueError(f"prompt ({T}) + max_new_tokens ({max_new_tokens}) = {T_new} exceeds the model's "
+                         f"block_size {model.config.block_size}")
+    max_seq_length = T_new
     device = prompt.device
     on_gpu = device.type == "cuda"
     model.setup_caches(max_batch_size=B, max_seq_length=max_seq_length)

@@ -510,6 +510,33 @@ def test_hash_keys_streamed_variant_equals_the_staged_one(dev):
     assert torch.allclose(vn[..., t0:t0 + S].cpu().float(), want_vn.float(), rtol=1e-3, atol=0)
 
 
+def test_hash_keys_drops_rows_whose_device_position_is_outside_the_cache(dev):
+    """Per-sequence positions live on the device; a row that would land at or past
+    the cache's capacity (or before its start) must be dropped, not written: the
+    word after the last row of `codes` is outside the buffer."""
+    g = torch.Generator().manual_seed(3)
+    B, Hkv, D, L, P, Tcap = 3, 2, 128, 60, 10, 64
+    NW = orc.words_per_key(L, P)
+    pw = hash_cache.permute_planes(torch.randn(L, P, D, generator=g).to(dev))
+    k = torch.randn(B, 1, Hkv, D, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(B, 1, Hkv, D, generator=g).to(torch.bfloat16).to(dev)
+    # one buffer with guard words around the cache proper
+    pad = 16
+    raw_c = torch.full((B * Hkv * NW * Tcap + 2 * pad,), -1, dtype=torch.int32, device=dev)
+    raw_n = torch.full((B * Hkv * Tcap + 2 * pad,), -1.0, dtype=torch.float16, device=dev)
+    codes = raw_c[pad:-pad].view(B, Hkv, NW, Tcap)
+    vn = raw_n[pad:-pad].view(B, Hkv, Tcap)
+    pos = torch.tensor([Tcap, 5, -1], dtype=torch.int32, device=dev)      # past the end, inside, before the start
+    hash_cache.hash_keys_into(k, v, pw, codes, vn, L, P, pos_b=pos, layout="bshd")
+    torch.cuda.synchronize()
+    assert (raw_c[:pad] == -1).all() and (raw_c[-pad:] == -1).all()
+    assert (raw_n[:pad] == -1).all() and (raw_n[-pad:] == -1).all()
+    assert (codes[0] == -1).all() and (codes[2] == -1).all() and (vn[0] == -1).all() and (vn[2] == -1).all()
+    assert (codes[1, :, :, 5] != -1).all() and (vn[1, :, 5] != -1).all()
+    touched = codes[1].clone(); touched[:, :, 5] = -1
+    assert (touched == -1).all()
+
+
 def test_hash_identity_planes_and_sign_flip(dev):
     """planes = +-unit vectors -> bits are the sign bits of key coordinates;
     hash(a*k) = hash(k) for a > 0; hash(-k) = ~hash(k) when no projection is 0."""

@@ -179,6 +179,15 @@ def test_sparse_hook_with_small_budget_keeps_cache_codes_consistent(monkeypatch)
     assert torch.equal(torch.from_numpy(have).permute(0, 3, 1, 2), want)
 
 
+def test_generate_refuses_a_request_longer_than_the_model_allows():
+    """Prompt + new tokens beyond block_size would decode past the end of the
+    cache; the harness says so before launching anything."""
+    model = toy_model()
+    prompt = torch.randint(0, 211, (1, 250))
+    with pytest.raises(ValueError, match="block_size"):
+        gen.generate(model, prompt, 7, decode_type="sparse")          # 257 > 256
+
+
 def test_sample_is_greedy():
     logits = torch.tensor([[[0.1, 2.0, -1.0], [3.0, 0.0, 0.5]]])
     tok, probs = gen.sample(logits)
