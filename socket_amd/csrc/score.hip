@@ -713,42 +713,58 @@ constexpr int kDmaKT4 = 2;  // token groups of four per lane in the direct-to-LD
 
 // How a scorer launch is shaped.
 struct ScorePlan {
-  int tile;   // tokens per workgroup
-  bool dma;   // table slices copied global -> LDS directly
-  bool solo;  // one query head per workgroup, its whole table resident in LDS
+  int tile;    // tokens per workgroup
+  bool dma;    // table slices copied global -> LDS directly
+  bool solo;   // one query head per workgroup, its whole table resident in LDS
+  float cost;  // rough time estimate, for comparing plans only
 };
 
-// Tile size: the largest of 8192 / 4096 / 2048 / 1024 tokens per workgroup that
-// still gives every CU a workgroup.  With a grouped table the largest tile uses
-// the direct-to-LDS variant.
-//
-// Few (b, kv head) pairs and a short context leave most CUs without a workgroup
-// at any useful tile size, and every workgroup still has to pull the pair's whole
-// table through LDS slice by slice, one exposed load latency per slice.  There a
-// workgroup takes ONE query head instead: that head's table (L*R elements) fits
-// LDS whole, is copied in once, and the tile runs with no barriers; the G
-// workgroups of a pair share its code stream through the XCD's L2.
+// Launch shapes and what they cost (microseconds measured at L60 x P10 bf16
+// tables on this GPU; only their ratios are used, to choose between shapes):
+//  * grouped / direct: 8192-token tiles, G heads per gather, table slices copied
+//    global -> LDS: ~53 per round of workgroups on a full chip, ~44 when the
+//    workgroups cover only part of it (a workgroup's time hardly depends on how
+//    many others there are);
+//  * reference layout through registers, 8192-token tiles: ~57 / ~50;
+//  * smaller tiles (4096 / 2048 / 1024) with staged slices: every workgroup still
+//    pulls the whole table through LDS, one exposed latency per slice, 60-70 per
+//    round whatever the tile: kept for tables whose slices do not fit LDS twice;
+//  * solo: ONE query head per workgroup, its whole table (L*R elements, if that
+//    fits LDS) copied in once, no barriers; the G workgroups of a kv head share its
+//    code stream through the XCD's L2.  ~5 + 31 * (tile / 8192) per round, but G
+//    times the workgroups: it wins while those still fit one round (short
+//    contexts, few kv heads) and loses to the grouped shape beyond.
+// Solo needs the [B,Hq,L,R] layout, the direct copy the grouped one: score_plan
+// prices the layout it is given, socket_score_prefers_grouped compares the two.
 ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_elem_bytes, int L, int P, int R) {
   const SocketDeviceLimits& lim = socket_device_limits();
   const int width = G == 1 ? 1 : G == 2 ? 2 : 4;
   const int64_t pairs = (int64_t)B * Hkv * ((G + width - 1) / width);  // groups of 5..8 heads go as two workgroups
   auto tiles = [&](int tw) { return (int64_t)((T + tw - 1) / tw); };
-  if (P > 0 && G > 1 && !grouped && pairs * tiles(8192) < lim.cu_count &&
-      (size_t)L * R * table_elem_bytes + kScoreScratchBytes <= (size_t)lim.max_lds_per_block) {
-    const int64_t heads = (int64_t)B * Hkv * G;
+  auto rounds = [&](int64_t wgs) { return (float)((wgs + lim.cu_count - 1) / lim.cu_count); };
+  const int64_t big = pairs * tiles(8192);  // workgroups of the 8192-token shapes
+  const size_t bytes_per_word = P > 0 ? (size_t)(32 / P) * R * width * table_elem_bytes : 0;
+  const bool slices_fit_twice = P > 0 && 2 * bytes_per_word + kScoreScratchBytes <= (size_t)lim.max_lds_per_block;
+  if (!slices_fit_twice) {
+    // staged small tiles: the largest that gives every CU a workgroup
     for (int tw = 8192; tw > 1024; tw >>= 1)
-      if (heads * tiles(tw) >= lim.cu_count) return {tw, true, true};
-    return {1024, true, true};
+      if (pairs * tiles(tw) >= lim.cu_count) return {tw, false, false, 65.f * rounds(pairs * tiles(tw))};
+    return {1024, false, false, 65.f * rounds(pairs * tiles(1024))};
   }
-  if (grouped && P > 0) {
-    const size_t bytes_per_word = (size_t)(32 / P) * R * width * table_elem_bytes;
-    if (2 * bytes_per_word + kScoreScratchBytes <= (size_t)lim.max_lds_per_block &&
-        pairs * tiles(1024 * 4 * kDmaKT4) >= lim.cu_count)
-      return {1024 * 4 * kDmaKT4, true, false};
+  if (grouped) return {1024 * 4 * kDmaKT4, true, false, big >= lim.cu_count ? 53.f * rounds(big) : 44.f};
+  ScorePlan best{8192, false, false, big >= lim.cu_count ? 57.f * rounds(big) : 50.f};
+  if (G > 1 && (size_t)L * R * table_elem_bytes + kScoreScratchBytes <= (size_t)lim.max_lds_per_block) {
+    const int64_t heads = (int64_t)B * Hkv * G;
+    int tw = 1024;
+    for (int t = 8192; t > 1024; t >>= 1)
+      if (heads * tiles(t) >= lim.cu_count) {
+        tw = t;
+        break;
+      }
+    const float cost = (5.f + 31.f * (float)tw / 8192.f) * rounds(heads * tiles(tw));
+    if (cost < best.cost) best = {tw, true, true, cost};
   }
-  for (int tw = 8192; tw > 1024; tw >>= 1)
-    if (pairs * tiles(tw) >= lim.cu_count) return {tw, false, false};
-  return {1024, false, false};
+  return best;
 }
 
 template <int GP, class TT>
@@ -858,7 +874,10 @@ extern "C" int socket_score_range_parts(int B, int Hq, int Hkv, int T, int q_dty
 
 extern "C" int socket_score_prefers_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {
   if (range_parts_of(B, Hq, Hkv, T, q_dtype, L, P, R, 0) == 0) return -1;
-  return score_plan(B, Hkv, Hq / Hkv, T, 0, q_dtype == SOCKET_F32 ? 4 : 2, L, P, R).solo ? 0 : 1;
+  const size_t eb = q_dtype == SOCKET_F32 ? 4 : 2;
+  const ScorePlan ref = score_plan(B, Hkv, Hq / Hkv, T, 0, eb, L, P, R);
+  const ScorePlan grp = score_plan(B, Hkv, Hq / Hkv, T, 1, eb, L, P, R);
+  return grp.cost <= ref.cost ? 1 : 0;
 }
 
 extern "C" int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {
