@@ -725,10 +725,11 @@ struct ScorePlan {
 //    global -> LDS: ~53 per round of workgroups on a full chip, ~44 when the
 //    workgroups cover only part of it (a workgroup's time hardly depends on how
 //    many others there are);
-//  * reference layout through registers, 8192-token tiles: ~57 / ~50;
-//  * smaller tiles (4096 / 2048 / 1024) with staged slices: every workgroup still
-//    pulls the whole table through LDS, one exposed latency per slice, 60-70 per
-//    round whatever the tile: kept for tables whose slices do not fit LDS twice;
+//  * slices staged through registers: 8192-token tiles ~57 per round (~50 on a part
+//    of the chip, ~73 with 32-bit entries); smaller tiles
+//    (4096 / 2048 / 1024, chosen so that every CU has a workgroup) ~45 per round
+//    from the reference layout and ~62 from the grouped one -- every workgroup
+//    still pulls the whole table through LDS, one exposed latency per slice;
 //  * solo: ONE query head per workgroup, its whole table (L*R elements, if that
 //    fits LDS) copied in once, no barriers; the G workgroups of a kv head share its
 //    code stream through the XCD's L2.  ~5 + 31 * (tile / 8192) per round, but G
@@ -745,14 +746,21 @@ ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_ele
   const int64_t big = pairs * tiles(8192);  // workgroups of the 8192-token shapes
   const size_t bytes_per_word = P > 0 ? (size_t)(32 / P) * R * width * table_elem_bytes : 0;
   const bool slices_fit_twice = P > 0 && 2 * bytes_per_word + kScoreScratchBytes <= (size_t)lim.max_lds_per_block;
-  if (!slices_fit_twice) {
-    // staged small tiles: the largest that gives every CU a workgroup
-    for (int tw = 8192; tw > 1024; tw >>= 1)
-      if (pairs * tiles(tw) >= lim.cu_count) return {tw, false, false, 65.f * rounds(pairs * tiles(tw))};
-    return {1024, false, false, 65.f * rounds(pairs * tiles(1024))};
+  // staged tiles: the largest that gives every CU a workgroup
+  ScorePlan staged{1024, false, false, (grouped ? 62.f : 45.f) * rounds(pairs * tiles(1024))};
+  for (int tw = 8192; tw > 1024; tw >>= 1)
+    if (pairs * tiles(tw) >= lim.cu_count) {
+      staged = {tw, false, false, (tw == 8192 ? 57.f : grouped ? 62.f : 45.f) * rounds(pairs * tiles(tw))};
+      break;
+    }
+  if (grouped) {
+    if (slices_fit_twice) return {1024 * 4 * kDmaKT4, true, false, big >= lim.cu_count ? 53.f * rounds(big) : 44.f};
+    return staged;
   }
-  if (grouped) return {1024 * 4 * kDmaKT4, true, false, big >= lim.cu_count ? 53.f * rounds(big) : 44.f};
-  ScorePlan best{8192, false, false, big >= lim.cu_count ? 57.f * rounds(big) : 50.f};
+  ScorePlan best = staged;
+  // 8192-token tiles on a part of the chip (16-bit entries ~50, 32-bit ~73)
+  const float big_part = table_elem_bytes == 2 ? 50.f : 73.f;
+  if (slices_fit_twice && big < lim.cu_count && big_part < best.cost) best = {8192, false, false, big_part};
   if (G > 1 && (size_t)L * R * table_elem_bytes + kScoreScratchBytes <= (size_t)lim.max_lds_per_block) {
     const int64_t heads = (int64_t)B * Hkv * G;
     int tw = 1024;
