@@ -271,9 +271,12 @@ class Transformer(nn.Module):
             # single launches; the position is handed on as it is (and once as int32
             # per sequence for the hashing kernel)
             step = DecodeStep(self.freqs_cis, input_pos.to(torch.int32).expand(idx.shape[0]).contiguous())
+            # a block hands on its residual stream and its FFN output separately: their sum
+            # is taken by the next norm's launch (the same add, rounded the same way)
+            ffn = None
             for layer in self.layers:
-                x = layer._run_fused(x, input_pos, sparse, step)
-            return self.output(decode_ops.add_rmsnorm(x, self.norm.weight, self.norm.eps)[1])
+                x, ffn = layer._run_fused(x, ffn, input_pos, sparse, step)
+            return self.output(decode_ops.add_rmsnorm(x, self.norm.weight, self.norm.eps, residual=ffn)[1])
         freqs_cis = self.freqs_cis[input_pos]
         for layer in self.layers:
             x = layer._run(x, input_pos, freqs_cis, sparse, pos0)
@@ -309,12 +312,15 @@ class TransformerBlock(nn.Module):
         h = x + self.attention._run(self.attention_norm(x), freqs_cis, input_pos, sparse, pos0)
         return h + self.feed_forward(self.ffn_norm(h))
 
-    def _run_fused(self, x, input_pos, sparse: bool, step: "DecodeStep"):
+    def _run_fused(self, x, pending, input_pos, sparse: bool, step: "DecodeStep"):
+        """One token through the block.  The block's input is x + pending (`pending`:
+        the previous block's FFN output, None for the first); returns the new
+        residual stream and this block's FFN output, not yet added."""
         an, fn, ff = self.attention_norm, self.ffn_norm, self.feed_forward
-        _, y = decode_ops.add_rmsnorm(x, an.weight, an.eps)
+        x, y = decode_ops.add_rmsnorm(x, an.weight, an.eps, residual=pending)
         a = self.attention._run_fused(y, input_pos, sparse, step)
         h, y = decode_ops.add_rmsnorm(x, fn.weight, fn.eps, residual=a)
-        return h + ff.w2(decode_ops.silu_mul(ff.w1(y), ff.w3(y)))
+        return h, ff.w2(decode_ops.silu_mul(ff.w1(y), ff.w3(y)))
 
     def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Tensor = None) -> Tensor:
         return self._run(x, input_pos, freqs_cis, False, None)
