@@ -120,7 +120,7 @@ def group_shape(n_heads: int, n_kv_heads: int) -> Tuple[int, int]:
     return parts.value, width.value
 
 
-@functools.lru_cache(maxsize=None)
+@functools.lru_cache(maxsize=4096)
 def _prefers_grouped(B: int, Hq: int, Hkv: int, T: int, dtype_code: int, L: int, P: int, R: int) -> bool:
     r = lib().socket_score_prefers_grouped(B, Hq, Hkv, T, dtype_code, L, P, R)
     if r < 0:
