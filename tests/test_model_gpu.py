@@ -134,6 +134,21 @@ def test_decode_graph_replays_equal_the_eager_step(dev, decode_type):
     assert torch.equal(seq_g, seq_e)
 
 
+def test_generate_up_to_the_last_row_of_the_cache_and_no_further(dev):
+    """prompt + new tokens == block_size: the last decoded position is the cache's
+    last row; graph and eager runs agree.  One token more is refused on the host."""
+    model = toy_model(dev, torch.bfloat16, seed=8)
+    g = torch.Generator().manual_seed(8)
+    prompt = torch.randint(0, 331, (1, 1000), generator=g).to(dev)
+    seq_g, st = gen.generate(model, prompt, 24, decode_type="sparse", use_graph=True)
+    assert seq_g.shape[1] == 1024 and model.max_seq_length == 1024
+    assert int(model.layers[0].attention.kv_cache.lens[0]) == 1023      # the last token is sampled, not appended
+    seq_e, _ = gen.generate(model, prompt, 24, decode_type="sparse", use_graph=False)
+    assert torch.equal(seq_g, seq_e)
+    with pytest.raises(ValueError, match="block_size"):
+        gen.generate(model, prompt, 25, decode_type="sparse")
+
+
 def test_all_covering_window_reproduces_dense_tokens_on_device(dev):
     model = toy_model(dev, torch.float32, seed=7, sink_size=0, window_size=4096, heavy_const=0)
     g = torch.Generator().manual_seed(7)
