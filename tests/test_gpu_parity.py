@@ -719,3 +719,61 @@ def test_decode_step_end_to_end(dev, name, T):
     # planted heavy keys are found: most of them are inside the selected set
     # (a sanity check of the whole chain, not a parity bar)
     assert out.dtype == w.dtype
+
+# ---------------------------------------------------------------- randomized shapes
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_shapes_score_and_select(dev, seed):
+    """Scorer and selector on randomly drawn geometries (head groups, table sizes,
+    context lengths around the tile and slice boundaries, ragged lengths, padding
+    in the cache rows), checked on the device against the definitions: the score
+    as a sequential fp32 sum over tables of gathered entries
+    (soft_hash_collision.cu:45-53), the heavy part of the list as a stable
+    descending sort of the row (ties: lower index first)."""
+    import random
+    rnd = random.Random(seed)
+    for _ in range(8):
+        G = rnd.choice([1, 2, 3, 4, 4, 7, 8])
+        Hkv = rnd.choice([1, 2, 4, 8])
+        B = rnd.choice([1, 1, 2, 4])
+        P = rnd.choice([10, 10, 8, 6])
+        L = rnd.choice([60, 48, 20, 7, 33])
+        T = rnd.choice([300, 1000, 4099, 8192, 8200, 16384, 20000, 40000, 65536, 65792, 70000, 98304, 131072])
+        if B * Hkv * G * T > 30e6:
+            T = 20000
+        dt = rnd.choice([torch.bfloat16, torch.float32])
+        R, Hq = 1 << P, Hkv * G
+        g = torch.Generator(device=dev).manual_seed(rnd.randrange(1 << 30))
+        case = f"B{B} Hq{Hq} Hkv{Hkv} L{L} P{P} T{T} {dt}"
+        qp = (torch.rand(B, Hq, L, R, generator=g, device=dev) *
+              torch.exp(-8 * torch.rand(B, Hq, L, R, generator=g, device=dev))).to(dt)
+        codes = torch.randint(0, R, (B, Hkv, L, T), generator=g, device=dev, dtype=torch.int32).to(torch.int16)
+        Tcap = (T + rnd.choice([0, 8, 64]) + 7) // 8 * 8
+        packed = torch.zeros(B, Hkv, orc.words_per_key(L, P), Tcap, dtype=torch.int32, device=dev)
+        hash_cache.pack_codes_into(codes, packed, P, t0=0)
+        vn = torch.zeros(B, Hkv, Tcap, dtype=torch.float16, device=dev)
+        vn[..., :T] = (torch.rand(B, Hkv, T, generator=g, device=dev) * 6).to(torch.float16)
+        lens = torch.randint(max(1, T // 3), T + 1, (B,), generator=g, device=dev, dtype=torch.int32)
+        a, ra = hash_cache.score_packed(qp, packed, vn, T, P, lens=lens, with_range=True)
+        b_ = hash_cache.score_packed(hash_cache.group_q_probs(qp, Hkv), packed, vn, T, P, lens=lens, n_heads=Hq)
+        want = torch.zeros(B, Hq, T, dtype=torch.float32, device=dev)
+        ce, qf = codes.long().repeat_interleave(G, dim=1), qp.float()
+        for l in range(L):
+            want += torch.gather(qf[:, :, l], 2, ce[:, :, l])
+        want *= vn[..., :T].float().repeat_interleave(G, dim=1)
+        want = want.masked_fill(torch.arange(T, device=dev)[None, None, :] >= lens[:, None, None], float("-inf"))
+        for name, got in (("[B,Hq,L,R] table", a[..., :T]), ("grouped table", b_[..., :T])):
+            assert torch.equal(torch.isinf(got), torch.isinf(want)), f"{case}: {name}"
+            rel = ((got - want).abs() / want.abs().clamp_min(1e-30)).nan_to_num(0).max().item()
+            assert rel <= (0.0 if dt == torch.float32 else 2e-6), f"{case}: {name} max rel diff {rel}"
+        M = rnd.choice([0, 1, 64, 1024, 2048, 3600])
+        sink, window = rnd.choice([(4, 256), (0, 0), (120, 120), (4, 16)])
+        sl, ln = sparse.select_list(a, sink, window, M, lens=lens, row_range=ra if rnd.random() < 0.5 else None)
+        for bb in range(B):
+            n = int(lens[bb])
+            m, s_e, w_e = min(M, n), min(sink, n), min(window, n)
+            ws = max(n - w_e, s_e)
+            nbase = s_e + (n - ws if w_e > 0 else 0)
+            nbase = max(nbase, 1)      # no sink, no window: the reference lists the newest token
+            order = torch.sort(a[bb, :, :n], dim=-1, descending=True, stable=True).indices[:, :m]
+            assert torch.equal(sl[bb, :, nbase:nbase + m].long(), order), f"{case}: sequence {bb}, M={M}"
+            assert (sl[bb, :, nbase + m:] == -1).all() and (ln[bb] == nbase + m).all(), f"{case}: sequence {bb}"
