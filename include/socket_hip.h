@@ -335,6 +335,27 @@ int socket_add_rmsnorm(const void* x, const void* residual, const void* weight, 
 /* out = round(silu(a)) * b elementwise over n elements (FeedForward, GPT-FAST/model.py:599-600). */
 int socket_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n, void* stream);
 
+/* Block-sparse prefill attention: out[b,h,row,:] = softmax over the listed key
+ * blocks (causal inside them) of q.k^T / sqrt(D), times v.  q, k, v, out are
+ * [B,H,T,D] views (element strides for dims 0-2, last dim contiguous), bf16 or
+ * fp16; seqlens int32 [B] (rows and keys at or past seqlens[b] do not take part,
+ * such rows of `out` are left untouched); block_index int32 [B,H,num_rows,klist],
+ * contiguous, every entry a key-block id in [0, ceil(T/64)) (entries outside are
+ * clamped into it); a block listed twice is attended twice.  num_rows must equal
+ * ceil(T/64); block_m and block_n must both be 64 (the reference's defaults).
+ * Replaces random_walk_fwd and its launcher random_walk_sparse_attention,
+ * kernels/block_sparse_flash_attention.py:280-437 (which pads T to whole blocks
+ * with zero rows instead of bounding the loads).  A row with no visible key in any
+ * listed block gives zeros here (the reference's exp2(-inf - -inf) gives NaN). */
+int socket_block_sparse_attention(const void* q, const void* k, const void* v, int dtype,
+                                  int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_m,
+                                  int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                  int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                                  const int32_t* seqlens, const int32_t* block_index, void* out,
+                                  int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_m,
+                                  int B, int H, int T, int D, int num_rows, int klist,
+                                  int block_m, int block_n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

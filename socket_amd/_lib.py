@@ -71,6 +71,7 @@ SIGNATURES = {
     "socket_dense_decode_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "socket_dense_decode": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L,
                                  _P, _P, _L, _L, _P, _Z, _I, _I, _I, _I, _I, _P]),
+    "socket_block_sparse_attention": (_I, [_P, _P, _P, _I] + [_L] * 9 + [_P, _P, _P] + [_L] * 3 + [_I] * 8 + [_P]),
 }
 
 _lib = None

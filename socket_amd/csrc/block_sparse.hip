@@ -1,0 +1,275 @@
+// Block-sparse prefill attention: every 64-row block of queries attends to a
+// listed set of 64-key blocks, causally, with an online softmax.
+//
+// Replaces random_walk_fwd + random_walk_sparse_attention,
+// kernels/block_sparse_flash_attention.py:280-437 (grid (row blocks, B*H), one
+// list of KLIST always-valid block ids per (b, h, row block), walked in order;
+// a block listed twice is attended twice, as there).
+//
+// One workgroup of four waves per row block; wave w owns query rows 16w .. 16w+15.
+// Both products run on v_mfma_f32_16x16x32 in the TRANSPOSED orientation, which
+// makes the query row the N index of every accumulator -- lane x holds row x % 16
+// in all its registers:
+//   S^T[key, row] = K . Q^T     A = K fragment (LDS), B = Q fragment (registers)
+//   O^T[dim, row] = V^T . P^T   A = V^T fragment (LDS), B = P^T (the lane's own
+//                                exponentials, rounded to the input type)
+// so the softmax needs no data movement at all: a row's maximum and sum are over a
+// lane's own registers plus the three other lane quarters (two lane-swap steps),
+// the rescale factor is uniform per lane, and the probabilities a lane computed
+// are exactly the B operand it has to supply.  The k index of the second product
+// is the key; its order inside an MFMA is free as long as both operands agree, so
+// slot i of lane quarter q stands for key 32c + 4q + i (i < 4) or 32c + 16 + 4q +
+// i - 4 -- the keys whose scores that quarter already holds.  V is stored
+// transposed in LDS ([dim][key], rows padded to 68 elements) so that those two
+// runs of four keys are two 8-byte reads.
+#include "socket_common.h"
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bs_bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 bs_f16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float bs_f32x4;
+
+constexpr int kBsBlock = 64;     // rows per query block, keys per key block
+constexpr int kBsThreads = 256;
+constexpr int kBsVtStride = kBsBlock + 4;  // elements per row of the transposed V tile
+
+template <class DT>
+struct BsType;
+template <>
+struct BsType<DType_bf16> {
+  static __device__ __forceinline__ bs_f32x4 mfma(const uint4& a, const uint4& b, bs_f32x4 c) {
+    union {
+      uint4 u;
+      bs_bf16x8 v;
+    } x, y;
+    x.u = a;
+    y.u = b;
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x.v, y.v, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+  }
+};
+template <>
+struct BsType<DType_f16> {
+  static __device__ __forceinline__ bs_f32x4 mfma(const uint4& a, const uint4& b, bs_f32x4 c) {
+    union {
+      uint4 u;
+      bs_f16x8 v;
+    } x, y;
+    x.u = a;
+    y.u = b;
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(x.v, y.v, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
+  }
+};
+
+// value of lane x ^ 16 / x ^ 32 (see hash.hip: v_permlane16_swap / v_permlane32_swap)
+__device__ __forceinline__ float bs_xor16(float v, bool odd_row) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(odd_row ? r[0] : r[1]);
+}
+__device__ __forceinline__ float bs_xor32(float v, bool upper_half) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(upper_half ? r[0] : r[1]);
+}
+
+template <class DT, int D>
+__global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
+    const uint16_t* __restrict__ q_, const uint16_t* __restrict__ k_, const uint16_t* __restrict__ v_,
+    int64_t q_sb, int64_t q_sh, int64_t q_sm, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t v_sb,
+    int64_t v_sh, int64_t v_sn, const int32_t* __restrict__ seqlens, const int32_t* __restrict__ block_index,
+    uint16_t* __restrict__ out, int64_t o_sb, int64_t o_sh, int64_t o_sm, int H, int T, int num_rows, int klist,
+    int num_cols, float scale_log2) {
+  constexpr int CH = D / 8;                 // 16-byte chunks per row
+  constexpr int KS = (D + 31) / 32;         // k-steps of the first product
+  constexpr int DB = D / 16;                // 16-dim blocks of the output
+  __shared__ __attribute__((aligned(16))) uint4 k_lds[kBsBlock * CH];
+  __shared__ __attribute__((aligned(16))) uint16_t vt_lds[D * kBsVtStride];
+
+  const int start_m = blockIdx.x, bh = blockIdx.y;
+  const int b = bh / H, h = bh % H;
+  const int seqlen = min(seqlens[b], T);
+  if (start_m * kBsBlock >= seqlen) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int prow = lane & 15, quarter = lane >> 4;
+  const int row = start_m * kBsBlock + wave * 16 + prow;   // this lane's query row (N index of every product)
+  const bool row_ok = row < seqlen;
+
+  const uint16_t* qb = q_ + b * q_sb + h * q_sh;
+  const uint16_t* kb = k_ + b * k_sb + h * k_sh;
+  const uint16_t* vb = v_ + b * v_sb + h * v_sh;
+
+  // Q fragments (B operand of S^T): row `row`, dims 32*ks + 8*quarter .. +7
+  uint4 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int chunk = 4 * ks + quarter;
+    qf[ks] = (chunk < CH && row_ok) ? *reinterpret_cast<const uint4*>(qb + (int64_t)row * q_sm + chunk * 8)
+                                    : make_uint4(0, 0, 0, 0);
+  }
+
+  bs_f32x4 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) o[db] = bs_f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_i = -INFINITY, l_part = 0.f;
+
+  const int32_t* blocks = block_index + ((int64_t)bh * num_rows + start_m) * klist;
+  for (int j = 0; j < klist; ++j) {
+    const int blk = min(max(blocks[j], 0), num_cols - 1);   // (the lists hold valid ids; a stray one must not fault)
+    const int start_n = blk * kBsBlock;
+    __syncthreads();  // the previous tiles have been consumed
+    for (int c = tid; c < kBsBlock * CH; c += kBsThreads) {
+      const int key = c / CH, chunk = c % CH;
+      const int col = start_n + key;
+      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
+      if (col < seqlen) {  // keys past the sequence read as zero (and are masked below)
+        kv = *reinterpret_cast<const uint4*>(kb + (int64_t)col * k_sn + chunk * 8);
+        vv = *reinterpret_cast<const uint4*>(vb + (int64_t)col * v_sn + chunk * 8);
+      }
+      k_lds[key * CH + (chunk ^ (key & (CH - 1)))] = kv;
+      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        vt_lds[(chunk * 8 + e) * kBsVtStride + key] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    }
+    __syncthreads();
+
+    // ---- S^T = K . Q^T: register r of block nb is key nb*16 + 4*quarter + r against row `row`
+    bs_f32x4 s[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) s[nb] = bs_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int chunk = 4 * ks + quarter;
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) {
+        const int key = nb * 16 + prow;
+        const uint4 a = chunk < CH ? k_lds[key * CH + (chunk ^ (key & (CH - 1)))] : make_uint4(0, 0, 0, 0);
+        s[nb] = BsType<DT>::mfma(a, qf[ks], s[nb]);
+      }
+    }
+    // ---- scale, causal mask, running maximum
+    float m_blk = -INFINITY;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int col = start_n + nb * 16 + 4 * quarter + r;
+        const float x = (row_ok && col <= row) ? s[nb][r] * scale_log2 : -INFINITY;
+        s[nb][r] = x;
+        m_blk = fmaxf(m_blk, x);
+      }
+    m_blk = fmaxf(m_blk, bs_xor16(m_blk, quarter & 1));
+    m_blk = fmaxf(m_blk, bs_xor32(m_blk, quarter & 2));
+    const float m_new = fmaxf(m_i, m_blk);
+    // (a row with nothing visible so far keeps alpha = 1 and p = 0 instead of the
+    // NaN of exp2(-inf - -inf))
+    const float alpha = (m_new == -INFINITY) ? 1.f : exp2f(m_i - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = (m_new == -INFINITY) ? 0.f : exp2f(s[nb][r] - m_new);
+        s[nb][r] = p;
+        psum += p;
+      }
+    l_part = l_part * alpha + psum;
+    m_i = m_new;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      o[db][0] *= alpha;
+      o[db][1] *= alpha;
+      o[db][2] *= alpha;
+      o[db][3] *= alpha;
+    }
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      uint4 pf;  // slots 0..3: keys 32c + 4q + r, slots 4..7: keys 32c + 16 + 4q + r
+      pf.x = BsType<DT>::pack2(s[2 * c][0], s[2 * c][1]);
+      pf.y = BsType<DT>::pack2(s[2 * c][2], s[2 * c][3]);
+      pf.z = BsType<DT>::pack2(s[2 * c + 1][0], s[2 * c + 1][1]);
+      pf.w = BsType<DT>::pack2(s[2 * c + 1][2], s[2 * c + 1][3]);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const uint16_t* vrow = vt_lds + (db * 16 + prow) * kBsVtStride + 32 * c + 4 * quarter;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        o[db] = BsType<DT>::mfma(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, o[db]);
+      }
+    }
+  }
+
+  float l = l_part;
+  l += bs_xor16(l, quarter & 1);
+  l += bs_xor32(l, quarter & 2);
+  if (!row_ok) return;
+  const float inv = 1.f / (l + 1e-9f);
+  uint16_t* orow = out + b * o_sb + h * o_sh + (int64_t)row * o_sm;
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    uint2 w;
+    w.x = BsType<DT>::pack2(o[db][0] * inv, o[db][1] * inv);
+    w.y = BsType<DT>::pack2(o[db][2] * inv, o[db][3] * inv);
+    *reinterpret_cast<uint2*>(orow + db * 16 + 4 * quarter) = w;
+  }
+}
+
+template <class DT>
+int launch_block_sparse(const void* q, const void* k, const void* v, int64_t q_sb, int64_t q_sh, int64_t q_sm,
+                        int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t v_sb, int64_t v_sh, int64_t v_sn,
+                        const int32_t* seqlens, const int32_t* block_index, void* out, int64_t o_sb, int64_t o_sh,
+                        int64_t o_sm, int B, int H, int T, int D, int num_rows, int klist, hipStream_t s) {
+  const int num_cols = (T + kBsBlock - 1) / kBsBlock;
+  const float scale_log2 = 1.44269504f / sqrtf((float)D);
+  const dim3 grid(num_rows, B * H);
+#define SOCKET_BS(DD)                                                                                        \
+  hipLaunchKernelGGL((block_sparse_fwd_kernel<DT, DD>), grid, dim3(kBsThreads), 0, s, (const uint16_t*)q,    \
+                     (const uint16_t*)k, (const uint16_t*)v, q_sb, q_sh, q_sm, k_sb, k_sh, k_sn, v_sb, v_sh, \
+                     v_sn, seqlens, block_index, (uint16_t*)out, o_sb, o_sh, o_sm, H, T, num_rows, klist,    \
+                     num_cols, scale_log2)
+  if (D == 128) SOCKET_BS(128);
+  else if (D == 64) SOCKET_BS(64);
+  else if (D == 32) SOCKET_BS(32);
+  else SOCKET_BS(16);
+#undef SOCKET_BS
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}
+
+}  // namespace
+
+extern "C" int socket_block_sparse_attention(const void* q, const void* k, const void* v, int dtype,
+                                             int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_m,
+                                             int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                             int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                                             const int32_t* seqlens, const int32_t* block_index, void* out,
+                                             int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_m, int B,
+                                             int H, int T, int D, int num_rows, int klist, int block_m,
+                                             int block_n, void* stream) {
+  SOCKET_REQUIRE(q && k && v && seqlens && block_index && out, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(dtype == SOCKET_BF16 || dtype == SOCKET_F16, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(D == 16 || D == 32 || D == 64 || D == 128, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(block_m == kBsBlock && block_n == kBsBlock, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(B > 0 && H > 0 && T > 0 && klist > 0 && (int64_t)B * H <= 65535, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(num_rows == (T + kBsBlock - 1) / kBsBlock, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(socket_aligned16(q) && socket_aligned16(k) && socket_aligned16(v) && socket_aligned16(out),
+                 SOCKET_ERR_ALIGN);
+  SOCKET_REQUIRE(q_stride_b % 8 == 0 && q_stride_h % 8 == 0 && q_stride_m % 8 == 0 && k_stride_b % 8 == 0 &&
+                     k_stride_h % 8 == 0 && k_stride_n % 8 == 0 && v_stride_b % 8 == 0 && v_stride_h % 8 == 0 &&
+                     v_stride_n % 8 == 0 && o_stride_b % 4 == 0 && o_stride_h % 4 == 0 && o_stride_m % 4 == 0,
+                 SOCKET_ERR_ALIGN);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == SOCKET_BF16)
+    return launch_block_sparse<DType_bf16>(q, k, v, q_stride_b, q_stride_h, q_stride_m, k_stride_b, k_stride_h,
+                                           k_stride_n, v_stride_b, v_stride_h, v_stride_n, seqlens, block_index,
+                                           out, o_stride_b, o_stride_h, o_stride_m, B, H, T, D, num_rows, klist, s);
+  return launch_block_sparse<DType_f16>(q, k, v, q_stride_b, q_stride_h, q_stride_m, k_stride_b, k_stride_h,
+                                        k_stride_n, v_stride_b, v_stride_h, v_stride_n, seqlens, block_index, out,
+                                        o_stride_b, o_stride_h, o_stride_m, B, H, T, D, num_rows, klist, s);
+}
