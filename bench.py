@@ -83,6 +83,28 @@ def time_launches(fn, iters, warmup=3):
     return start.elapsed_time(end) * 1000.0 / iters
 
 
+def block_sparse_bench(dev, iters, warmup):
+    """Block-sparse prefill attention (kernels/block_sparse_flash_attention.py) at the
+    C4 prompt: B1, 32 heads, T 65536, D128, bf16, 8 key blocks of 64 per 64-row block
+    (window of 4 + best-scoring others, from random block scores)."""
+    from socket_amd import block_sparse_flash_attention as bsa
+    B, H, T, D, K = 1, 32, 65536, 128, 8
+    g = torch.Generator(device=dev).manual_seed(4000)
+    q, k, v = (torch.randn(B, H, T, D, generator=g, device=dev, dtype=torch.bfloat16) for _ in range(3))
+    R = T // 64
+    blocks = bsa.random_walk_indices_from_block_probs(torch.rand(B, R, R, generator=g, device=dev), K, window_blocks=4)
+    blocks = bsa.expand_block_index_to_heads(blocks, H)
+    seqlens = torch.full((B,), T, dtype=torch.int32, device=dev)
+    us = time_launches(lambda: bsa.random_walk_sparse_attention(q, k, v, seqlens, blocks), iters, warmup=warmup)
+    flops = 2.0 * 2 * 64 * 64 * D * K * R * B * H              # both products over every listed block
+    tile_bytes = (2 * K * 64 * D * 2 + 2 * 64 * D * 2) * R * B * H   # K/V tiles fetched + q read + out written
+    print(json.dumps({"only": "block_sparse", "shape": f"B{B} H{H} T{T} D{D} bf16, {K} key blocks per row block",
+                      "us": round(us, 1), "mfma_tflops": round(flops / us / 1e6, 1),
+                      "mfma_frac": round(flops / us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+                      "tile_traffic_gbs": round(tile_bytes / us / 1e3, 1),
+                      "unique_MB": round(4 * B * H * T * D * 2 / 1e6, 1)}))
+
+
 def copy_ceiling_gbs(dev):
     """Measured device-to-device copy rate (read + write bytes) of a 1 GiB buffer."""
     n = 1 << 28
@@ -165,7 +187,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--only", default=None,
-                    choices=["score", "score_f32", "score_grouped", "select", "attend", "hash", "prefill_hash", "dense", "copy"])
+                    choices=["score", "score_f32", "score_grouped", "select", "attend", "hash", "prefill_hash", "dense", "copy",
+                             "block_sparse"])
     ap.add_argument("--reference-table-layout", action="store_true",
                     help="feed the scorer q_probs as [B,Hq,L,R] instead of the grouped layout the soft-hash kernel writes")
     ap.add_argument("--no-cpu", action="store_true")
@@ -185,6 +208,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.only == "block_sparse":
+        block_sparse_bench(dev, max(args.steps, 1), args.warmup)
+        return
     w = WORKLOADS[args.workload]
     t_gen = time.perf_counter()
     inp = make_inputs(w, device=dev, device_rng=True)

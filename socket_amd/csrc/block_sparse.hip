@@ -20,8 +20,10 @@
 // is the key; its order inside an MFMA is free as long as both operands agree, so
 // slot i of lane quarter q stands for key 32c + 4q + i (i < 4) or 32c + 16 + 4q +
 // i - 4 -- the keys whose scores that quarter already holds.  V is stored
-// transposed in LDS ([dim][key], rows padded to 68 elements) so that those two
-// runs of four keys are two 8-byte reads.
+// transposed in LDS ([dim][key]) so that those two runs of four keys are two
+// 8-byte reads: rows of 72 elements, the sixteen 4-key groups of a row placed at
+// group ^ (dim / 8 % 16), which keeps both the transposing stores and the
+// fragment reads at the two LDS passes their 512 bytes need.
 #include "socket_common.h"
 
 namespace {
@@ -32,7 +34,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float bs_f32x4;
 
 constexpr int kBsBlock = 64;     // rows per query block, keys per key block
 constexpr int kBsThreads = 256;
-constexpr int kBsVtStride = kBsBlock + 4;  // elements per row of the transposed V tile
+constexpr int kBsVtStride = kBsBlock + 8;  // elements per row of the transposed V tile
 
 template <class DT>
 struct BsType;
@@ -47,8 +49,16 @@ struct BsType<DType_bf16> {
     y.u = b;
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x.v, y.v, c, 0, 0, 0);
   }
+  // (the conversion instruction of the target, round to nearest even)
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    union {
+      bf2 v;
+      uint32_t u;
+    } r;
+    r.v = __builtin_convertvector(f2{lo, hi}, bf2);
+    return r.u;
   }
 };
 template <>
@@ -63,7 +73,14 @@ struct BsType<DType_f16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(x.v, y.v, c, 0, 0, 0);
   }
   static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return (uint32_t)f32_to_f16_bits(lo) | ((uint32_t)f32_to_f16_bits(hi) << 16);
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    union {
+      h2 v;
+      uint32_t u;
+    } r;
+    r.v = __builtin_convertvector(f2{lo, hi}, h2);
+    return r.u;
   }
 };
 
@@ -90,7 +107,20 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
   __shared__ __attribute__((aligned(16))) uint4 k_lds[kBsBlock * CH];
   __shared__ __attribute__((aligned(16))) uint16_t vt_lds[D * kBsVtStride];
 
-  const int start_m = blockIdx.x, bh = blockIdx.y;
+  // Workgroups are dealt to the 8 XCDs round-robin by linear id.  Renumbered so
+  // that each XCD walks one contiguous eighth of the (head, row block) space in
+  // order: neighbouring row blocks share their window tiles, which then come from
+  // that XCD's L2 instead of being fetched once per XCD.
+  int start_m = blockIdx.x, bh = blockIdx.y;
+  {
+    const int64_t total = (int64_t)gridDim.x * gridDim.y;
+    if (total % 8 == 0) {
+      const int64_t n = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+      const int64_t id = (n % 8) * (total / 8) + n / 8;
+      start_m = (int)(id % num_rows);
+      bh = (int)(id / num_rows);
+    }
+  }
   const int b = bh / H, h = bh % H;
   const int seqlen = min(seqlens[b], T);
   if (start_m * kBsBlock >= seqlen) return;
@@ -118,25 +148,54 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
   float m_i = -INFINITY, l_part = 0.f;
 
   const int32_t* blocks = block_index + ((int64_t)bh * num_rows + start_m) * klist;
-  for (int j = 0; j < klist; ++j) {
+  // Staging: thread t < 16*CH takes chunk t % CH of the four keys 4*(t / CH) .. +3 of
+  // a tile.  The K chunks go to LDS as they are; the V chunks are transposed in
+  // registers (two byte-selects per output word) so that the four keys of one dim
+  // leave as a single 8-byte store.  The next tile's chunks are requested before
+  // the current tile is contracted and are in registers by the time it is done.
+  const bool stager = tid < 16 * CH;
+  const int st_chunk = tid % CH, st_key0 = 4 * (tid / CH);
+  uint4 kr[4], vr[4];
+  auto fetch_tile = [&](int j) {
     const int blk = min(max(blocks[j], 0), num_cols - 1);   // (the lists hold valid ids; a stray one must not fault)
-    const int start_n = blk * kBsBlock;
-    __syncthreads();  // the previous tiles have been consumed
-    for (int c = tid; c < kBsBlock * CH; c += kBsThreads) {
-      const int key = c / CH, chunk = c % CH;
-      const int col = start_n + key;
-      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (col < seqlen) {  // keys past the sequence read as zero (and are masked below)
-        kv = *reinterpret_cast<const uint4*>(kb + (int64_t)col * k_sn + chunk * 8);
-        vv = *reinterpret_cast<const uint4*>(vb + (int64_t)col * v_sn + chunk * 8);
-      }
-      k_lds[key * CH + (chunk ^ (key & (CH - 1)))] = kv;
-      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        vt_lds[(chunk * 8 + e) * kBsVtStride + key] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+    for (int i = 0; i < 4; ++i) {
+      const int col = blk * kBsBlock + st_key0 + i;
+      kr[i] = vr[i] = make_uint4(0, 0, 0, 0);
+      if (stager && col < seqlen) {  // keys past the sequence read as zero (and are masked below)
+        kr[i] = *reinterpret_cast<const uint4*>(kb + (int64_t)col * k_sn + st_chunk * 8);
+        vr[i] = *reinterpret_cast<const uint4*>(vb + (int64_t)col * v_sn + st_chunk * 8);
+      }
     }
+  };
+  auto store_tile = [&]() {
+    if (!stager) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = st_key0 + i;
+      k_lds[key * CH + (st_chunk ^ (key & (CH - 1)))] = kr[i];
+    }
+    const uint32_t w[4][4] = {{vr[0].x, vr[0].y, vr[0].z, vr[0].w},
+                              {vr[1].x, vr[1].y, vr[1].z, vr[1].w},
+                              {vr[2].x, vr[2].y, vr[2].z, vr[2].w},
+                              {vr[3].x, vr[3].y, vr[3].z, vr[3].w}};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;   // high / low halves of the two words
+      uint2 t;
+      t.x = __builtin_amdgcn_perm(w[1][e >> 1], w[0][e >> 1], sel);   // keys 0, 1
+      t.y = __builtin_amdgcn_perm(w[3][e >> 1], w[2][e >> 1], sel);   // keys 2, 3
+      *reinterpret_cast<uint2*>(vt_lds + (st_chunk * 8 + e) * kBsVtStride + (((st_key0 >> 2) ^ st_chunk) << 2)) = t;
+    }
+  };
+
+  fetch_tile(0);
+  for (int j = 0; j < klist; ++j) {
+    const int start_n = min(max(blocks[j], 0), num_cols - 1) * kBsBlock;
+    __syncthreads();  // the previous tiles have been consumed
+    store_tile();
     __syncthreads();
+    if (j + 1 < klist) fetch_tile(j + 1);
 
     // ---- S^T = K . Q^T: register r of block nb is key nb*16 + 4*quarter + r against row `row`
     bs_f32x4 s[4];
@@ -152,29 +211,43 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
         s[nb] = BsType<DT>::mfma(a, qf[ks], s[nb]);
       }
     }
-    // ---- scale, causal mask, running maximum
+    // ---- causal mask, running maximum (of the raw dot products: the scale is
+    // positive and is applied inside the exponent).  A tile wholly at or left of
+    // this wave's first row needs no mask.
+    const bool tile_open = start_n + kBsBlock - 1 <= start_m * kBsBlock + wave * 16 &&
+                           start_m * kBsBlock + wave * 16 + 15 < seqlen;   // (wave-uniform)
     float m_blk = -INFINITY;
+    if (tile_open) {
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+      for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int col = start_n + nb * 16 + 4 * quarter + r;
-        const float x = (row_ok && col <= row) ? s[nb][r] * scale_log2 : -INFINITY;
-        s[nb][r] = x;
-        m_blk = fmaxf(m_blk, x);
-      }
+        for (int r = 0; r < 4; ++r) m_blk = fmaxf(m_blk, s[nb][r]);
+    } else {
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int col = start_n + nb * 16 + 4 * quarter + r;
+          const float x = (row_ok && col <= row) ? s[nb][r] : -INFINITY;
+          s[nb][r] = x;
+          m_blk = fmaxf(m_blk, x);
+        }
+    }
     m_blk = fmaxf(m_blk, bs_xor16(m_blk, quarter & 1));
     m_blk = fmaxf(m_blk, bs_xor32(m_blk, quarter & 2));
-    const float m_new = fmaxf(m_i, m_blk);
+    const float m_new = fmaxf(m_i, m_blk * scale_log2);
     // (a row with nothing visible so far keeps alpha = 1 and p = 0 instead of the
-    // NaN of exp2(-inf - -inf))
-    const float alpha = (m_new == -INFINITY) ? 1.f : exp2f(m_i - m_new);
+    // NaN of exp2(-inf - -inf); v_exp_f32 directly: its arguments are <= 0 and a
+    // result that underflows may as well be zero)
+    const bool blind = m_new == -INFINITY;
+    const float alpha = blind ? 1.f : __builtin_amdgcn_exp2f(m_i - m_new);
+    const float shift = blind ? 0.f : -m_new;
     float psum = 0.f;
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = (m_new == -INFINITY) ? 0.f : exp2f(s[nb][r] - m_new);
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nb][r], scale_log2, shift));
         s[nb][r] = p;
         psum += p;
       }
@@ -197,9 +270,10 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
       pf.w = BsType<DT>::pack2(s[2 * c + 1][2], s[2 * c + 1][3]);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const uint16_t* vrow = vt_lds + (db * 16 + prow) * kBsVtStride + 32 * c + 4 * quarter;
-        const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
-        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        const int dim = db * 16 + prow, swz = (dim >> 3) & 15;
+        const uint16_t* vrow = vt_lds + dim * kBsVtStride;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow + (((8 * c + quarter) ^ swz) << 2));
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + (((8 * c + quarter + 4) ^ swz) << 2));
         o[db] = BsType<DT>::mfma(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, o[db]);
       }
     }
