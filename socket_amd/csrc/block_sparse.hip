@@ -151,8 +151,7 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
   // Staging: thread t < 16*CH takes chunk t % CH of the four keys 4*(t / CH) .. +3 of
   // a tile.  The K chunks go to LDS as they are; the V chunks are transposed in
   // registers (two byte-selects per output word) so that the four keys of one dim
-  // leave as a single 8-byte store.  The next tile's chunks are requested before
-  // the current tile is contracted and are in registers by the time it is done.
+  // leave as a single 8-byte store.
   const bool stager = tid < 16 * CH;
   const int st_chunk = tid % CH, st_key0 = 4 * (tid / CH);
   uint4 kr[4], vr[4];
@@ -189,13 +188,28 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
     }
   };
 
-  fetch_tile(0);
+  // what of the fragment addresses does not change from tile to tile
+  const uint4* k_frag[KS];   // key row `prow`, this lane's chunk of k-step ks; key block nb adds nb*16 rows
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    k_frag[ks] = k_lds + prow * CH + (((4 * ks + quarter) & (CH - 1)) ^ (prow & (CH - 1)));
+  const uint16_t* v_row[DB];  // row of dim db*16 + prow in the transposed V tile
+  int v_grp[DB];              // element offset of 4-key group `quarter` in that row, swizzled
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+    const int dim = db * 16 + prow;
+    v_row[db] = vt_lds + dim * kBsVtStride;
+    v_grp[db] = (quarter ^ ((dim >> 3) & 15)) << 2;
+  }
+
   for (int j = 0; j < klist; ++j) {
     const int start_n = min(max(blocks[j], 0), num_cols - 1) * kBsBlock;
+    // (requested here rather than a tile ahead: holding the next tile in registers
+    // during the contraction costs a wave of occupancy per SIMD and is slower)
+    fetch_tile(j);
     __syncthreads();  // the previous tiles have been consumed
     store_tile();
     __syncthreads();
-    if (j + 1 < klist) fetch_tile(j + 1);
 
     // ---- S^T = K . Q^T: register r of block nb is key nb*16 + 4*quarter + r against row `row`
     bs_f32x4 s[4];
@@ -203,11 +217,9 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
     for (int nb = 0; nb < 4; ++nb) s[nb] = bs_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int chunk = 4 * ks + quarter;
 #pragma unroll
       for (int nb = 0; nb < 4; ++nb) {
-        const int key = nb * 16 + prow;
-        const uint4 a = chunk < CH ? k_lds[key * CH + (chunk ^ (key & (CH - 1)))] : make_uint4(0, 0, 0, 0);
+        const uint4 a = (4 * ks + quarter < CH) ? k_frag[ks][nb * 16 * CH] : make_uint4(0, 0, 0, 0);
         s[nb] = BsType<DT>::mfma(a, qf[ks], s[nb]);
       }
     }
@@ -253,12 +265,18 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
       }
     l_part = l_part * alpha + psum;
     m_i = m_new;
+    // The output accumulators are rescaled only when some row of the wave has a new
+    // maximum (alpha == 1 is the identity, so skipping it changes nothing): after the
+    // first few tiles that is rare, and the accumulators need not leave the matrix
+    // core's registers.
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      o[db][0] *= alpha;
-      o[db][1] *= alpha;
-      o[db][2] *= alpha;
-      o[db][3] *= alpha;
+      for (int db = 0; db < DB; ++db) {
+        o[db][0] *= alpha;
+        o[db][1] *= alpha;
+        o[db][2] *= alpha;
+        o[db][3] *= alpha;
+      }
     }
     // ---- O^T += V^T . P^T
 #pragma unroll
@@ -270,10 +288,9 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
       pf.w = BsType<DT>::pack2(s[2 * c + 1][2], s[2 * c + 1][3]);
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const int dim = db * 16 + prow, swz = (dim >> 3) & 15;
-        const uint16_t* vrow = vt_lds + dim * kBsVtStride;
-        const uint2 lo = *reinterpret_cast<const uint2*>(vrow + (((8 * c + quarter) ^ swz) << 2));
-        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + (((8 * c + quarter + 4) ^ swz) << 2));
+        // group (8c + quarter [+ 4]) ^ swizzle = (quarter ^ swizzle) ^ (8c [+ 4]): one xor on the lane's constant
+        const uint2 lo = *reinterpret_cast<const uint2*>(v_row[db] + (v_grp[db] ^ (32 * c)));
+        const uint2 hi = *reinterpret_cast<const uint2*>(v_row[db] + (v_grp[db] ^ (32 * c + 16)));
         o[db] = BsType<DT>::mfma(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, o[db]);
       }
     }
