@@ -25,6 +25,14 @@ FLAGS = [
 ]
 
 
+# Per-file additions.  block_sparse.hip: keep MFMA accumulators in ordinary
+# registers (its softmax reads and rescales them every tile; the default form
+# parks them in the accumulator file and moves them back and forth).
+FILE_FLAGS = {
+    "block_sparse.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -47,7 +55,7 @@ def build(verbose: bool = False, extra_flags=()) -> str:
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        out = _run([hipcc, *FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj])
+        out = _run([hipcc, *FLAGS, *FILE_FLAGS.get(src, []), *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)
         return obj

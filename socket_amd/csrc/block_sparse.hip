@@ -95,7 +95,7 @@ __device__ __forceinline__ float bs_xor32(float v, bool upper_half) {
 }
 
 template <class DT, int D>
-__global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
+__global__ __launch_bounds__(kBsThreads) __attribute__((amdgpu_waves_per_eu(4, 4))) void block_sparse_fwd_kernel(
     const uint16_t* __restrict__ q_, const uint16_t* __restrict__ k_, const uint16_t* __restrict__ v_,
     int64_t q_sb, int64_t q_sh, int64_t q_sm, int64_t k_sb, int64_t k_sh, int64_t k_sn, int64_t v_sb,
     int64_t v_sh, int64_t v_sn, const int32_t* __restrict__ seqlens, const int32_t* __restrict__ block_index,
@@ -193,14 +193,10 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
     k_frag[ks] = k_lds + prow * CH + (((4 * ks + quarter) & (CH - 1)) ^ (prow & (CH - 1)));
-  const uint16_t* v_row[DB];  // row of dim db*16 + prow in the transposed V tile
-  int v_grp[DB];              // element offset of 4-key group `quarter` in that row, swizzled
-#pragma unroll
-  for (int db = 0; db < DB; ++db) {
-    const int dim = db * 16 + prow;
-    v_row[db] = vt_lds + dim * kBsVtStride;
-    v_grp[db] = (quarter ^ ((dim >> 3) & 15)) << 2;
-  }
+  // transposed V tile: row of dim db*16 + prow is v_row0 + db*16 rows; 4-key group g of it sits at
+  // element ((g ^ (dim / 8 % 16)) * 4, and dim / 8 = 2*db + prow / 8
+  const uint16_t* v_row0 = vt_lds + prow * kBsVtStride;
+  const int v_swz0 = prow >> 3;
 
   for (int j = 0; j < klist; ++j) {
     const int start_n = min(max(blocks[j], 0), num_cols - 1) * kBsBlock;
@@ -289,8 +285,10 @@ __global__ __launch_bounds__(kBsThreads) void block_sparse_fwd_kernel(
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         // group (8c + quarter [+ 4]) ^ swizzle = (quarter ^ swizzle) ^ (8c [+ 4]): one xor on the lane's constant
-        const uint2 lo = *reinterpret_cast<const uint2*>(v_row[db] + (v_grp[db] ^ (32 * c)));
-        const uint2 hi = *reinterpret_cast<const uint2*>(v_row[db] + (v_grp[db] ^ (32 * c + 16)));
+        const uint16_t* vrow = v_row0 + db * 16 * kBsVtStride;
+        const int grp = (quarter ^ (2 * db + v_swz0)) << 2;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow + (grp ^ (32 * c)));
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + (grp ^ (32 * c + 16)));
         o[db] = BsType<DT>::mfma(make_uint4(lo.x, lo.y, hi.x, hi.y), pf, o[db]);
       }
     }
