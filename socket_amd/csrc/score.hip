@@ -20,6 +20,8 @@
 //    the copy is global_load_lds: global memory straight into LDS.
 //  * collision_i16_kernel: the reference's own operand layout (int16 codes per
 //    query head), for drop-in callers.
+#include <type_traits>
+
 #include "socket_common.h"
 
 namespace {
@@ -199,6 +201,15 @@ __device__ __forceinline__ void interleave_heads(const uint4 (&x)[GP], uint4 (&o
 // table is already in LDS from the tile this workgroup did before (single-buffer
 // launches only), so nothing is copied.  `red_off`: byte offset in LDS, past the
 // table buffers, of the small scratch area of the key-range reduction.
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order
+template <int N, int I = 0, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
+}
+
 template <int GP, class TT, int KT4, int THREADS, int PT, int MODE>
 __device__ __forceinline__ void score_tile(
     const typename TT::elem* __restrict__ q_probs, const uint32_t* __restrict__ codes,
@@ -321,7 +332,16 @@ __device__ __forceinline__ void score_tile(
     // word being consumed, ring[d] the word d steps ahead.  The code stream is the
     // HBM traffic of this kernel and a CU needs tens of KB of it in flight to cover
     // the memory latency; one word ahead (16 B x tokens/4 per lane) is not enough.
-    constexpr int kPrefetch = DMA ? 4 : 3;  // the direct-to-LDS variant has the registers for one more
+    // In the direct-to-LDS variant word w lives in slot w % kPrefetch for as long as
+    // it is needed and the word loop is unrolled by kPrefetch, so that every slot is
+    // a fixed set of registers: a ring that is shifted at the loop's back edge has
+    // its newest, still outstanding load copied there, and the copy waits for it --
+    // every word would then cost a full memory latency.
+    // (Only where the adds run on the matrix core: with plain adds the compiler
+    // lets the unrolled loop's register use run far past what a 1024-thread
+    // workgroup has.)
+    constexpr bool kFlat = DMA && GP > 1 && std::is_same<TT, TabBF16>::value;
+    constexpr int kPrefetch = kFlat ? (KT4 == 1 ? 8 : 4) : DMA ? 4 : 3;
     uint4 ring[kPrefetch][KT4];
 #pragma unroll
     for (int d = 0; d < kPrefetch; ++d)
@@ -403,6 +423,111 @@ __device__ __forceinline__ void score_tile(
       __syncthreads();
     }
 
+    if constexpr (kFlat) {
+      constexpr int EB = GP * (int)sizeof(TE);
+      constexpr int CPW = PT ? 32 / PT : 1;
+      // one word of one token group: all its tables, `d` = the word's ring slot
+      auto word_full = [&](const TE* tw, int w, auto slot) {
+        constexpr int d = decltype(slot)::value;
+        // The lookups are cut into batches of four (one table, one group of four
+        // tokens) and the LDS reads of batch k+1 are issued before batch k is
+        // accumulated, so the gather latency overlaps the adds.
+        constexpr int NB = KT4 * CPW;
+        RawEntry<EB> ent[2][4];
+        auto issue = [&](int bi, RawEntry<EB>(&dst)[4]) {
+          const int j = bi / CPW, jj = bi % CPW;
+          const uint32_t wv[4] = {ring[d][j].x, ring[d][j].y, ring[d][j].z, ring[d][j].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t code = __builtin_amdgcn_ubfe(wv[i], jj * (PT ? PT : 1), PT ? PT : 1);
+            dst[i] = load_entry<EB>(tw + (size_t)jj * R * GP + (size_t)code * GP);
+          }
+          if (jj == CPW - 1)  // last use of this group's word: its slot takes the word kPrefetch ahead
+            ring[d][j] = load_stream16(codes_pair + (int64_t)min(w + kPrefetch, NW - 1) * Tcap + tsafe[j]);
+        };
+        issue(0, ent[0]);
+#pragma unroll
+        for (int bi = 0; bi < NB; ++bi) {
+          if (bi + 1 < NB) issue(bi + 1, ent[(bi + 1) & 1]);
+          const int j = bi / CPW;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) accumulate<GP>(acc[j][i], ent[bi & 1][i], (const TT*)nullptr, sel);
+        }
+      };
+      // a word with fewer real tables than it has room for (the last one), or a
+      // code width that is not a template constant
+      auto word_any = [&](const TE* tw, int w, int ntw, auto slot) {
+        constexpr int d = decltype(slot)::value;
+#pragma unroll
+        for (int j = 0; j < KT4; ++j) {
+          const uint32_t wv[4] = {ring[d][j].x, ring[d][j].y, ring[d][j].z, ring[d][j].w};
+          for (int jj = 0; jj < ntw; ++jj) {
+            const TE* tb = tw + (size_t)jj * R * GP;
+            const int sh = jj * P;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const uint32_t code = (wv[i] >> sh) & code_mask;
+              accumulate<GP>(acc[j][i], load_entry<EB>(tb + (size_t)code * GP), (const TT*)nullptr, sel);
+            }
+          }
+          ring[d][j] = load_stream16(codes_pair + (int64_t)min(w + kPrefetch, NW - 1) * Tcap + tsafe[j]);
+        }
+      };
+
+      int w0 = 0, wend = min(chunk_words, NW), buf = 0;
+      if (wend < NW) dma_slice(wend * cpw, 1);
+      // One word: the slice switch if the word opens a slice, then its lookups.
+      // `full`: the word holds CPW real tables (straight-line body).
+      auto word = [&](int w, auto slot, auto full) {
+        if (w == wend) {
+          // The copies of the slice that starts here were issued at the top of the
+          // one that ends; since then this wave has issued one code load per word
+          // and token group.  Loads retire in order, so allowing that many to be
+          // outstanding, less one word's worth as a margin, means the copies have
+          // landed.
+          wait_vmcnt(max(0, (wend - w0 - 1) * KT4));
+          __syncthreads();
+          if (nbuf == 2) buf ^= 1;
+          w0 = w;
+          wend = min(w + chunk_words, NW);
+          if (wend < NW) dma_slice(wend * cpw, buf ^ 1);
+        }
+        const TE* tw =
+            reinterpret_cast<const TE*>(lds_raw) + (size_t)buf * chunk_elems + (size_t)(w - w0) * cpw * R * GP;
+        if constexpr (decltype(full)::value) word_full(tw, w, slot);
+        else word_any(tw, w, min(cpw, L - w * cpw), slot);
+        // keep the words apart: left alone, the scheduler hoists the gathers of later
+        // words over the adds of earlier ones until the registers run out
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      // Words [0, wlimit).  Whole rounds of the ring run without a test per word: a
+      // path on which some slots are skipped would make the compiler assume, where a
+      // slot is consumed, that its load may be the newest one outstanding, and wait
+      // for everything.  The two bodies are never mixed in one loop either: the two
+      // definitions of a slot's next word would end up in different registers and be
+      // copied at the join, and the copy of an outstanding load waits for it.
+      auto run = [&](int wlimit, auto full) {
+        int wb = 0;
+        for (; wb + kPrefetch <= wlimit; wb += kPrefetch)
+          static_for<kPrefetch>([&](auto slot) { word(wb + decltype(slot)::value, slot, full); });
+        static_for<kPrefetch>([&](auto slot) {
+          const int w = wb + decltype(slot)::value;
+          if (w < wlimit) word(w, slot, full);
+        });
+      };
+      if constexpr (PT != 0) {
+        const int nfull = min(NW, L / CPW);  // all but possibly the last word
+        run(nfull, std::true_type{});
+        if (nfull < NW)
+          static_for<kPrefetch>([&](auto slot) {
+            if (nfull % kPrefetch == decltype(slot)::value) word(nfull, slot, std::false_type{});
+          });
+      } else {
+        run(NW, std::false_type{});
+      }
+      wait_vmcnt(0);
+      __syncthreads();
+    } else {
     int chunk = 0;
     for (int w0 = 0; w0 < NW; w0 += chunk_words, ++chunk) {
       const int l0 = w0 * cpw;
@@ -497,6 +622,7 @@ __device__ __forceinline__ void score_tile(
         __syncthreads();
       }
     }
+    }  // staged / in-place variants
 
   }
 
@@ -721,10 +847,12 @@ struct ScorePlan {
 
 // Launch shapes and what they cost (microseconds measured at L60 x P10 bf16
 // tables on this GPU; only their ratios are used, to choose between shapes):
-//  * grouped / direct: 8192-token tiles, G heads per gather, table slices copied
-//    global -> LDS: ~53 per round of workgroups on a full chip, ~44 when the
+//  * grouped / direct: G heads per gather, table slices copied global -> LDS.
+//    8192-token tiles: ~53 per round of workgroups on a full chip, ~40 when the
 //    workgroups cover only part of it (a workgroup's time hardly depends on how
-//    many others there are);
+//    many others there are); 4096 / 2048 / 1024-token tiles (16-bit entries):
+//    ~29 / 20 / 20 per round -- every workgroup pulls the whole table through LDS,
+//    so small tiles pay off only while they add CUs, not rounds;
 //  * slices staged through registers: 8192-token tiles ~57 per round (~50 on a part
 //    of the chip, ~73 with 32-bit entries); smaller tiles
 //    (4096 / 2048 / 1024, chosen so that every CU has a workgroup) ~45 per round
@@ -754,7 +882,21 @@ ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_ele
       break;
     }
   if (grouped) {
-    if (slices_fit_twice) return {1024 * 4 * kDmaKT4, true, false, big >= lim.cu_count ? 53.f * rounds(big) : 44.f};
+    if (slices_fit_twice) {
+      ScorePlan best = {1024 * 4 * kDmaKT4, true, false, big >= lim.cu_count ? 53.f * rounds(big) : 40.f};
+      if (table_elem_bytes == 2) {
+        // smaller tiles (16-bit entries: the variants whose code prefetch runs ahead):
+        // a round of them on a full chip / on a part of it
+        const int tw[3] = {4096, 2048, 1024};
+        const float full[3] = {29.f, 20.f, 20.f}, part[3] = {25.f, 19.f, 20.f};
+        for (int i = 0; i < 3; ++i) {
+          const int64_t wgs = pairs * tiles(tw[i]);
+          const float cost = wgs >= lim.cu_count ? full[i] * rounds(wgs) : part[i];
+          if (cost < best.cost) best = {tw[i], true, false, cost};
+        }
+      }
+      return best;
+    }
     return staged;
   }
   ScorePlan best = staged;
@@ -779,12 +921,9 @@ template <int GP, class TT>
 int dispatch_tile(const ScoreArgs& a, const ScorePlan& plan) {
   if (plan.dma) {
     if (plan.tile == 8192) return dispatch_p<GP, TT, 2, 1024, 2>(a);
-    if (GP == 1) {
-      if (plan.tile == 4096) return dispatch_p<1, TT, 1, 1024, 2>(a);
-      if (plan.tile == 2048) return dispatch_p<1, TT, 1, 512, 2>(a);
-      return dispatch_p<1, TT, 1, 256, 2>(a);
-    }
-    return SOCKET_ERR_UNSUPPORTED;
+    if (plan.tile == 4096) return dispatch_p<GP, TT, 1, 1024, 2>(a);
+    if (plan.tile == 2048) return dispatch_p<GP, TT, 1, 512, 2>(a);
+    return dispatch_p<GP, TT, 1, 256, 2>(a);
   }
   if (plan.tile == 8192) return dispatch_layout<GP, TT, 2, 1024>(a);
   if (plan.tile == 4096) return dispatch_layout<GP, TT, 2, 512>(a);

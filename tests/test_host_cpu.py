@@ -102,11 +102,14 @@ def test_sizes_helpers(lib):
     assert lib.socket_score_range_parts_grouped(4, 32, 8, 131072, 1, 60, 10, 1024) == 16
     assert lib.socket_score_range_parts(1, 5, 2, 100, 1, 60, 10, 1024) == 0
     # which table layout a producer should write (bf16 entries, L60 x P10): the grouped
-    # one wherever its 8192-token tiles are at least as cheap as one head per workgroup
+    # one wherever its tiles are at least as cheap as one head per workgroup
     assert lib.socket_score_prefers_grouped(4, 32, 8, 131072, 1, 60, 10, 1024) == 1    # full chip, two rounds
     assert lib.socket_score_prefers_grouped(1, 32, 8, 131072, 1, 60, 10, 1024) == 1    # half the chip, still cheaper
-    assert lib.socket_score_prefers_grouped(1, 32, 8, 65536, 1, 60, 10, 1024) == 0     # one round of one-head workgroups
-    assert lib.socket_score_prefers_grouped(1, 32, 8, 32768, 1, 60, 10, 1024) == 0
+    assert lib.socket_score_prefers_grouped(1, 32, 8, 65536, 1, 60, 10, 1024) == 1     # one round of 2048-token tiles
+    assert lib.socket_score_prefers_grouped(1, 32, 8, 32768, 1, 60, 10, 1024) == 1
+    assert lib.socket_score_range_parts_grouped(1, 32, 8, 131072, 1, 60, 10, 1024) == 32   # 4096-token tiles fill the chip
+    assert lib.socket_score_range_parts_grouped(1, 32, 8, 65536, 1, 60, 10, 1024) == 32    # 2048-token tiles
+    assert lib.socket_score_range_parts_grouped(1, 32, 8, 65536, 0, 60, 10, 1024) == 8     # fp32 entries stay at 8192
     assert lib.socket_score_prefers_grouped(1, 32, 8, 65536, 0, 60, 10, 1024) == 1     # fp32: a head's table exceeds LDS
     assert lib.socket_score_prefers_grouped(1, 5, 2, 100, 1, 60, 10, 1024) == -1
 
