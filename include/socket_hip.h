@@ -335,6 +335,16 @@ int socket_add_rmsnorm(const void* x, const void* residual, const void* weight, 
 /* out = round(silu(a)) * b elementwise over n elements (FeedForward, GPT-FAST/model.py:599-600). */
 int socket_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n, void* stream);
 
+/* y[m,n] = sum_k x[m,k] * w[n,k]: the linear layers of a single-token step as matrix-vector
+ * products (M <= 4 rows, bf16, fp32 accumulation; K a multiple of 2048; x rows `x_stride`
+ * elements apart, y rows `y_stride`; w [N,K] contiguous).  With w_gate (another [N,K]):
+ * y = round(silu(round(x.w[n]))) * round(x.w_gate[n]), i.e. w1, w3 and the product of
+ * FeedForward in one pass.  Replaces the nn.Linear calls of a decode step
+ * (GPT-FAST/model.py:436, :476, :599-600); SOCKET_ERR_UNSUPPORTED tells the caller to use its
+ * own matrix product. */
+int socket_gemv_bf16(const void* x, int64_t x_stride, const void* w, const void* w_gate, void* y,
+                     int64_t y_stride, int M, int N, int K, void* stream);
+
 /* Block-sparse prefill attention: out[b,h,row,:] = softmax over the listed key
  * blocks (causal inside them) of q.k^T / sqrt(D), times v.  q, k, v, out are
  * [B,H,T,D] views (element strides for dims 0-2, last dim contiguous), bf16 or

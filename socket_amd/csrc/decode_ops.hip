@@ -219,6 +219,85 @@ __global__ void silu_mul_kernel(const void* __restrict__ a, const void* __restri
   }
 }
 
+
+// y[m,n] = sum_k x[m,k] * w[n,k] for a handful of rows m (a decode step's linear
+// layers are matrix-vector products: the weight matrix is streamed once, HBM bound).
+// One wave per output feature n: 16 bytes of the weight row per lane and step,
+// four steps in flight, fp32 accumulation, a butterfly over the lanes at the end.
+// GATE: two weight matrices, y = round(silu(round(x.w[n]))) * round(x.wg[n]) -- the
+// roundings of the three torch ops this replaces.
+constexpr int kGemvThreads = 256;
+constexpr int kGemvUnroll = 4;
+constexpr int kGemvStep = 64 * 8;  // elements of a row per wave and step
+
+template <int M, bool GATE>
+__global__ __launch_bounds__(kGemvThreads) void gemv_bf16_kernel(
+    const uint16_t* __restrict__ x, int64_t x_stride, const uint16_t* __restrict__ w,
+    const uint16_t* __restrict__ wg, uint16_t* __restrict__ y, int64_t y_stride, int N, int K) {
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x * (kGemvThreads / 64) + wave;
+  if (n >= N) return;
+  const uint16_t* wr = w + (int64_t)n * K;
+  const uint16_t* gr = GATE ? wg + (int64_t)n * K : nullptr;
+  float acc[M], accg[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) acc[m] = accg[m] = 0.f;
+  for (int k0 = lane * 8; k0 < K; k0 += kGemvStep * kGemvUnroll) {  // K is a multiple of the unrolled step
+    u32x4 wv[kGemvUnroll], gv[kGemvUnroll];
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      wv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wr + k0 + u * kGemvStep));
+      if (GATE) gv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(gr + k0 + u * kGemvStep));
+    }
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const uint4 xv = *reinterpret_cast<const uint4*>(x + (int64_t)m * x_stride + k0 + u * kGemvStep);
+        const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float x0 = __uint_as_float(xw[i] << 16), x1 = __uint_as_float(xw[i] & 0xffff0000u);
+          acc[m] = fmaf(__uint_as_float(wv[u][i] << 16), x0, acc[m]);
+          acc[m] = fmaf(__uint_as_float(wv[u][i] & 0xffff0000u), x1, acc[m]);
+          if (GATE) {
+            accg[m] = fmaf(__uint_as_float(gv[u][i] << 16), x0, accg[m]);
+            accg[m] = fmaf(__uint_as_float(gv[u][i] & 0xffff0000u), x1, accg[m]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+      acc[m] += __shfl_xor(acc[m], d, 64);
+      if (GATE) accg[m] += __shfl_xor(accg[m], d, 64);
+    }
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      float r = acc[m];
+      if (GATE) {
+        const float a = rnd<DType_bf16>(acc[m]);
+        r = rnd<DType_bf16>(a / (1.f + expf(-a))) * rnd<DType_bf16>(accg[m]);
+      }
+      y[(int64_t)m * y_stride + n] = f32_to_bf16_bits(r);
+    }
+  }
+}
+
+template <int M>
+void launch_gemv(const uint16_t* x, int64_t xs, const uint16_t* w, const uint16_t* wg, uint16_t* y, int64_t ys, int N,
+                 int K, hipStream_t s) {
+  const dim3 grid((unsigned)((N + kGemvThreads / 64 - 1) / (kGemvThreads / 64))), block(kGemvThreads);
+  if (wg) hipLaunchKernelGGL((gemv_bf16_kernel<M, true>), grid, block, 0, s, x, xs, w, wg, y, ys, N, K);
+  else hipLaunchKernelGGL((gemv_bf16_kernel<M, false>), grid, block, 0, s, x, xs, w, wg, y, ys, N, K);
+}
+
 }  // namespace
 
 extern "C" int socket_rope_append(const void* qkv, int dtype, int64_t qkv_stride_b, const void* freqs_cis,
@@ -286,6 +365,28 @@ extern "C" int socket_silu_mul(const void* a, const void* b, void* out, int dtyp
   if (dtype == SOCKET_F32) hipLaunchKernelGGL((silu_mul_kernel<DType_f32>), grid, block, 0, s, a, b, out, n, vec_ok);
   else if (dtype == SOCKET_BF16) hipLaunchKernelGGL((silu_mul_kernel<DType_bf16>), grid, block, 0, s, a, b, out, n, vec_ok);
   else hipLaunchKernelGGL((silu_mul_kernel<DType_f16>), grid, block, 0, s, a, b, out, n, vec_ok);
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}
+
+extern "C" int socket_gemv_bf16(const void* x, int64_t x_stride, const void* w, const void* w_gate, void* y,
+                                int64_t y_stride, int M, int N, int K, void* stream) {
+  SOCKET_REQUIRE(x && w && y, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(M >= 1 && N >= 1 && K >= 1 && x_stride >= K && y_stride >= N, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(M <= 4 && K % (kGemvStep * kGemvUnroll) == 0, SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(socket_aligned16(x) && socket_aligned16(w) && (!w_gate || socket_aligned16(w_gate)) && x_stride % 8 == 0,
+                 SOCKET_ERR_ALIGN);
+  hipStream_t s = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* wp = (const uint16_t*)w;
+  const uint16_t* gp = (const uint16_t*)w_gate;
+  uint16_t* yp = (uint16_t*)y;
+  switch (M) {
+    case 1: launch_gemv<1>(xp, x_stride, wp, gp, yp, y_stride, N, K, s); break;
+    case 2: launch_gemv<2>(xp, x_stride, wp, gp, yp, y_stride, N, K, s); break;
+    case 3: launch_gemv<3>(xp, x_stride, wp, gp, yp, y_stride, N, K, s); break;
+    default: launch_gemv<4>(xp, x_stride, wp, gp, yp, y_stride, N, K, s); break;
+  }
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }

@@ -72,3 +72,26 @@ def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     check("socket_silu_mul", lib().socket_silu_mul(ptr(a), ptr(b), ptr(out), dtype_enum(a.dtype), a.numel(),
                                                    stream_ptr(a.device)))
     return out
+
+
+@torch.no_grad()
+def linear_rows(x: torch.Tensor, weight: torch.Tensor, gate_weight: torch.Tensor = None) -> torch.Tensor:
+    """x @ weight.T for the few rows of a decode step (nn.Linear without bias,
+    GPT-FAST/model.py:436, :476), or with `gate_weight` silu(x @ weight.T) * (x @ gate_weight.T)
+    (FeedForward, :599-600) in one pass over both matrices.  Shapes the
+    matrix-vector kernel does not take go to torch's own product."""
+    rows = x.numel() // x.shape[-1]
+    K, N = x.shape[-1], weight.shape[0]
+    # measured against torch's product: ahead for one row (and, gated, up to four); behind for more
+    fits = (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+            and rows <= (1 if gate_weight is None else 4)
+            and K % 2048 == 0 and weight.is_contiguous() and x.is_contiguous()
+            and (gate_weight is None or (gate_weight.is_contiguous() and gate_weight.shape == weight.shape
+                                         and gate_weight.dtype == torch.bfloat16)))
+    if not fits:
+        y = torch.nn.functional.linear(x, weight)
+        return y if gate_weight is None else silu_mul(y, torch.nn.functional.linear(x, gate_weight))
+    y = torch.empty(*x.shape[:-1], N, dtype=x.dtype, device=x.device)
+    check("socket_gemv_bf16", lib().socket_gemv_bf16(ptr(x), K, ptr(weight), ptr(gate_weight),
+                                                     ptr(y), N, rows, N, K, stream_ptr(x.device)))
+    return y

@@ -276,7 +276,8 @@ class Transformer(nn.Module):
             ffn = None
             for layer in self.layers:
                 x, ffn = layer._run_fused(x, ffn, input_pos, sparse, step)
-            return self.output(decode_ops.add_rmsnorm(x, self.norm.weight, self.norm.eps, residual=ffn)[1])
+            return decode_ops.linear_rows(decode_ops.add_rmsnorm(x, self.norm.weight, self.norm.eps, residual=ffn)[1],
+                                          self.output.weight)
         freqs_cis = self.freqs_cis[input_pos]
         for layer in self.layers:
             x = layer._run(x, input_pos, freqs_cis, sparse, pos0)
@@ -320,7 +321,7 @@ class TransformerBlock(nn.Module):
         x, y = decode_ops.add_rmsnorm(x, an.weight, an.eps, residual=pending)
         a = self.attention._run_fused(y, input_pos, sparse, step)
         h, y = decode_ops.add_rmsnorm(x, fn.weight, fn.eps, residual=a)
-        return h, ff.w2(decode_ops.silu_mul(ff.w1(y), ff.w3(y)))
+        return h, decode_ops.linear_rows(decode_ops.linear_rows(y, ff.w1.weight, ff.w3.weight), ff.w2.weight)
 
     def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Tensor = None) -> Tensor:
         return self._run(x, input_pos, freqs_cis, False, None)
@@ -433,7 +434,7 @@ class Attention(nn.Module):
         update in one launch (same values)."""
         bsz = x.shape[0]
         cache = self.kv_cache
-        qkv = self.wqkv(x)
+        qkv = decode_ops.linear_rows(x, self.wqkv.weight)
         if sparse:
             q_bhd, k_new, v_new = decode_ops.rope_append(qkv, step.freqs_table, input_pos, cache.k_cache,
                                                          cache.v_cache, cache.lens, self.n_head,
@@ -447,7 +448,7 @@ class Attention(nn.Module):
             q_bhd = decode_ops.rope_append(qkv, step.freqs_table, input_pos, cache.k_cache, cache.v_cache,
                                            cache.lens, self.n_head, self.n_local_heads)
             out_bhd = _dense_step(q_bhd, cache)
-        return self.wo(out_bhd.reshape(bsz, 1, self.dim))
+        return decode_ops.linear_rows(out_bhd.reshape(bsz, 1, self.dim), self.wo.weight)
 
     def _prefill_attention(self, q, k, v, input_pos, pos0) -> Tensor:
         """Causal attention of a block of new tokens over the cache prefix and

@@ -225,6 +225,34 @@ def test_add_rmsnorm_and_silu_mul_equal_the_torch_chain(dev, dtype, tol):
         assert float((got != want).float().mean()) <= few
 
 
+@pytest.mark.parametrize("rows,N,K", [(1, 6144, 4096), (1, 4096, 14336), (4, 1000, 2048), (3, 4099, 4096), (2, 128256, 4096)])
+def test_linear_rows_equals_the_fp32_product_rounded_once(dev, rows, N, K):
+    """The matrix-vector kernel against the float64 product: within one bf16
+    rounding of it (torch's own bf16 linear is held to the same bar here), and the
+    gated form against the chain of three torch ops."""
+    from socket_amd import decode_ops
+    g = torch.Generator().manual_seed(N + K + rows)
+    x = torch.randn(rows, 1, K, generator=g).to(torch.bfloat16).to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    got = decode_ops.linear_rows(x, w)
+    assert got.shape == (rows, 1, N) and got.dtype == torch.bfloat16
+    exact = x.double() @ w.double().T
+    scale = float(exact.abs().max())
+    ulp = 2.0 ** -8                                                     # half a bf16 ulp relative, plus summation noise
+    assert float((got.double() - exact).abs().max()) <= 1.5 * ulp * scale
+    theirs = torch.nn.functional.linear(x, w)
+    assert float((theirs.double() - exact).abs().max()) <= 1.5 * ulp * scale
+    assert float((got != theirs).float().mean()) <= 0.1                 # last-bit differences only, and few
+    if N <= 8192:
+        wg = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+        gated = decode_ops.linear_rows(x, w, wg)
+        want = torch.nn.functional.silu(torch.nn.functional.linear(x, w)) * torch.nn.functional.linear(x, wg)
+        assert float((gated.float() - want.float()).abs().max()) <= 3e-2 * float(want.float().abs().max())
+    # shapes outside the kernel's range take torch's product
+    x5 = torch.randn(5, 1, K, generator=g).to(torch.bfloat16).to(dev)
+    assert torch.equal(decode_ops.linear_rows(x5, w), torch.nn.functional.linear(x5, w))
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
 @pytest.mark.parametrize("sparse", [True, False])
 def test_fused_decode_step_equals_the_plain_one(dev, dtype, tol, sparse):
