@@ -115,6 +115,18 @@ def copy_ceiling_gbs(dev):
     return 2 * n * 4 / us / 1e3
 
 
+def read_ceiling_gbs(dev):
+    """Measured rate of a pure read stream: the matrix-vector kernel over a 1 GiB
+    bf16 matrix (non-temporal 16-byte loads, 8 KB per output feature, 262 KB written)."""
+    from socket_amd import decode_ops
+    n_out, k = 131072, 4096
+    w_ = torch.empty(n_out, k, dtype=torch.bfloat16, device=dev).normal_(0, 0.02)
+    x = torch.empty(1, 1, k, dtype=torch.bfloat16, device=dev).normal_()
+    us = time_launches(lambda: decode_ops.linear_rows(x, w_), 10)
+    del w_, x
+    return n_out * k * 2 / us / 1e3
+
+
 def cpu_baseline(w, inp_cpu, codes_cpu, vnorm_cpu, seconds_budget=20.0):
     """The CPU oracle on a slice of the workload: sequence 0, the first two kv
     heads (2*G query heads), full context; scaled to the whole layer."""
@@ -417,6 +429,7 @@ def main():
         replay_ok = bool(torch.equal(out_graph, out_eager))
 
     ceiling = copy_ceiling_gbs(dev)
+    read_ceiling = read_ceiling_gbs(dev)
 
     result = {
         "metric": "sparse-attn us/layer/step at 128k ctx (score+select+attend+hash-append), % of HBM peak"
@@ -451,6 +464,7 @@ def main():
                          "attend_block_seq": None},
         "hash_prefill": hash_report,
         "copy_ceiling_gbs": round(ceiling, 1),
+        "read_ceiling_gbs": round(read_ceiling, 1),
         "parity": parity,
         "graph_replay_equals_eager": replay_ok,
         "wall_ms_timed_region": round(wall_ms, 2),
