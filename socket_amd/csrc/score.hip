@@ -339,9 +339,10 @@ __device__ __forceinline__ void score_tile(
     // every word would then cost a full memory latency.
     // (Only where the adds run on the matrix core: with plain adds the compiler
     // lets the unrolled loop's register use run far past what a 1024-thread
-    // workgroup has.)
-    constexpr bool kFlat = DMA && GP > 1 && std::is_same<TT, TabBF16>::value;
-    constexpr int kPrefetch = kFlat ? (KT4 == 1 ? 8 : 4) : DMA ? 4 : 3;
+    // workgroup has.  There it serves the direct copies and the double-buffered
+    // register staging alike.)
+    constexpr bool kFlat = GP > 1 && std::is_same<TT, TabBF16>::value;
+    constexpr int kPrefetch = kFlat ? (DMA ? (KT4 == 1 ? 8 : 4) : 3) : DMA ? 4 : 3;
     uint4 ring[kPrefetch][KT4];
 #pragma unroll
     for (int d = 0; d < kPrefetch; ++d)
@@ -423,7 +424,9 @@ __device__ __forceinline__ void score_tile(
       __syncthreads();
     }
 
-    if constexpr (kFlat) {
+    bool flat_done = false;
+    if constexpr (kFlat) if (DMA || staged) {
+      flat_done = true;
       constexpr int EB = GP * (int)sizeof(TE);
       constexpr int CPW = PT ? 32 / PT : 1;
       // one word of one token group: all its tables, `d` = the word's ring slot
@@ -475,7 +478,10 @@ __device__ __forceinline__ void score_tile(
       };
 
       int w0 = 0, wend = min(chunk_words, NW), buf = 0;
-      if (wend < NW) dma_slice(wend * cpw, 1);
+      if (wend < NW) {
+        if (DMA) dma_slice(wend * cpw, 1);
+        else stage_load(wend * cpw);
+      }
       // One word: the slice switch if the word opens a slice, then its lookups.
       // `full`: the word holds CPW real tables (straight-line body).
       auto word = [&](int w, auto slot, auto full) {
@@ -485,12 +491,16 @@ __device__ __forceinline__ void score_tile(
           // and token group.  Loads retire in order, so allowing that many to be
           // outstanding, less one word's worth as a margin, means the copies have
           // landed.
-          wait_vmcnt(max(0, (wend - w0 - 1) * KT4));
+          if (DMA) wait_vmcnt(max(0, (wend - w0 - 1) * KT4));
+          else stage_store(w * cpw, buf ^ 1);  // the slice fetched into registers while the last one was read
           __syncthreads();
           if (nbuf == 2) buf ^= 1;
           w0 = w;
           wend = min(w + chunk_words, NW);
-          if (wend < NW) dma_slice(wend * cpw, buf ^ 1);
+          if (wend < NW) {
+            if (DMA) dma_slice(wend * cpw, buf ^ 1);
+            else stage_load(wend * cpw);
+          }
         }
         const TE* tw =
             reinterpret_cast<const TE*>(lds_raw) + (size_t)buf * chunk_elems + (size_t)(w - w0) * cpw * R * GP;
@@ -525,9 +535,10 @@ __device__ __forceinline__ void score_tile(
       } else {
         run(NW, std::false_type{});
       }
-      wait_vmcnt(0);
+      if (DMA) wait_vmcnt(0);
       __syncthreads();
-    } else {
+    }
+    if (!flat_done) {
     int chunk = 0;
     for (int w0 = 0; w0 < NW; w0 += chunk_words, ++chunk) {
       const int l0 = w0 * cpw;
