@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SOCKET_ABI_VERSION 1
+#define SOCKET_ABI_VERSION 2
 
 /* status codes */
 #define SOCKET_OK 0
@@ -248,6 +248,7 @@ int socket_select_list(const float* scores, int64_t score_stride, const int32_t*
  * mid_lse[b,h,s] = max + log(sum_exp) (fp32 [B,Hq,nsplit]); a split with no
  * live row gets mid_lse = -inf, mid_o = 0; splits at or beyond len are left
  * untouched.  Strides are in elements; the last dim of q, k, v is contiguous.
+ * list_width: entries in a row of sparse_list; a length beyond it is cut to it.
  * Replaces sparse_decode_stage1, kernels/socket_triton_kernels.py:167-205
  * (kernel :31-118).  D in {16,32,64,128}; q,k,v of one dtype. */
 int socket_attend_stage1(const void* q, const void* k, const void* v, int dtype,
@@ -257,8 +258,8 @@ int socket_attend_stage1(const void* q, const void* k, const void* v, int dtype,
                          const int32_t* sparse_list, int64_t list_stride_b, int64_t list_stride_h,
                          const int32_t* sparse_len, int64_t len_stride_b, int64_t len_stride_h,
                          float* mid_o, float* mid_lse,
-                         int B, int Hq, int Hkv, int D, int kv_rows, int nsplit, int block_seq,
-                         void* stream);
+                         int B, int Hq, int Hkv, int D, int kv_rows, int list_width, int nsplit,
+                         int block_seq, void* stream);
 
 /* Stage 2: merge the ceil(len / block_seq) splits of every (b,h) into
  * out[b,h,:] (out_dtype); len == 0 gives NaN like the reference's 0/0.
@@ -310,7 +311,8 @@ int socket_dense_decode(const void* q, const void* k, const void* v, int dtype,
  * cache, from the fused projection qkv [B, (Hq + 2*Hkv) * D] (row stride
  * qkv_stride_b): q_out [B,Hq,D] contiguous; rotated k and v are written at
  * row pos of k_cache / v_cache (element strides b, h, s; unit-stride last dim),
- * and lens[b] (may be NULL) is raised to pos + 1.  pos: int64 on the device,
+ * and lens[b] (may be NULL) is set to pos + 1 (the cached length follows the
+ * position, as the reference's mask arange(T) <= pos does, GPT-FAST/model.py:486-487).  pos: int64 on the device,
  * one for all sequences (pos_stride 0) or one each (pos_stride 1); a position
  * outside [0, min(Tcap, n_pos)) writes nothing.  freqs_cis [n_pos, D/2, 2] holds
  * (cos, sin) in bf16 or f32.  k_new / v_new (may be NULL): [B,Hkv,D] contiguous

@@ -62,7 +62,7 @@ SIGNATURES = {
     "socket_gemv_bf16": (_I, [_P, _L, _P, _P, _P, _L, _I, _I, _I, _P]),
     "socket_attend_stage1": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L,
                                   _P, _L, _L, _P, _L, _L, _P, _P,
-                                  _I, _I, _I, _I, _I, _I, _I, _P]),
+                                  _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "socket_attend_stage2": (_I, [_P, _P, _P, _L, _L, _P, _I, _L, _L, _I, _I, _I, _I, _I, _P]),
     "socket_sparse_attention_block_seq": (_I, [_I, _I, _I]),
     "socket_sparse_attention_workspace_bytes": (_Z, [_I, _I, _I, _I]),
@@ -100,7 +100,7 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.socket_abi_version() != 1:
+        if handle.socket_abi_version() != 2:
             raise RuntimeError("libsocket_hip.so ABI version mismatch; rebuild it")
         _lib = handle
     return _lib

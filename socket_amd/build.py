@@ -48,13 +48,26 @@ def _run(cmd):
     return "\n".join(lines)
 
 
-def build(verbose: bool = False, extra_flags=()) -> str:
+def _stale(src_path: str, obj: str) -> bool:
+    """True if the object is older than its source or any header beside it."""
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [src_path, os.path.join(CSRC, "socket_common.h"), os.path.join(HERE, "..", "include", "socket_hip.h")]
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(verbose: bool = False, extra_flags=(), only_changed: bool = False) -> str:
+    """Compile every source (or, with only_changed, those newer than their
+    object) and link the library."""
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        if only_changed and not _stale(os.path.join(CSRC, src), obj):
+            return obj
         out = _run([hipcc, *FLAGS, *FILE_FLAGS.get(src, []), *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)
@@ -69,4 +82,4 @@ def build(verbose: bool = False, extra_flags=()) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose="-v" in sys.argv))
+    print(build(verbose="-v" in sys.argv, only_changed="--changed" in sys.argv))

@@ -102,8 +102,8 @@ __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
     int64_t q_sb, int64_t q_sh, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb,
     int64_t v_sh, int64_t v_ss, const int32_t* __restrict__ sparse_list, int64_t list_sb,
     int64_t list_sh, const int32_t* __restrict__ sparse_len, int64_t len_sb, int64_t len_sh,
-    float* __restrict__ mid_o, float* __restrict__ mid_lse, int Hq, int G, int kv_rows, int nsplit,
-    int block_seq, float sm_scale) {
+    float* __restrict__ mid_o, float* __restrict__ mid_lse, int Hq, int G, int kv_rows, int list_width,
+    int nsplit, int block_seq, float sm_scale) {
   typedef typename DT::storage ST;
   constexpr int E = DT::kPer16B;
   constexpr int LPR = D / E;
@@ -111,7 +111,8 @@ __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
   __shared__ float lds[kAttWaves * (D + 2)];
 
   const int s = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int len = sparse_len[b * len_sb + h * len_sh];
+  // a length beyond the list row's width would read the next row's entries
+  const int len = min(sparse_len[b * len_sb + h * len_sh], list_width);
   const int lo = s * block_seq;
   const int hi = min(len, lo + block_seq);
   if (hi <= lo) return;
@@ -198,6 +199,7 @@ __global__ __launch_bounds__(kMergeThreads) void stage2_kernel(
     const float* __restrict__ mid_o, const float* __restrict__ mid_lse,
     const int32_t* __restrict__ sparse_len, int64_t len_sb, int64_t len_sh, void* __restrict__ out,
     int out_dtype, int64_t out_sb, int64_t out_sh, int Hq, int nsplit, int block_seq) {
+  // (a length beyond nsplit * block_seq is cut to the splits that exist, below)
   constexpr int LPD = D / 4;                    // lanes across the head dimension
   constexpr int NG = kMergeThreads / LPD;       // splits handled side by side
   constexpr int kW = kMergeThreads / SOCKET_WAVE;
@@ -392,12 +394,12 @@ int check_common(const AttArgs& a, int B, int Hq, int Hkv, int D) {
 template <class DT, int D>
 void launch_sparse_stage1(const AttArgs& a, const int32_t* list, int64_t list_sb, int64_t list_sh,
                           const int32_t* len, int64_t len_sb, int64_t len_sh, float* mid_o,
-                          float* mid_lse, int B, int Hq, int Hkv, int kv_rows, int nsplit,
-                          int block_seq, hipStream_t s) {
+                          float* mid_lse, int B, int Hq, int Hkv, int kv_rows, int list_width,
+                          int nsplit, int block_seq, hipStream_t s) {
   hipLaunchKernelGGL((sparse_stage1_kernel<DT, D>), dim3(nsplit, Hq, B), dim3(kAttThreads), 0, s,
                      a.q, a.k, a.v, a.q_sb, a.q_sh, a.k_sb, a.k_sh, a.k_ss, a.v_sb, a.v_sh, a.v_ss,
                      list, list_sb, list_sh, len, len_sb, len_sh, mid_o, mid_lse, Hq, Hq / Hkv,
-                     kv_rows, nsplit, block_seq, 1.0f / sqrtf((float)D));
+                     kv_rows, list_width, nsplit, block_seq, 1.0f / sqrtf((float)D));
 }
 
 template <class DT, int D>
@@ -456,18 +458,19 @@ extern "C" int socket_attend_stage1(const void* q, const void* k, const void* v,
                                     int64_t list_stride_h, const int32_t* sparse_len,
                                     int64_t len_stride_b, int64_t len_stride_h, float* mid_o,
                                     float* mid_lse, int B, int Hq, int Hkv, int D, int kv_rows,
-                                    int nsplit, int block_seq, void* stream) {
+                                    int list_width, int nsplit, int block_seq, void* stream) {
   AttArgs a{q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h, k_stride_s,
             v_stride_b, v_stride_h, v_stride_s};
   int st = check_common(a, B, Hq, Hkv, D);
   if (st != SOCKET_OK) return st;
   SOCKET_REQUIRE(sparse_list && sparse_len && mid_o && mid_lse, SOCKET_ERR_NULL);
-  SOCKET_REQUIRE(nsplit > 0 && nsplit <= 65535 * 32 && block_seq > 0 && kv_rows > 0, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(nsplit > 0 && nsplit <= 65535 * 32 && block_seq > 0 && kv_rows > 0 && list_width > 0,
+                 SOCKET_ERR_SHAPE);
   hipStream_t s = (hipStream_t)stream;
 #define SOCKET_S1(DT, DD)                                                                          \
   launch_sparse_stage1<DT, DD>(a, sparse_list, list_stride_b, list_stride_h, sparse_len,           \
                                len_stride_b, len_stride_h, mid_o, mid_lse, B, Hq, Hkv, kv_rows,    \
-                               nsplit, block_seq, s)
+                               list_width, nsplit, block_seq, s)
 #define SOCKET_S1_D(DD)                                    \
   do {                                                     \
     if (dtype == SOCKET_BF16) SOCKET_S1(DType_bf16, DD);   \
@@ -519,6 +522,30 @@ extern "C" size_t socket_sparse_attention_workspace_bytes(int B, int Hq, int D, 
   return (size_t)B * Hq * nsplit * (D + 1) * sizeof(float);
 }
 
+namespace {
+
+int sparse_attention_on(void* workspace, const void* q, const void* k, const void* v, int dtype,
+                        int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_h,
+                        int64_t k_stride_s, int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                        const int32_t* sparse_list, int64_t list_stride_b, int64_t list_stride_h,
+                        const int32_t* sparse_len, int64_t len_stride_b, int64_t len_stride_h, void* out,
+                        int64_t out_stride_b, int64_t out_stride_h, int B, int Hq, int Hkv, int D,
+                        int kv_rows, int max_len, void* stream) {
+  const int bs = socket_sparse_attention_block_seq(B, Hq, max_len);
+  const int nsplit = (max_len + bs - 1) / bs;
+  float* mid_o = (float*)workspace;
+  float* mid_lse = mid_o + (size_t)B * Hq * nsplit * D;
+  int st = socket_attend_stage1(q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h,
+                                k_stride_s, v_stride_b, v_stride_h, v_stride_s, sparse_list,
+                                list_stride_b, list_stride_h, sparse_len, len_stride_b, len_stride_h,
+                                mid_o, mid_lse, B, Hq, Hkv, D, kv_rows, max_len, nsplit, bs, stream);
+  if (st != SOCKET_OK) return st;
+  return socket_attend_stage2(mid_o, mid_lse, sparse_len, len_stride_b, len_stride_h, out, dtype,
+                              out_stride_b, out_stride_h, B, Hq, D, nsplit, bs, stream);
+}
+
+}  // namespace
+
 extern "C" int socket_sparse_attention(const void* q, const void* k, const void* v, int dtype,
                                        int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_b,
                                        int64_t k_stride_h, int64_t k_stride_s, int64_t v_stride_b,
@@ -534,17 +561,10 @@ extern "C" int socket_sparse_attention(const void* q, const void* k, const void*
   SOCKET_REQUIRE(workspace_bytes >= socket_sparse_attention_workspace_bytes(B, Hq, D, max_len),
                  SOCKET_ERR_WORKSPACE);
   SOCKET_REQUIRE(socket_aligned16(workspace), SOCKET_ERR_ALIGN);
-  const int bs = socket_sparse_attention_block_seq(B, Hq, max_len);
-  const int nsplit = (max_len + bs - 1) / bs;
-  float* mid_o = (float*)workspace;
-  float* mid_lse = mid_o + (size_t)B * Hq * nsplit * D;
-  int st = socket_attend_stage1(q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h,
-                                k_stride_s, v_stride_b, v_stride_h, v_stride_s, sparse_list,
-                                list_stride_b, list_stride_h, sparse_len, len_stride_b, len_stride_h,
-                                mid_o, mid_lse, B, Hq, Hkv, D, kv_rows, nsplit, bs, stream);
-  if (st != SOCKET_OK) return st;
-  return socket_attend_stage2(mid_o, mid_lse, sparse_len, len_stride_b, len_stride_h, out, dtype,
-                              out_stride_b, out_stride_h, B, Hq, D, nsplit, bs, stream);
+  return sparse_attention_on(workspace, q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h,
+                             k_stride_s, v_stride_b, v_stride_h, v_stride_s, sparse_list, list_stride_b,
+                             list_stride_h, sparse_len, len_stride_b, len_stride_h, out, out_stride_b,
+                             out_stride_h, B, Hq, Hkv, D, kv_rows, max_len, stream);
 }
 
 extern "C" size_t socket_dense_decode_workspace_bytes(int B, int Hq, int D, int T) {

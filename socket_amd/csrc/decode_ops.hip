@@ -85,7 +85,8 @@ __global__ void rope_append_kernel(const void* __restrict__ qkv, int64_t qkv_sb,
   const int hh = blockIdx.x, b = blockIdx.y, i = threadIdx.x;
   const int64_t p = pos[(int64_t)b * pos_stride];
   const bool ok = p >= 0 && p < Tcap && p < n_pos;   // a position outside the cache or the table writes nothing
-  if (hh == 0 && i == 0 && ok && lens) lens[b] = max(lens[b], (int32_t)p + 1);
+  // the cached length follows the position: rows past it are older contents, not context
+  if (hh == 0 && i == 0 && ok && lens) lens[b] = (int32_t)p + 1;
   const int64_t src = (int64_t)b * qkv_sb + (int64_t)hh * D + 2 * i;
   const float x0 = ld<DT>(qkv, src), x1 = ld<DT>(qkv, src + 1);
   if (hh >= Hq + Hkv) {  // value: plain copy

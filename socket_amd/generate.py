@@ -193,8 +193,6 @@ def generate(model: Transformer, prompt: torch.Tensor, max_new_tokens: int, *, d
     device = prompt.device
     on_gpu = device.type == "cuda"
     model.setup_caches(max_batch_size=B, max_seq_length=max_seq_length)
-    for layer in model.layers:                       # a fresh sequence: forget earlier lengths
-        layer.attention.kv_cache.lens.zero_()
     if on_gpu and decode_type != "dense":
         warmup_sparse_decode(model, device, T=min(model.max_seq_length, T))
     seq = torch.empty((B, T_new), dtype=prompt.dtype, device=device)

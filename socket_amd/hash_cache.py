@@ -302,4 +302,4 @@ class SocketHashCache:
         self.v_cache[:, :, pos0:pos0 + S].copy_(v_bshd.permute(0, 2, 1, 3))
         hash_keys_into(self.k_cache[:, :, pos0:pos0 + S], self.v_cache[:, :, pos0:pos0 + S],
                        self.planes_words, self.codes, self.v_norm, self.L, self.P, t0=pos0)
-        self.lens.clamp_(min=pos0 + S)
+        self.lens.fill_(pos0 + S)      # the cached length follows the position

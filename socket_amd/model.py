@@ -152,16 +152,23 @@ class KVCache(nn.Module):
         if S == 0:
             return self.k_cache, self.v_cache
         if S == 1 and pos0 is None:
-            # decode step: positions stay on the device
+            # decode step: the position stays on the device.  One outside the cache
+            # writes nothing (the reference raises; here the host never sees the value).
+            Tcap = self.k_cache.size(2)
             pos = input_pos.long()
-            self.k_cache.index_copy_(2, pos, k_val.permute(0, 2, 1, 3))
-            self.v_cache.index_copy_(2, pos, v_val.permute(0, 2, 1, 3))
+            ok = (pos >= 0) & (pos < Tcap)
+            at = pos.clamp(0, Tcap - 1)
+            for buf, val in ((self.k_cache, k_val), (self.v_cache, v_val)):
+                buf.index_copy_(2, at, torch.where(ok, val.permute(0, 2, 1, 3), buf.index_select(2, at)))
             pos_b = input_pos.to(torch.int32).expand(self.lens.numel()).contiguous()
             if hash_keys:
                 _hash_rows(self, k_val, v_val, pos_b=pos_b)
             elif k_hard is not None:
                 raise RuntimeError("KVCache.update: precomputed k_hard needs the host position (pass pos0)")
-            torch.maximum(self.lens, pos_b + 1, out=self.lens)
+            # the cached length follows the position (the reference masks by it every
+            # step, GPT-FAST/model.py:486-487): a cache reused at an earlier position
+            # does not expose the rows a longer sequence left behind
+            self.lens.copy_(torch.where(ok, pos_b + 1, self.lens))
             return self.k_cache, self.v_cache
         if pos0 is None:
             pos0 = int(input_pos[0])
@@ -175,7 +182,7 @@ class KVCache(nn.Module):
                 self.v_norm[:, :, pos0:pos0 + S].copy_(v_norm.permute(0, 2, 1))
             if k_hard is not None:
                 hash_cache.pack_codes_into(k_hard.permute(0, 2, 3, 1), self.codes, self.K, t0=pos0)
-        self.lens.clamp_(min=pos0 + S)
+        self.lens.fill_(pos0 + S)
         return self.k_cache, self.v_cache
 
 
@@ -278,7 +285,8 @@ class Transformer(nn.Module):
                 x, ffn = layer._run_fused(x, ffn, input_pos, sparse, step)
             return decode_ops.linear_rows(decode_ops.add_rmsnorm(x, self.norm.weight, self.norm.eps, residual=ffn)[1],
                                           self.output.weight)
-        freqs_cis = self.freqs_cis[input_pos]
+        # (a decode step's position is unchecked on the host: keep the table lookup in range)
+        freqs_cis = self.freqs_cis[input_pos if pos0 is not None else input_pos.clamp(0, self.freqs_cis.size(0) - 1)]
         for layer in self.layers:
             x = layer._run(x, input_pos, freqs_cis, sparse, pos0)
         if last_only:

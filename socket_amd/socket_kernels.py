@@ -78,7 +78,8 @@ def sparse_decode_stage1(
         ptr(sparse_list), sparse_list.stride(0), sparse_list.stride(1),
         ptr(sparse_len), sparse_len.stride(0), sparse_len.stride(1),
         ptr(mid_out), ptr(mid_out_logsumexp),
-        B, H, k.shape[1], D, k.shape[2], mid_out.shape[2], int(block_seq), stream_ptr(q.device)))
+        B, H, k.shape[1], D, k.shape[2], sparse_list.shape[-1], mid_out.shape[2], int(block_seq),
+        stream_ptr(q.device)))
 
 
 @torch.no_grad()

@@ -40,7 +40,7 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_status_strings_and_version(lib):
-    assert lib.socket_abi_version() == 1
+    assert lib.socket_abi_version() == 2
     seen = set()
     for st in range(0, -7, -1):
         s = lib.socket_status_string(st).decode()
@@ -77,10 +77,10 @@ def test_entry_points_reject_bad_arguments_without_a_device(lib):
     assert lib.socket_select_list(one, 64, nul, nul, nul, 0, 1, 1, 64, 20000, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # M too large
     assert lib.socket_select_list(one, 32, nul, nul, nul, 0, 1, 1, 64, 4, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_SHAPE  # pitch < T
     a = [one, one, one, 1, 128, 128, 0, 0, 128, 0, 0, 128, one, 8, 8, one, 1, 1, one, one]
-    assert lib.socket_attend_stage1(*a, 1, 4, 1, 48, 16, 1, 256, nul) == _lib.SOCKET_ERR_UNSUPPORTED       # D = 48
-    assert lib.socket_attend_stage1(*a, 1, 5, 2, 128, 16, 1, 256, nul) == _lib.SOCKET_ERR_SHAPE             # Hq % Hkv
+    assert lib.socket_attend_stage1(*a, 1, 4, 1, 48, 16, 8, 1, 256, nul) == _lib.SOCKET_ERR_UNSUPPORTED       # D = 48
+    assert lib.socket_attend_stage1(*a, 1, 5, 2, 128, 16, 8, 1, 256, nul) == _lib.SOCKET_ERR_SHAPE             # Hq % Hkv
     a[5] = 100                                                                                            # q head stride not 16-byte aligned for bf16
-    assert lib.socket_attend_stage1(*a, 1, 4, 1, 128, 16, 1, 256, nul) == _lib.SOCKET_ERR_ALIGN
+    assert lib.socket_attend_stage1(*a, 1, 4, 1, 128, 16, 8, 1, 256, nul) == _lib.SOCKET_ERR_ALIGN
     # workspace too small
     need = lib.socket_sparse_attention_workspace_bytes(1, 4, 128, 300)
     assert need > 0

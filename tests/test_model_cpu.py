@@ -114,8 +114,11 @@ def test_kv_cache_update_bookkeeping(monkeypatch):
     k1 = torch.randn(2, 1, 1, 128, generator=g); v1 = torch.randn(2, 1, 1, 128, generator=g)
     c.update(torch.tensor([8]), k1, v1, hash_keys=True)                                 # decode step: device positions
     assert c.lens.tolist() == [9, 9] and torch.equal(c.k_cache[:, 0, 8], k1[:, 0, 0])
-    c.update(torch.tensor([2]), k1, v1)                                                 # earlier position: lens stay
-    assert c.lens.tolist() == [9, 9]
+    c.update(torch.tensor([2]), k1, v1)                                                 # earlier position: the length follows it
+    assert c.lens.tolist() == [3, 3]
+    before = c.k_cache.clone()
+    c.update(torch.tensor([32]), k1, v1)                                                # outside the cache: nothing written
+    assert c.lens.tolist() == [3, 3] and torch.equal(c.k_cache, before)
     with pytest.raises(RuntimeError, match="out-of-bounds"):
         c.update(torch.arange(30, 35), k, v)
     with pytest.raises(AssertionError):
@@ -159,6 +162,36 @@ def test_decode_steps_equal_one_long_prefill(monkeypatch):
     model(ids[:, :6], torch.arange(6), pos0=0)
     tail = model(ids[:, 6:], torch.arange(6, 14), pos0=6)
     torch.testing.assert_close(tail, full[:, 6:], rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("sparse", [True, False])
+def test_a_cache_reused_for_a_shorter_prompt_forgets_the_longer_one(monkeypatch, sparse):
+    """A long prompt, then a shorter one on the same caches through the public
+    forward calls (no generate(), nothing reset by hand): rows the longer sequence
+    left behind are past the current position and must be neither scored nor
+    attended (GPT-FAST/model.py:486-487 masks by the position every step)."""
+    oracle_backend.install(monkeypatch, M)
+    g = torch.Generator().manual_seed(8)
+    long_ids = torch.randint(0, 211, (1, 40), generator=g)
+    short_ids = torch.randint(0, 211, (1, 12), generator=g)
+
+    def run(model, ids, n_prompt):
+        fwd = model.sparse_forward if sparse else model.forward
+        out = [fwd(ids[:, :n_prompt], torch.arange(n_prompt), pos0=0)[:, -1]]
+        for t in range(n_prompt, ids.shape[1]):
+            out.append(fwd(ids[:, t:t + 1], torch.tensor([t]))[:, -1])
+        return torch.stack(out, 1)
+
+    used = toy_model(seed=3, heavy_const=5)
+    used.setup_caches(1, 48)
+    run(used, long_ids, 30)
+    assert used.layers[0].attention.kv_cache.lens.tolist() == [40]
+    have = run(used, short_ids, 7)
+    assert used.layers[0].attention.kv_cache.lens.tolist() == [12]
+    fresh = toy_model(seed=3, heavy_const=5)
+    fresh.setup_caches(1, 48)
+    want = run(fresh, short_ids, 7)
+    torch.testing.assert_close(have, want, rtol=0, atol=0)
 
 
 def test_sparse_hook_with_small_budget_keeps_cache_codes_consistent(monkeypatch):

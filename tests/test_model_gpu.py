@@ -71,6 +71,48 @@ def test_sparse_hook_matches_oracle_attention(dev, monkeypatch, dtype, tol):
         assert torch.equal(have.argmax(-1), want.argmax(-1))
 
 
+@pytest.mark.parametrize("sparse", [True, False])
+def test_a_cache_reused_for_a_shorter_prompt_forgets_the_longer_one(dev, sparse):
+    """A long prompt and some decode steps, then a shorter prompt on the same caches
+    through the public forward calls: identical logits to a model whose caches
+    never held the longer sequence."""
+    g = torch.Generator().manual_seed(21)
+    long_ids = torch.randint(0, 331, (2, 300), generator=g).to(dev)
+    short_ids = torch.randint(0, 331, (2, 90), generator=g).to(dev)
+    used = toy_model(dev, torch.bfloat16, seed=9)
+    used.setup_caches(2, 320)
+    _run_steps(used, long_ids, 290, sparse=sparse)
+    assert used.layers[0].attention.kv_cache.lens.tolist() == [300, 300]
+    have = _run_steps(used, short_ids, 80, sparse=sparse)
+    assert used.layers[0].attention.kv_cache.lens.tolist() == [90, 90]
+    fresh = toy_model(dev, torch.bfloat16, seed=9)
+    fresh.setup_caches(2, 320)
+    want = _run_steps(fresh, short_ids, 80, sparse=sparse)
+    assert torch.equal(have, want)
+
+
+def test_eager_decode_step_at_a_position_outside_the_cache_writes_nothing(dev):
+    """The unfused single-token path with a device-side position past the cache:
+    no row is written and the length stays (the fused path and the hashing kernel
+    behave the same way)."""
+    c = M.KVCache(2, 64, 2, 128, L=20, R=1024, dtype=torch.bfloat16, K=10, device=dev)
+    g = torch.Generator().manual_seed(22)
+    k = torch.randn(2, 1, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    c.planes_words = hash_cache_planes(dev)
+    c.update(torch.tensor([5], device=dev), k, k, hash_keys=True)
+    assert c.lens.tolist() == [6, 6] and torch.equal(c.k_cache[:, :, 5], k[:, 0])
+    snap = (c.k_cache.clone(), c.codes.clone(), c.v_norm.clone())
+    c.update(torch.tensor([64], device=dev), k, k, hash_keys=True)
+    assert c.lens.tolist() == [6, 6]
+    assert torch.equal(c.k_cache, snap[0]) and torch.equal(c.codes, snap[1]) and torch.equal(c.v_norm, snap[2])
+
+
+def hash_cache_planes(dev):
+    from socket_amd import hash_cache
+    g = torch.Generator().manual_seed(23)
+    return hash_cache.permute_planes(torch.randn(20, 10, 128, generator=g).to(dev))
+
+
 def test_cache_hash_state_after_prefill_and_decode(dev):
     """Codes and value norms written by the fused append equal the oracle's hash
     of the cached rows wherever the fp64 projection is clear of zero."""
@@ -188,7 +230,7 @@ def test_rope_append_equals_the_torch_chain(dev, dtype):
         kc[:, :, pos] = 0
         vc[:, :, pos] = 0
         assert not kc.any() and not vc.any()                                   # nothing else was touched
-        assert lens.tolist() == [max(3, pos + 1), max(10, pos + 1), 70]
+        assert lens.tolist() == [pos + 1] * 3                                  # the length follows the position
     # per-sequence positions; one of them outside the cache writes nothing
     kc = torch.zeros(B, Hkv, Tcap, D, dtype=dtype, device=dev)
     vc = torch.zeros_like(kc)
