@@ -290,6 +290,31 @@ int socket_sparse_attention(const void* q, const void* k, const void* v, int dty
                             void* workspace, size_t workspace_bytes,
                             int B, int Hq, int Hkv, int D, int kv_rows, int max_len, void* stream);
 
+/* socket_sparse_attention without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The per-split partials go to a fixed array of SOCKET_STATIC_SCRATCH_BYTES in
+ * device memory that belongs to the library's image (each GPU the library runs
+ * on holds one copy until the process ends); a call whose
+ * socket_sparse_attention_workspace_bytes(B, Hq, D, max_len) exceeds that size
+ * returns SOCKET_ERR_WORKSPACE and launches nothing.  The call allocates and
+ * frees nothing.  All calls on one GPU share the array: calls that overlap in
+ * time on the same GPU (different streams or threads) race; serialise them.
+ * Same results as socket_sparse_attention.
+ * socket_static_scratch_init looks the array's device address up for the current
+ * device ahead of the first call (optional; the first call does it otherwise). */
+#define SOCKET_STATIC_SCRATCH_BYTES (4u << 20)
+size_t socket_static_scratch_bytes(void);
+int socket_static_scratch_init(void);
+int socket_sparse_attention_static(const void* q, const void* k, const void* v, int dtype,
+                                   int64_t q_stride_b, int64_t q_stride_h,
+                                   int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                                   int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                                   const int32_t* sparse_list, int64_t list_stride_b, int64_t list_stride_h,
+                                   const int32_t* sparse_len, int64_t len_stride_b, int64_t len_stride_h,
+                                   void* out, int64_t out_stride_b, int64_t out_stride_h,
+                                   int B, int Hq, int Hkv, int D, int kv_rows, int max_len, void* stream);
+
 /* Dense split-K flash-decode over rows [0, len(b)) of the cache (the
  * comparator the sparse path is timed against; the reference's dense decode is
  * Attention.forward, GPT-FAST/model.py:562-589).  K/V rows are read once per kv

@@ -69,6 +69,11 @@ SIGNATURES = {
     "socket_sparse_attention": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L,
                                      _P, _L, _L, _P, _L, _L, _P, _L, _L, _P, _Z,
                                      _I, _I, _I, _I, _I, _I, _P]),
+    "socket_static_scratch_bytes": (_Z, []),
+    "socket_static_scratch_init": (_I, []),
+    "socket_sparse_attention_static": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L,
+                                            _P, _L, _L, _P, _L, _L, _P, _L, _L,
+                                            _I, _I, _I, _I, _I, _I, _P]),
     "socket_dense_decode_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "socket_dense_decode": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L,
                                  _P, _P, _L, _L, _P, _Z, _I, _I, _I, _I, _I, _P]),

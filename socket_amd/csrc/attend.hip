@@ -15,6 +15,8 @@
 // before any is consumed to keep enough gathers in flight.
 #include <math.h>
 
+#include <atomic>
+
 #include "socket_common.h"
 
 namespace {
@@ -562,6 +564,66 @@ extern "C" int socket_sparse_attention(const void* q, const void* k, const void*
                  SOCKET_ERR_WORKSPACE);
   SOCKET_REQUIRE(socket_aligned16(workspace), SOCKET_ERR_ALIGN);
   return sparse_attention_on(workspace, q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h,
+                             k_stride_s, v_stride_b, v_stride_h, v_stride_s, sparse_list, list_stride_b,
+                             list_stride_h, sparse_len, len_stride_b, len_stride_h, out, out_stride_b,
+                             out_stride_h, B, Hq, Hkv, D, kv_rows, max_len, stream);
+}
+
+// ---------------------------------------------------------------------------
+// socket_sparse_attention for callers that cannot allocate: the per-split
+// partials live in a fixed array in device memory that is part of the library's
+// image.  Every GPU the library runs on holds its own copy until the process ends.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[SOCKET_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (the array's name is only a
+// host-side handle).  Looked up once per device; no allocation.
+int static_scratch(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SOCKET_ERR_LAUNCH;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return SOCKET_ERR_LAUNCH;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same address
+  }
+  *out = p;
+  return SOCKET_OK;
+}
+
+}  // namespace
+
+extern "C" size_t socket_static_scratch_bytes(void) { return (size_t)SOCKET_STATIC_SCRATCH_BYTES; }
+
+extern "C" int socket_static_scratch_init(void) {
+  void* p = nullptr;
+  return static_scratch(&p);
+}
+
+extern "C" int socket_sparse_attention_static(const void* q, const void* k, const void* v, int dtype,
+                                              int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_b,
+                                              int64_t k_stride_h, int64_t k_stride_s, int64_t v_stride_b,
+                                              int64_t v_stride_h, int64_t v_stride_s,
+                                              const int32_t* sparse_list, int64_t list_stride_b,
+                                              int64_t list_stride_h, const int32_t* sparse_len,
+                                              int64_t len_stride_b, int64_t len_stride_h, void* out,
+                                              int64_t out_stride_b, int64_t out_stride_h, int B, int Hq,
+                                              int Hkv, int D, int kv_rows, int max_len, void* stream) {
+  SOCKET_REQUIRE(out, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(max_len > 0 && B > 0 && Hq > 0 && D > 0, SOCKET_ERR_SHAPE);
+  // the partials of this call must fit the fixed array
+  SOCKET_REQUIRE(socket_sparse_attention_workspace_bytes(B, Hq, D, max_len) <= (size_t)SOCKET_STATIC_SCRATCH_BYTES,
+                 SOCKET_ERR_WORKSPACE);
+  void* ws = nullptr;
+  const int st = static_scratch(&ws);
+  if (st != SOCKET_OK) return st;
+  // Nothing in the array has to start at zero: stage 1 writes every split stage 2
+  // reads (the first ceil(len / split size) of a row); older contents are never read.
+  return sparse_attention_on(ws, q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h,
                              k_stride_s, v_stride_b, v_stride_h, v_stride_s, sparse_list, list_stride_b,
                              list_stride_h, sparse_len, len_stride_b, len_stride_h, out, out_stride_b,
                              out_stride_h, B, Hq, Hkv, D, kv_rows, max_len, stream);

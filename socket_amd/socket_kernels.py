@@ -146,6 +146,34 @@ def sparse_attention_fwd(
 
 
 @torch.no_grad()
+def sparse_attention_fwd_static(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                sparse_list: torch.Tensor, sparse_len: torch.Tensor,
+                                out: torch.Tensor) -> torch.Tensor:
+    """`sparse_attention_fwd` into a caller-provided `out` [B,H,D] without allocating
+    anything: the per-split partials live in a fixed array inside the library
+    (one per GPU, shared by every call on it: calls that overlap on one GPU race).
+    `sparse_list` / `sparse_len` must already be int32.  Raises RuntimeError when
+    the call needs more than the array holds."""
+    assert query.is_cuda and key.is_cuda and value.is_cuda and sparse_list.is_cuda and sparse_len.is_cuda
+    D = _check_qkv(query, key, value)
+    B, H, _ = query.shape
+    assert sparse_list.dtype == torch.int32 and sparse_len.dtype == torch.int32 and sparse_list.stride(-1) == 1
+    assert out.is_cuda and tuple(out.shape) == (B, H, D) and out.dtype == query.dtype and out.stride(-1) == 1
+    width = sparse_list.shape[-1]
+    assert width > 0
+    check("socket_sparse_attention_static", lib().socket_sparse_attention_static(
+        ptr(query), ptr(key), ptr(value), dtype_enum(query.dtype),
+        query.stride(0), query.stride(1),
+        key.stride(0), key.stride(1), key.stride(2),
+        value.stride(0), value.stride(1), value.stride(2),
+        ptr(sparse_list), sparse_list.stride(0), sparse_list.stride(1),
+        ptr(sparse_len), sparse_len.stride(0), sparse_len.stride(1),
+        ptr(out), out.stride(0), out.stride(1),
+        B, H, key.shape[1], D, key.shape[2], width, stream_ptr(query.device)))
+    return out
+
+
+@torch.no_grad()
 def dense_decode_fwd(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                      lengths: torch.Tensor) -> torch.Tensor:
     """Dense flash-decode over rows [0, lengths[b]) of the cache: the comparator

@@ -89,6 +89,13 @@ def test_entry_points_reject_bad_arguments_without_a_device(lib):
     assert r == _lib.SOCKET_ERR_WORKSPACE
     with pytest.raises(_lib.SocketHipError, match="workspace"):
         _lib.check("socket_sparse_attention", r)
+    # the variant on the library's own fixed array refuses what does not fit it (checked before any device call)
+    assert lib.socket_static_scratch_bytes() == 4 << 20
+    big = lib.socket_sparse_attention_workspace_bytes(64, 512, 128, 4096)
+    assert big > lib.socket_static_scratch_bytes()
+    r = lib.socket_sparse_attention_static(one, one, one, 1, 128, 128, 0, 0, 128, 0, 0, 128, one, 4096, 4096, one, 512, 1,
+                                           one, 65536, 128, 64, 512, 8, 128, 16, 4096, nul)
+    assert r == _lib.SOCKET_ERR_WORKSPACE
 
 
 def test_sizes_helpers(lib):

@@ -1,0 +1,56 @@
+"""socket_sparse_attention_static (the entry point that allocates nothing: its
+per-split partials live in a fixed array inside the library) against
+socket_sparse_attention on the same inputs, through the C ABI.  Both run the
+same kernels with the same split, so the outputs must be identical bit for bit.
+Two calls in a row share the array; the second is smaller than the first."""
+import pytest
+import torch
+
+from socket_amd import _lib, socket_kernels
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(dev, seed, B, Hq, Hkv, T, width, dtype):
+    g = torch.Generator().manual_seed(seed)
+    D = 128
+    q = torch.randn(B, Hq, D, generator=g).to(dtype).to(dev)
+    k = torch.randn(B, Hkv, T, D, generator=g).to(dtype).to(dev)
+    v = torch.randn(B, Hkv, T, D, generator=g).to(dtype).to(dev)
+    sl = torch.randint(0, T, (B, Hq, width), generator=g, dtype=torch.int32)
+    ln = torch.randint(1, width + 1, (B, Hq), generator=g, dtype=torch.int32)
+    ln[0, 0] = width
+    sl[0, 1, :3] = -1            # skipped entries
+    return q, k, v, sl.to(dev), ln.to(dev)
+
+
+def test_static_scratch_variant_equals_the_workspace_variant(dev):
+    lib = _lib.lib()
+    assert lib.socket_static_scratch_init() == 0
+    # first a large call, then a smaller one that reuses the front of the same array
+    for seed, (B, Hq, Hkv, T, width, dtype) in enumerate([
+            (4, 32, 8, 6000, 2308, torch.bfloat16),
+            (1, 8, 2, 900, 196, torch.float32),
+            (2, 28, 4, 3000, 1100, torch.float16)]):
+        q, k, v, sl, ln = _case(dev, 100 + seed, B, Hq, Hkv, T, width, dtype)
+        want = socket_kernels.sparse_attention_fwd(q, k, v, sl, ln)
+        out = torch.full_like(want, float("nan"))
+        torch.cuda.synchronize()
+        allocs = torch.cuda.memory_stats()["allocation.all.allocated"]
+        got = socket_kernels.sparse_attention_fwd_static(q, k, v, sl, ln, out)
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == allocs   # no allocation through torch either
+        torch.cuda.synchronize()
+        assert torch.isfinite(want.float()).all()
+        assert torch.equal(got, want), f"case {seed}: max diff {(got.float() - want.float()).abs().max()}"
+
+
+def test_static_scratch_variant_refuses_what_does_not_fit(dev):
+    lib = _lib.lib()
+    B, Hq, Hkv, T, width = 64, 512, 8, 64, 4096
+    assert lib.socket_sparse_attention_workspace_bytes(B, Hq, 128, width) > lib.socket_static_scratch_bytes()
+    q = torch.zeros(B, Hq, 128, dtype=torch.bfloat16, device=dev)
+    k = torch.zeros(B, Hkv, T, 128, dtype=torch.bfloat16, device=dev)
+    sl = torch.zeros(B, Hq, width, dtype=torch.int32, device=dev)
+    ln = torch.ones(B, Hq, dtype=torch.int32, device=dev)
+    with pytest.raises(_lib.SocketHipError, match="workspace"):
+        socket_kernels.sparse_attention_fwd_static(q, k, k, sl, ln, torch.empty_like(q))
