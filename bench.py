@@ -8,14 +8,19 @@ sink + window list, and attend over the listed rows.  The default workload is
 configuration 3 (batch 4, 32/8 heads, head dim 128, 131072-token bf16 cache,
 L=60 x P=10, top-k 2048 + 4 sink + 256 window).
 
-Prints one JSON line: `value` is microseconds per layer per step for the sparse
-path; `roofline` prices the scorer (the kernel moving the most bytes) against
-HBM peak; `kernels` does the same for every kernel; `dense` is the dense
-flash-decode comparator on the same GPU; `cpu_baseline` is the CPU oracle timed
-on the host's cores on a slice of the same workload.
+Prints one JSON line.  `value` is microseconds per layer per step of the sparse
+path on configuration 3, exactly --steps graph replays after --warmup; `roofline`
+prices the scorer (the kernel moving the most bytes) against HBM peak; `kernels`
+does the same for every kernel of the step and for the dense flash-decode
+comparator on the same GPU (each timed as a HIP-graph replay of ten launches, so
+small kernels are not priced at the cost of an eager Python call); `c2` and `c5`
+are the same records for configurations 2 and 5; `decode_tok_s` is the end-to-end
+greedy decode of the 32-layer Llama-3.1-8B-shaped model, sparse and dense, at
+128k context and at configuration 4's 65536-token prompt; `cpu_baseline` is the
+CPU oracle timed on the host's cores on a slice of configuration 3.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5]
-                  [--only score|select|attend|hash|dense] [--no-cpu] [--no-parity]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5] [--no-extra]
+                  [--only score|score_grouped|select|attend|hash|dense|step|decode|...] [--no-cpu] [--no-parity]
 """
 from __future__ import annotations
 
@@ -34,11 +39,13 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+BOX_CPU_SHARE = 16              # host cores a one-GPU job is given on the benchmark box
 
 # HBM bytes per launch of the scorer from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `bench.py --only score` (see profiles/), keyed by workload; None until
 # a counter run for that workload has been recorded there.
-MEASURED_TRAFFIC_BYTES = {"c3": int((195969 + 65561) * 1024 * 1.00)}
+MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_SOURCE = None
 
 
 def algorithmic_bytes(w, lens=None, budgets=None):
@@ -65,6 +72,40 @@ def algorithmic_bytes(w, lens=None, budgets=None):
         "attend": w.Hq * kt * (4 * w.D + 4) + w.B * w.Hq * 4 * w.D,
         "dense": w.Hkv * tok * 4 * w.D,
     }
+
+
+def time_graph(fn, iters, warmup=2, per_graph=10):
+    """Average device time in microseconds of one call of `fn`: `per_graph` calls are
+    recorded into one HIP graph and the graph is replayed between two HIP events, so
+    the figure is kernel time plus the in-graph launch gap, without the Python and
+    ctypes cost of an eager call (which is several microseconds, more than some of
+    these kernels take).  Falls back to eager launches if capture fails."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(max(warmup, 2)):
+                fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(per_graph):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        reps = max(1, (iters + per_graph - 1) // per_graph)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1000.0 / (reps * per_graph)
+    except Exception as e:  # noqa: BLE001
+        print(f"bench: graph timing unavailable ({e}); timing eager launches", file=sys.stderr)
+        return time_launches(fn, iters, warmup)
 
 
 def time_launches(fn, iters, warmup=3):
@@ -132,7 +173,10 @@ def cpu_baseline(w, inp_cpu, codes_cpu, vnorm_cpu, seconds_budget=20.0):
     heads (2*G query heads), full context; scaled to the whole layer."""
     from oracle import socket_oracle as orc
 
-    cores = min(os.cpu_count() or 1, 16)
+    # every core this job may use: the GPU box gives a one-GPU job 16 of the host's cores
+    # (its os.cpu_count() reports the whole host); both figures are in the record
+    host_cores = os.cpu_count() or 1
+    cores = min(host_cores, BOX_CPU_SHARE)
     torch.set_num_threads(cores)
     G = w.Hq // w.Hkv
     nkv = min(2, w.Hkv)
@@ -172,6 +216,7 @@ def cpu_baseline(w, inp_cpu, codes_cpu, vnorm_cpu, seconds_budget=20.0):
         "value": round(total_us, 1),
         "unit": "us/layer/step",
         "cores": cores,
+        "host_cpu_count": host_cores,
         "kind": "port",
         "sample": f"sequence 0, {nkv} of {w.Hkv} kv heads ({nkv * G} query heads), context {T}, "
                   f"median of {len(reps)} reps, scaled x{scale:.2f} to the whole layer",
@@ -192,6 +237,255 @@ def _cpu_model():
     return "unknown"
 
 
+class Step:
+    """One workload's tensors on the device and the closures that run each kernel of the
+    step on them (the same calls the attention hook makes)."""
+
+    def __init__(self, w, dev, reference_table_layout=False):
+        from socket_amd import hash_cache, socket_kernels, sparse
+        from socket_amd.workloads import make_inputs
+        self.w, self.dev = w, dev
+        self.hc, self.sk, self.sp = hash_cache, socket_kernels, sparse
+        t0 = time.perf_counter()
+        self.inp = inp = make_inputs(w, device=dev, device_rng=True)
+        torch.cuda.synchronize()
+        self.input_generation_s = time.perf_counter() - t0
+        B, Hq, Hkv, T = w.B, w.Hq, w.Hkv, w.T
+        self.NW = hash_cache.words_per_key(w.L, w.P)
+        Tcap = (T + 7) // 8 * 8
+        self.codes = torch.zeros((B, Hkv, self.NW, Tcap), dtype=torch.int32, device=dev)
+        self.v_norm = torch.zeros((B, Hkv, Tcap), dtype=torch.float16, device=dev)
+        self.planes_words = hash_cache.permute_planes(inp.planes)
+        self.lens, self.budgets = inp.lens, inp.budgets
+        self.abytes = algorithmic_bytes(w, None if self.lens is None else self.lens.cpu(),
+                                        None if self.budgets is None else self.budgets.cpu())
+        pitch = (T + 3) // 4 * 4
+        self.scores_buf = torch.empty((B, Hq, pitch), dtype=torch.float32, device=dev)
+        self.new_pos = None if self.lens is None else (self.lens - w.new_keys).to(torch.int32)
+        # the soft-hash table in the dtype the model produces it in: the reference's
+        # soft_hash runs in the model dtype (GPT-FAST/model.py:392-401), bf16 here
+        self.q_table = inp.q_probs.to(torch.bfloat16) if w.dtype == torch.bfloat16 else inp.q_probs
+        self.q_table_f32 = self.q_table.float()
+        # ... and in the layout the fused soft-hash kernel writes it in (heads of a KV head
+        # interleaved per bucket: the scorer's LDS image); same values
+        self.q_table_grouped = hash_cache.group_q_probs(self.q_table, Hkv)
+        # the step uses the layout the library asks its producers for at this shape
+        self.use_grouped = (not reference_table_layout and
+                            hash_cache._prefers_grouped(B, Hq, Hkv, T, 1 if self.q_table.dtype == torch.bfloat16 else 0,
+                                                        w.L, w.P, self.q_table.shape[-1]))
+        self.dense_lens = self.lens if self.lens is not None else torch.full((B,), T, dtype=torch.int32, device=dev)
+
+    # ---- K1 at scale: hash of the whole cache
+    def prefill_hash(self):
+        w = self.w
+        self.hc.hash_keys_into(self.inp.k, self.inp.v, self.planes_words, self.codes, self.v_norm, w.L, w.P, t0=0,
+                               layout="bhsd")
+
+    # ---- the kernels of one step
+    def k_hash(self):
+        # the newly appended key(s) of every (sequence, kv head) land on the last
+        # position(s), so the context length is the same every step
+        w = self.w
+        self.hc.hash_keys_into(self.inp.k_new, self.inp.v_new, self.planes_words, self.codes, self.v_norm, w.L, w.P,
+                               t0=w.T - w.new_keys, pos_b=self.new_pos, layout="bshd")
+
+    def k_score_ref(self):
+        return self.hc.score_packed(self.q_table, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
+                                    out=self.scores_buf, with_range=True)
+
+    def k_score_grouped(self):
+        return self.hc.score_packed(self.q_table_grouped, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
+                                    out=self.scores_buf, with_range=True, n_heads=self.w.Hq)
+
+    def k_score_f32(self):
+        return self.hc.score_packed(self.q_table_f32, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
+                                    out=self.scores_buf)
+
+    def k_score(self):
+        return self.k_score_grouped() if self.use_grouped else self.k_score_ref()
+
+    def k_select(self, scores, rng=None):
+        w = self.w
+        return self.sp.select_list(scores, w.sink, w.window, w.M, lens=self.lens, budgets=self.budgets, row_range=rng)
+
+    def k_attend(self, sl, ln):
+        return self.sk.sparse_attention_fwd(self.inp.q, self.inp.k, self.inp.v, sl, ln)
+
+    def k_dense(self):
+        return self.sk.dense_decode_fwd(self.inp.q, self.inp.k, self.inp.v, self.dense_lens)
+
+    def step(self):
+        """hash-append + score + select + attend, as `hash_cache.sparse_decode_step` after the append."""
+        w = self.w
+        self.k_hash()
+        return self.hc.sparse_decode_step(self.inp.q, self.q_table_grouped if self.use_grouped else self.q_table,
+                                          self.inp.k, self.inp.v, self.codes, self.v_norm, w.T, w.P, w.sink, w.window,
+                                          w.M, lens=self.lens, budgets=self.budgets)
+
+    # ---- parity gates on the full-size tensors (device-side checks, not timed)
+    def parity(self, scores, sl, ln, out):
+        w, inp, dev = self.w, self.inp, self.dev
+        T, D, Hq, Hkv = w.T, w.D, w.Hq, w.Hkv
+        res = {}
+        s0 = scores[0, :8]
+        n0 = T if self.lens is None else int(self.lens[0])
+        m0 = w.M if self.budgets is None else int(self.budgets[0])
+        order = torch.sort(s0[:, :n0], dim=-1, descending=True, stable=True).indices[:, :m0].to(torch.int32)
+        nbase = int(ln[0, 0]) - m0
+        res["topk_exact_rows_checked"] = 8
+        res["topk_exact"] = bool(torch.equal(sl[0, :8, nbase:nbase + m0], order))
+        # attention vs an fp32 gather-softmax over the same list, one sequence
+        idx = sl[0, :, :int(ln[0, 0])].long()
+        kvh = (torch.arange(Hq, device=dev) // (Hq // Hkv))[:, None]
+        kk = inp.k[0][kvh, idx].float()
+        vv = inp.v[0][kvh, idx].float()
+        att = torch.softmax((kk @ inp.q[0].float().unsqueeze(-1)).squeeze(-1) / D ** 0.5, -1)
+        ref = (att.unsqueeze(1) @ vv).squeeze(1)
+        res["attend_max_abs_err"] = float((out[0].float() - ref).abs().max())
+        # scores vs an fp32 gather-sum in table order on the unpacked codes, one kv head
+        c16 = self.hc.unpack_codes(self.codes[:1, :1].contiguous(), w.L, w.P, 0, n0).long()[0, 0]   # [L,T]
+        acc = torch.zeros(n0, dtype=torch.float32, device=dev)
+        for l in range(w.L):
+            acc = acc + self.q_table_f32[0, 0, l].gather(0, c16[l])
+        ref_s = acc * self.v_norm[0, 0, :n0].float()
+        res["score_max_rel_err"] = float(((scores[0, 0, :n0] - ref_s).abs() / ref_s.abs().clamp_min(1e-30)).max())
+        return res
+
+
+def timed_graph_steps(step_fn, steps, warmup, eager=False):
+    """Records one step into a HIP graph, checks three replays against the eager
+    result, then times exactly `steps` replays after `warmup` untimed ones.  Returns
+    (ms per step, wall ms of the timed region, "hip graph replay" | "eager", replay == eager)."""
+    graph, ok = None, None
+    if not eager:
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(2):
+                    step_fn()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            out_eager = step_fn().clone()   # the state is stationary from here on (same key re-appended)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out_graph = step_fn()
+            for _ in range(3):
+                graph.replay()
+                torch.cuda.synchronize()
+                if not torch.equal(out_graph, out_eager):
+                    raise RuntimeError("graph replay differs from the eager step")
+                _ = float(out_eager.float().sum())        # unrelated eager work between the replays
+            ok = True
+        except Exception as e:  # noqa: BLE001  fall back to eager launches, and say so in the result
+            print(f"bench: HIP graph capture unavailable ({e}); timing eager launches", file=sys.stderr)
+            graph, ok = None, None
+    run = graph.replay if graph is not None else step_fn
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall_ms, "hip graph replay" if graph is not None else "eager", ok
+
+
+def measure_workload(w, dev, steps, warmup, args, full):
+    """Per-kernel times, the graph-replayed step and the dense comparator for one
+    workload.  `full`: also the scorer's other table layouts, the prefill hash and
+    the parity gates (the headline workload)."""
+    st = Step(w, dev, reference_table_layout=args.reference_table_layout)
+    prefill_us = time_launches(st.prefill_hash, 3, warmup=1)
+    scores, rng = st.k_score()
+    sl, ln = st.k_select(scores, rng)
+    out = st.k_attend(sl, ln)
+    torch.cuda.synchronize()
+    iters = max(steps, 1)
+    parity = None if (args.no_parity or not full) else st.parity(scores, sl, ln, out)
+    per = {
+        "hash": time_graph(st.k_hash, iters),
+        "score": time_graph(st.k_score, iters),
+        "select": time_graph(lambda: st.k_select(scores, rng), iters),
+        "attend": time_graph(lambda: st.k_attend(sl, ln), iters),
+        "dense": time_graph(st.k_dense, max(iters // 2, 5), per_graph=5),
+    }
+    if full:
+        per["score_reference_layout"] = time_graph(st.k_score_ref, iters)
+        per["score_f32_table"] = time_graph(st.k_score_f32, iters)
+        per["select_own_range"] = time_graph(lambda: st.k_select(scores), iters)
+    ab = st.abytes
+    kernels = {k: {"us": round(v, 2), "algorithmic_MB": round(ab[k] / 1e6, 2), "gbs": round(ab[k] / v / 1e3, 1),
+                   "hbm_frac": round(ab[k] / v / 1e3 / HBM_PEAK_GBS, 4)} for k, v in per.items()}
+    ms_per_step, wall_ms, launch, replay_ok = timed_graph_steps(st.step, steps, warmup, eager=args.eager)
+    sparse_us = ms_per_step * 1e3
+    sparse_bytes = ab["score"] + ab["select"] + ab["attend"]
+    kernel_sum_us = per["score"] + per["select"] + per["attend"]
+    from socket_amd._lib import lib
+    rows = w.B * w.Hkv * w.T
+    rec = {
+        "workload": f"{w.name}: B{w.B} Hq{w.Hq}/Hkv{w.Hkv} D{w.D} T{w.T} bf16 KV cache, L{w.L}xP{w.P} packed codes, "
+                    f"{str(st.q_table.dtype).split('.')[-1]} soft-hash table "
+                    f"({'grouped' if st.use_grouped else '[B,Hq,L,R]'} layout), "
+                    f"top-k {w.M} + sink {w.sink} + window {w.window}" + (", ragged lengths" if w.ragged else ""),
+        "step_us": round(sparse_us, 2),
+        "ms_per_step": ms_per_step,
+        "launch": launch,
+        "kernel_timing": "HIP-graph replay of 10 launches between two HIP events (kernel time + in-graph launch gap)",
+        "kernels": kernels,
+        "sparse_total": {"algorithmic_MB": round(sparse_bytes / 1e6, 2), "kernel_sum_us": round(kernel_sum_us, 2),
+                         "hbm_frac_of_kernel_sum": round(sparse_bytes / kernel_sum_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "hbm_frac_of_step": round(sparse_bytes / sparse_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "speedup_vs_dense": round(per["dense"] / sparse_us, 3),
+                         "attend_block_seq": lib().socket_sparse_attention_block_seq(w.B, w.Hq, sl.shape[-1])},
+        "hash_prefill": {
+            "prefill_ms": round(prefill_us / 1e3, 3), "rows": rows,
+            # flops of the contraction the reference performs: 2 * D * L * P per key row
+            "mfma_tflops": round(2.0 * rows * w.D * w.L * w.P / prefill_us / 1e6, 1),
+            "mfma_frac": round(2.0 * rows * w.D * w.L * w.P / prefill_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "hbm_gbs": round(rows * (2 * 2 * w.D + 4 * st.NW + 2) / prefill_us / 1e3, 1),
+            "hbm_frac": round(rows * (2 * 2 * w.D + 4 * st.NW + 2) / prefill_us / 1e3 / HBM_PEAK_GBS, 4)},
+        "parity": parity,
+        "graph_replay_equals_eager": replay_ok,
+        "wall_ms_timed_region": round(wall_ms, 2),
+        "input_generation_s": round(st.input_generation_s, 1),
+        "new_keys_hashed_per_step": w.B * w.Hkv * w.new_keys,
+    }
+    return rec, st, per
+
+
+def decode_tok_s(dev, prompt_len, new_tokens, n_layer=None, kinds=("sparse", "dense")):
+    """End-to-end greedy decode of the Llama-3.1-8B-shaped random-weight model through
+    socket_amd.generate: decode-only tokens per second (the prefill's token excluded, as
+    GPT-FAST/generate.py:361-369 counts), whole step replayed as one HIP graph."""
+    from socket_amd import generate as gen
+    from socket_amd.model import ModelArgs
+    cfg = ModelArgs.from_name("Llama-3.1-8B")
+    if n_layer is not None:
+        cfg.n_layer = n_layer
+    model = gen.load_random_model(cfg, dev, torch.bfloat16, 1234)
+    g = torch.Generator().manual_seed(1234)
+    prompt = torch.randint(0, cfg.vocab_size, (1, prompt_len), generator=g).to(dev)
+    rec = {"model": f"Llama-3.1-8B geometry, {cfg.n_layer} layers, random bf16 weights N(0, 0.02)",
+           "prompt_len": prompt_len, "new_tokens": new_tokens, "batch": 1,
+           "budget": f"top-k {cfg.heavy_const} + sink {cfg.sink_size} + window {cfg.window_size}"}
+    for kind in kinds:
+        _, st = gen.generate(model, prompt, new_tokens, decode_type=kind, use_graph=True)
+        rec[kind] = {"decode_tok_s": round(st["decode_only_tokens"] / st["decode_time_s"], 2),
+                     "ms_per_token": round(1e3 * st["decode_time_s"] / st["decode_only_tokens"], 3),
+                     "prefill_s": round(st["prefill_time_s"], 2), "graph": st["graph"]}
+    if "sparse" in rec and "dense" in rec:
+        rec["sparse_vs_dense"] = round(rec["sparse"]["decode_tok_s"] / rec["dense"]["decode_tok_s"], 3)
+    del model
+    torch.cuda.empty_cache()
+    return rec
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,11 +494,13 @@ def main():
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--only", default=None,
                     choices=["score", "score_f32", "score_grouped", "select", "attend", "hash", "prefill_hash", "dense", "copy",
-                             "block_sparse"])
+                             "block_sparse", "step", "decode"])
     ap.add_argument("--reference-table-layout", action="store_true",
                     help="feed the scorer q_probs as [B,Hq,L,R] instead of the grouped layout the soft-hash kernel writes")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the other workloads' sub-records and the end-to-end decode runs")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of a recorded HIP graph")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -215,111 +511,20 @@ def main():
         print("bench.py needs a HIP device", file=sys.stderr)
         sys.exit(2)
 
-    from socket_amd import hash_cache, socket_kernels, sparse
-    from socket_amd.workloads import WORKLOADS, make_inputs
+    from socket_amd import hash_cache
+    from socket_amd.workloads import WORKLOADS
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.only == "block_sparse":
         block_sparse_bench(dev, max(args.steps, 1), args.warmup)
         return
-    w = WORKLOADS[args.workload]
-    t_gen = time.perf_counter()
-    inp = make_inputs(w, device=dev, device_rng=True)
-    torch.cuda.synchronize()
-    t_gen = time.perf_counter() - t_gen
-
-    B, Hq, Hkv, D, T = w.B, w.Hq, w.Hkv, w.D, w.T
-    NW = hash_cache.words_per_key(w.L, w.P)
-    Tcap = (T + 7) // 8 * 8
-    codes = torch.zeros((B, Hkv, NW, Tcap), dtype=torch.int32, device=dev)
-    v_norm = torch.zeros((B, Hkv, Tcap), dtype=torch.float16, device=dev)
-    planes_words = hash_cache.permute_planes(inp.planes)
-    lens, budgets = inp.lens, inp.budgets
-    abytes = algorithmic_bytes(w, None if lens is None else lens.cpu(), None if budgets is None else budgets.cpu())
-
-    # ---- prefill hash of the whole cache (K1 at scale) -----------------------------
-    def prefill_hash():
-        hash_cache.hash_keys_into(inp.k, inp.v, planes_words, codes, v_norm, w.L, w.P, t0=0, layout="bhsd")
-
-    if args.only == "prefill_hash":
-        us = time_launches(prefill_hash, max(args.steps, 1), warmup=args.warmup)
-        rows = B * Hkv * T
-        print(json.dumps({"only": "prefill_hash", "workload": w.name, "us": round(us, 1), "rows": rows,
-                          "mfma_tflops": round(2.0 * rows * D * NW * 32 / us / 1e6, 1)}))
+    if args.only == "decode":
+        print(json.dumps({"only": "decode", "ctx_128k": decode_tok_s(dev, 131072 - 128, 128)}))
         return
-    prefill_us = time_launches(prefill_hash, 3, warmup=1)
-    rows = B * Hkv * T
-    prefill_flops = 2.0 * rows * D * NW * 32          # columns actually contracted (incl. pad bits)
-    prefill_bytes = rows * (2 * 2 * D + 4 * NW + 2)
-    hash_report = {
-        "prefill_ms": round(prefill_us / 1e3, 3),
-        "rows": rows,
-        "mfma_tflops": round(prefill_flops / prefill_us / 1e6, 1),
-        "mfma_frac": round(prefill_flops / prefill_us / 1e6 / MFMA_BF16_PEAK_TFLOPS, 4),
-        "hbm_gbs": round(prefill_bytes / prefill_us / 1e3, 1),
-        "hbm_frac": round(prefill_bytes / prefill_us / 1e3 / HBM_PEAK_GBS, 4),
-    }
-
-    # ---- the step --------------------------------------------------------------------
-    pitch = (T + 3) // 4 * 4
-    scores_buf = torch.empty((B, Hq, pitch), dtype=torch.float32, device=dev)
-    new_pos = None
-    if lens is not None:
-        new_pos = (lens - w.new_keys).to(torch.int32)
-
-    def k_hash():
-        # the newly appended key(s) of every (sequence, kv head) land on the last
-        # position(s), so the context length is the same every step
-        hash_cache.hash_keys_into(inp.k_new, inp.v_new, planes_words, codes, v_norm, w.L, w.P,
-                                  t0=T - w.new_keys, pos_b=new_pos, layout="bshd")
-
-    # the soft-hash table in the dtype the model produces it in: the reference's
-    # soft_hash runs in the model dtype (GPT-FAST/model.py:392-401), bf16 here
-    q_table = inp.q_probs.to(torch.bfloat16) if w.dtype == torch.bfloat16 else inp.q_probs
-    q_table_f32 = q_table.float()
-
-    def k_score():
-        return hash_cache.score_packed(q_table, codes, v_norm, T, w.P, lens=lens, out=scores_buf, with_range=True)
-
-    # ... and in the layout the fused soft-hash kernel writes it in (heads of a KV head
-    # interleaved per bucket: the scorer's LDS image); same values
-    q_table_grouped = hash_cache.group_q_probs(q_table, Hkv)
-    # the step uses the layout the library asks its producers for at this shape
-    use_grouped = (not args.reference_table_layout and
-                   hash_cache._prefers_grouped(B, Hq, Hkv, T, 1 if q_table.dtype == torch.bfloat16 else 0,
-                                               w.L, w.P, q_table.shape[-1]))
-
-    def k_score_grouped():
-        return hash_cache.score_packed(q_table_grouped, codes, v_norm, T, w.P, lens=lens, out=scores_buf,
-                                       with_range=True, n_heads=Hq)
-
-    def k_score_f32():
-        return hash_cache.score_packed(q_table_f32, codes, v_norm, T, w.P, lens=lens, out=scores_buf)
-
-    def k_select(scores, rng=None):
-        return sparse.select_list(scores, w.sink, w.window, w.M, lens=lens, budgets=budgets, row_range=rng)
-
-    def k_attend(sl, ln):
-        return socket_kernels.sparse_attention_fwd(inp.q, inp.k, inp.v, sl, ln)
-
-    dense_lens = lens if lens is not None else torch.full((B,), T, dtype=torch.int32, device=dev)
-
-    def k_dense():
-        return socket_kernels.dense_decode_fwd(inp.q, inp.k, inp.v, dense_lens)
-
-    def step():
-        k_hash()
-        s, r = k_score_grouped() if use_grouped else k_score()
-        sl, ln = k_select(s, r)
-        return k_attend(sl, ln)
-
-    scores, rng = k_score_grouped() if use_grouped else k_score()
-    sl, ln = k_select(scores, rng)
-    out = k_attend(sl, ln)
-    torch.cuda.synchronize()
-
+    w = WORKLOADS[args.workload]
     iters = max(args.steps, 1)
+
     if args.only == "copy":
         # a plain device copy of known size (256 MiB read + 256 MiB written per launch):
         # the calibration kernel for the FETCH_SIZE / WRITE_SIZE counters
@@ -330,159 +535,99 @@ def main():
                           "us": round(us, 2), "gbs": round(2 * a.numel() * 4 / us / 1e3, 1), "iters": iters}))
         return
     if args.only:
-        fn = {"score": k_score, "score_f32": k_score_f32, "score_grouped": k_score_grouped, "select": lambda: k_select(scores, rng), "attend": lambda: k_attend(sl, ln),
-              "hash": k_hash, "dense": k_dense}[args.only]
+        st = Step(w, dev, reference_table_layout=args.reference_table_layout)
+        if args.only == "prefill_hash":
+            us = time_launches(st.prefill_hash, iters, warmup=args.warmup)
+            rows = w.B * w.Hkv * w.T
+            print(json.dumps({"only": "prefill_hash", "workload": w.name, "us": round(us, 1), "rows": rows,
+                              "mfma_tflops": round(2.0 * rows * w.D * w.L * w.P / us / 1e6, 1)}))
+            return
+        st.prefill_hash()
+        scores, rng = st.k_score()
+        sl, ln = st.k_select(scores, rng)
+        torch.cuda.synchronize()
+        fn = {"score": st.k_score_ref, "score_f32": st.k_score_f32, "score_grouped": st.k_score_grouped,
+              "select": lambda: st.k_select(scores, rng), "attend": lambda: st.k_attend(sl, ln), "hash": st.k_hash,
+              "dense": st.k_dense, "step": st.step}[args.only]
         us = time_launches(fn, iters, warmup=args.warmup)
+        key = args.only.replace("_grouped", "")
+        nbytes = st.abytes[key] if key in st.abytes else st.abytes["score"] + st.abytes["select"] + st.abytes["attend"]
         print(json.dumps({"only": args.only, "workload": w.name, "us": round(us, 2),
-                          "gbs": round(abytes[args.only.replace("_grouped", "")] / us / 1e3, 1), "iters": iters}))
+                          "gbs": round(nbytes / us / 1e3, 1), "iters": iters}))
         return
 
-    # ---- parity gates on the full-size run (device-side checks, not timed) --------------
-    parity = None
-    if not args.no_parity:
-        parity = {}
-        s0 = scores[0, :8]
-        n0 = T if lens is None else int(lens[0])
-        m0 = w.M if budgets is None else int(budgets[0])
-        order = torch.sort(s0[:, :n0], dim=-1, descending=True, stable=True).indices[:, :m0].to(torch.int32)
-        nbase = int(ln[0, 0]) - m0
-        parity["topk_exact_rows_checked"] = 8
-        parity["topk_exact"] = bool(torch.equal(sl[0, :8, nbase:nbase + m0], order))
-        # attention vs an fp32 gather-softmax over the same list, one sequence
-        idx = sl[0, :, :int(ln[0, 0])].long()
-        G = Hq // Hkv
-        kk = inp.k[0].repeat_interleave(G, 0).gather(1, idx.unsqueeze(-1).expand(-1, -1, D)).float()
-        vv = inp.v[0].repeat_interleave(G, 0).gather(1, idx.unsqueeze(-1).expand(-1, -1, D)).float()
-        att = torch.softmax((kk @ inp.q[0].float().unsqueeze(-1)).squeeze(-1) / D ** 0.5, -1)
-        ref = (att.unsqueeze(1) @ vv).squeeze(1)
-        parity["attend_max_abs_err"] = float((out[0].float() - ref).abs().max())
-        # scores vs an fp32 gather-sum in table order on the unpacked codes, one kv head
-        c16 = hash_cache.unpack_codes(codes[:1, :1].contiguous(), w.L, w.P, 0, n0).long()[0, 0]   # [L,T]
-        acc = torch.zeros(n0, dtype=torch.float32, device=dev)
-        for l in range(w.L):
-            acc = acc + q_table_f32[0, 0, l].gather(0, c16[l])
-        ref_s = acc * v_norm[0, 0, :n0].float()
-        parity["score_max_rel_err"] = float(((scores[0, 0, :n0] - ref_s).abs() / ref_s.abs().clamp_min(1e-30)).max())
-        del kk, vv, c16
-
-    # ---- per-kernel timings ------------------------------------------------------------------
-    per = {
-        "hash": time_launches(k_hash, iters),
-        "score": time_launches(k_score_grouped if use_grouped else k_score, iters),
-        "score_reference_layout": time_launches(k_score, iters),
-        "score_f32_table": time_launches(k_score_f32, iters),
-        "select": time_launches(lambda: k_select(scores, rng), iters),
-        "select_own_range": time_launches(lambda: k_select(scores), iters),
-        "attend": time_launches(lambda: k_attend(sl, ln), iters),
-        "dense": time_launches(k_dense, max(iters // 2, 5)),
-    }
-    kernels = {k: {"us": round(v, 2), "algorithmic_MB": round(abytes[k] / 1e6, 2),
-                   "gbs": round(abytes[k] / v / 1e3, 1), "hbm_frac": round(abytes[k] / v / 1e3 / HBM_PEAK_GBS, 4)}
-               for k, v in per.items()}
-
-    # ---- the timed region: exactly K steps -----------------------------------------------------
-    # The step is recorded once into a HIP graph (four library calls, about ten
-    # launches, no host reads) and replayed, so the Python and launch overhead of
-    # the wrappers is not what is timed; --eager times the plain calls instead.
-    # Every replay is checked against the eager result.
-    graph = None
-    if not args.eager:
-        try:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                for _ in range(2):
-                    step()
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            out_eager = step().clone()   # the state is stationary from here on (same key re-appended)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                out_graph = step()
-            for _ in range(3):
-                graph.replay()
-                torch.cuda.synchronize()
-                if not torch.equal(out_graph, out_eager):
-                    raise RuntimeError("graph replay differs from the eager step")
-        except Exception as e:  # fall back to eager launches, and say so in the result
-            print(f"bench: HIP graph capture unavailable ({e}); timing eager launches", file=sys.stderr)
-            graph = None
-    run_step = graph.replay if graph is not None else step
-    for _ in range(args.warmup):
-        run_step()
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(args.steps):
-        run_step()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    ms_per_step = e0.elapsed_time(e1) / args.steps
-    sparse_us = ms_per_step * 1e3
-    sparse_bytes = abytes["score"] + abytes["select"] + abytes["attend"]
-    kernel_sum_us = per["score"] + per["select"] + per["attend"]
-    replay_ok = None
-    if graph is not None:
-        replay_ok = bool(torch.equal(out_graph, out_eager))
-
+    # ---- the headline workload: exactly --steps timed steps after --warmup -------------------
+    rec, st, per = measure_workload(w, dev, args.steps, args.warmup, args, full=True)
     ceiling = copy_ceiling_gbs(dev)
     read_ceiling = read_ceiling_gbs(dev)
-
+    ab = st.abytes
     result = {
         "metric": "sparse-attn us/layer/step at 128k ctx (score+select+attend+hash-append), % of HBM peak"
                   if w.name == "c3" else "sparse-attn us/layer/step (score+select+attend+hash-append), % of HBM peak",
-        "value": round(sparse_us, 2),
+        "value": rec["step_us"],
         "unit": "us/layer/step",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 5),
+        "ms_per_step": round(rec["ms_per_step"], 5),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": f"{w.name}: B{B} Hq{Hq}/Hkv{Hkv} D{D} T{T} bf16 KV cache, L{w.L}xP{w.P} packed codes, "
-                               f"{str(q_table.dtype).split('.')[-1]} soft-hash table "
-                               f"({'grouped' if use_grouped else '[B,Hq,L,R]'} layout), "
-                               f"top-k {w.M} + sink {w.sink} + window {w.window}"
-                               + (", ragged lengths" if w.ragged else ""),
-                   "layers_timed": 1, "new_keys_hashed_per_step": B * Hkv * w.new_keys,
-                   "launch": "hip graph replay" if graph is not None else "eager"},
+        "config": {"workload": rec["workload"], "layers_timed": 1,
+                   "new_keys_hashed_per_step": rec["new_keys_hashed_per_step"], "launch": rec["launch"]},
         "roofline": {"kernel": "score_packed_kernel", "bound": "hbm",
-                     "achieved": round(abytes["score"] / per["score"] / 1e3, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(abytes["score"] / per["score"] / 1e3 / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(w.name)},
-        "kernels": kernels,
-        "sparse_total": {"algorithmic_MB": round(sparse_bytes / 1e6, 2), "kernel_sum_us": round(kernel_sum_us, 2),
-                         "hbm_frac_of_kernel_sum": round(sparse_bytes / kernel_sum_us / 1e3 / HBM_PEAK_GBS, 4),
-                         "hbm_frac_of_step": round(sparse_bytes / sparse_us / 1e3 / HBM_PEAK_GBS, 4),
-                         "speedup_vs_dense": round(per["dense"] / sparse_us, 3),
-                         "attend_block_seq": None},
-        "hash_prefill": hash_report,
+                     "achieved": round(ab["score"] / per["score"] / 1e3, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(ab["score"] / per["score"] / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+                     "traffic_source": MEASURED_TRAFFIC_SOURCE if MEASURED_TRAFFIC_BYTES.get(w.name) else None},
+        "kernels": rec["kernels"],
+        "kernel_timing": rec["kernel_timing"],
+        "sparse_total": rec["sparse_total"],
+        "hash_prefill": rec["hash_prefill"],
         "copy_ceiling_gbs": round(ceiling, 1),
         "read_ceiling_gbs": round(read_ceiling, 1),
-        "parity": parity,
-        "graph_replay_equals_eager": replay_ok,
-        "wall_ms_timed_region": round(wall_ms, 2),
-        "input_generation_s": round(t_gen, 1),
+        "parity": rec["parity"],
+        "graph_replay_equals_eager": rec["graph_replay_equals_eager"],
+        "wall_ms_timed_region": rec["wall_ms_timed_region"],
+        "input_generation_s": rec["input_generation_s"],
     }
-    from socket_amd._lib import lib
-    result["sparse_total"]["attend_block_seq"] = lib().socket_sparse_attention_block_seq(B, Hq, sl.shape[-1])
 
     if not args.no_cpu:
+        T, Hkv, Hq = w.T, w.Hkv, w.Hq
+        lens, budgets = st.lens, st.budgets
         n0 = T if lens is None else int(lens[0])
         m0 = w.M if budgets is None else int(budgets[0])
         nkv = min(2, Hkv)
         G = Hq // Hkv
-        inp_cpu = {"q": inp.q.cpu(), "q_probs": inp.q_probs[:1, :nkv * G].cpu(), "k": inp.k[:1, :nkv].cpu(),
-                   "v": inp.v[:1, :nkv].cpu(), "len0": n0, "m0": m0,
-                   "tok_total": B * T if lens is None else int(lens.sum())}
-        codes_cpu = hash_cache.unpack_codes(codes[:1, :nkv].contiguous(), w.L, w.P, 0, n0).cpu()
-        result["cpu_baseline"] = cpu_baseline(w, inp_cpu, codes_cpu, v_norm[:1, :nkv].cpu())
+        inp_cpu = {"q": st.inp.q.cpu(), "q_probs": st.inp.q_probs[:1, :nkv * G].cpu(), "k": st.inp.k[:1, :nkv].cpu(),
+                   "v": st.inp.v[:1, :nkv].cpu(), "len0": n0, "m0": m0,
+                   "tok_total": w.B * T if lens is None else int(lens.sum())}
+        codes_cpu = hash_cache.unpack_codes(st.codes[:1, :nkv].contiguous(), w.L, w.P, 0, n0).cpu()
+        vn_cpu = st.v_norm[:1, :nkv].cpu()
+    del st
+    torch.cuda.empty_cache()
+
+    # ---- the other single-layer workloads and the end-to-end decode runs ---------------------
+    if not args.no_extra and args.workload == "c3":
+        sub_steps = max(10, args.steps // 2)
+        for name in ("c2", "c5"):
+            r, s2, _ = measure_workload(WORKLOADS[name], dev, sub_steps, 3, args, full=False)
+            for k in ("ms_per_step", "parity", "input_generation_s", "kernel_timing"):
+                r.pop(k, None)
+            r["steps"] = sub_steps
+            result[name] = r
+            del s2
+            torch.cuda.empty_cache()
+        # the metric's second half: decode tokens per second at 128k context (prompt
+        # 130944 + 128 new tokens = the model's block_size), and configuration 4 as BASELINE
+        # states it (65536-token prompt, 256 greedy tokens)
+        result["decode_tok_s"] = {"ctx_128k": decode_tok_s(dev, 131072 - 128, 128),
+                                  "c4_prompt_65536": decode_tok_s(dev, 65536, 256)}
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(w, inp_cpu, codes_cpu, vn_cpu)
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result))
