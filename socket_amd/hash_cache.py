@@ -27,6 +27,9 @@ from .socket_kernels import sparse_attention_fwd
 from .sparse import select_list
 
 
+HASH_DIM = 128     # coordinates the hashing kernel contracts over
+
+
 def words_per_key(L: int, P: int) -> int:
     nw = lib().socket_words_per_key(int(L), int(P))
     if nw <= 0:
@@ -36,9 +39,15 @@ def words_per_key(L: int, P: int) -> int:
 
 @torch.no_grad()
 def permute_planes(planes_lpd: torch.Tensor) -> torch.Tensor:
-    """[L,P,D] hyperplanes -> bf16 [NW*32, D] in packed-bit column order."""
+    """[L,P,D] hyperplanes -> bf16 [NW*32, D] in packed-bit column order.  The
+    hashing kernel contracts over 128 coordinates: planes of a narrower head are
+    padded with zeros up to 128 (`hash_keys_into` pads the rows to match; a zero
+    coordinate changes no projection)."""
     assert planes_lpd.is_cuda and planes_lpd.dim() == 3
     L, P, D = planes_lpd.shape
+    if D < HASH_DIM:
+        planes_lpd = torch.nn.functional.pad(planes_lpd, (0, HASH_DIM - D))
+        D = HASH_DIM
     planes_lpd = planes_lpd.contiguous()
     out = torch.empty((words_per_key(L, P) * 32, D), dtype=torch.bfloat16, device=planes_lpd.device)
     check("socket_permute_planes", lib().socket_permute_planes(
@@ -65,6 +74,18 @@ def hash_keys_into(k: torch.Tensor, v: Optional[torch.Tensor], planes_words: tor
     else:
         raise ValueError(layout)
     assert k.stride(-1) == 1 and (v is None or (v.stride(-1) == 1 and v.shape == k.shape and v.dtype == k.dtype))
+    if D < HASH_DIM and planes_words.shape[1] == HASH_DIM and S > 0:
+        # a narrower head: the new rows are padded with zeros to the kernel's 128 coordinates
+        # (same sign bits, same value norms); strides are then those of the padded copies
+        k = torch.nn.functional.pad(k, (0, HASH_DIM - D))
+        v = None if v is None else torch.nn.functional.pad(v, (0, HASH_DIM - D))
+        D = HASH_DIM
+        if layout == "bhsd":
+            ks = (k.stride(0), k.stride(1), k.stride(2))
+            vs = (v.stride(0), v.stride(1), v.stride(2)) if v is not None else (0, 0, 0)
+        else:
+            ks = (k.stride(0), k.stride(2), k.stride(1))
+            vs = (v.stride(0), v.stride(2), v.stride(1)) if v is not None else (0, 0, 0)
     NW, Tcap = codes.shape[2], codes.shape[3]
     assert codes.shape[0] == B and codes.shape[1] == Hkv and NW == words_per_key(L, P)
     if v is not None:

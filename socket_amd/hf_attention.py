@@ -98,15 +98,19 @@ class SocketLlamaAttention(nn.Module):
         self._rng_cache = {}
 
     # ---- planes, prototypes, hashes (modeling_llama.py:458-638) --------------------------
+    PLANE_SEED_OFFSET = 7777      # modeling_llama.py:463 seeds its plane generator with seed + 7777
+
     def _rng(self, device) -> Optional[torch.Generator]:
+        """One seeded generator per device for drawing the hyperplanes (none when the
+        seed is unset: planes then come from torch's default generator)."""
         if self._seed is None:
             return None
-        g = self._rng_cache.get(device)
-        if g is None:
-            g = torch.Generator(device=device)
-            g.manual_seed(int(self._seed) + 7777)
-            self._rng_cache[device] = g
-        return g
+        try:
+            return self._rng_cache[device]
+        except KeyError:
+            gen = torch.Generator(device=device).manual_seed(int(self._seed) + self.PLANE_SEED_OFFSET)
+            self._rng_cache[device] = gen
+            return gen
 
     def get_hyper_planes(self, cache, D: int, L: int, P: int, device, dtype, rng=None) -> torch.Tensor:
         key = (D, device, dtype, L, P)
@@ -158,13 +162,14 @@ class SocketLlamaAttention(nn.Module):
         return int(size * N) if isinstance(size, float) else int(size)
 
     def _get_states_container(self, past_key_values, runtime_states):
-        if past_key_values is not None:
-            states = getattr(past_key_values, "bucket_states", None)
-            if states is None:
-                states = {}
-                setattr(past_key_values, "bucket_states", states)
-            return states
-        return {} if runtime_states is None else runtime_states
+        """Where the per-layer hash state lives between decode steps: on the HF cache
+        object (attribute `bucket_states`, created on first use) when there is one,
+        else in the dict the caller passes (modeling_llama.py:651-678)."""
+        if past_key_values is None:
+            return runtime_states if runtime_states is not None else {}
+        if not hasattr(past_key_values, "bucket_states") or past_key_values.bucket_states is None:
+            past_key_values.bucket_states = {}
+        return past_key_values.bucket_states
 
     # ---- bucket state ----------------------------------------------------------------------------
     def _hash_append(self, st: dict, k: torch.Tensor, v: torch.Tensor, T_k: int) -> None:

@@ -373,7 +373,10 @@ class Attention(nn.Module):
     # ---- hashes (GPT-FAST/model.py:392-413) ------------------------------------------
     def soft_hash(self, queries_bhd: Tensor) -> Tensor:
         """softmax_r( tanh(q . planes) / sqrt(D) @ protos_T ): [B,H,D] -> [B,H,L,R].
-        One fused kernel on the device; the torch expression below on the host."""
+        One fused kernel on the device.  For tensors on the host the reference's own
+        torch expression is evaluated instead: that branch exists for the host-side
+        tests of the glue (tests/test_model_cpu.py) and is not a decode path -- the
+        attention step itself has no host route."""
         if queries_bhd.is_cuda:
             return _soft_hash(queries_bhd, self.planes, self.protos_T, self.n_local_heads)
         proj = torch.einsum("bhd,lkd->bhlk", queries_bhd, self.planes)
@@ -392,7 +395,8 @@ class Attention(nn.Module):
         """int16 codes [B,S,Hkv,L] of keys [B,S,Hkv,D]: sign bits of the K
         projections of each table, zero counting as set.  On the device the
         packed words come from the hashing kernel and are unpacked into the
-        reference's layout; the cache itself never takes this detour."""
+        reference's layout; the cache itself never takes this detour.  (Host
+        tensors: the reference's einsum, for the host-side tests only.)"""
         if keys_bshd.is_cuda:
             B, S, H, _ = keys_bshd.shape
             NW = hash_cache.words_per_key(self.L, self.K)
@@ -428,7 +432,8 @@ class Attention(nn.Module):
         if sparse:
             T = cache.k_cache.size(2)       # upper bound; the kernels stop at cache.lens
             cfg = self.config
-            # on the device the table is written in the layout the scorer prefers (same values)
+            # on the device the table is written in the layout the scorer prefers (same values);
+            # host tensors only occur in the host-side tests, whose checker stands in for the step
             q_probs = (_soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, T)
                        if q_bhd.is_cuda else self.soft_hash(q_bhd))
             out_bhd = _sparse_step(q_bhd, q_probs, cache, T, int(cfg.sink_size), int(cfg.window_size),

@@ -113,6 +113,29 @@ def hash_cache_planes(dev):
     return hash_cache.permute_planes(torch.randn(20, 10, 128, generator=g).to(dev))
 
 
+def test_sparse_hook_with_64_dim_heads(dev, monkeypatch):
+    """A model whose heads are 64 wide (the hashing kernel contracts over 128
+    coordinates: rows and planes are zero-padded on the way in): cached codes
+    equal the oracle's hash of the cached keys, logits equal the oracle hook's."""
+    model = toy_model(dev, torch.float32, n_head=8, n_local_heads=4)
+    assert model.config.head_dim == 64
+    g = torch.Generator().manual_seed(31)
+    ids = torch.randint(0, 331, (2, 120), generator=g).to(dev)
+    model.setup_caches(2, 128)
+    have = _run_steps(model, ids, 110)
+    attn, cache = model.layers[1].attention, model.layers[1].attention.kv_cache
+    # (the kernel contracts keys and planes rounded to bf16, with fp32 accumulation)
+    keys = cache.k_cache[:, :, :120].permute(0, 2, 1, 3).cpu().to(torch.bfloat16).float()
+    proj = orc.projections_f64(keys, attn.planes.float().cpu().to(torch.bfloat16).float())
+    clear = (proj.abs() > 1e-3 * proj.abs().mean()).all(-1)
+    assert clear.float().mean() > 0.9
+    assert torch.equal(cache.k_hard(120).cpu().permute(0, 2, 1, 3)[clear], orc.pack_bits(proj >= 0)[clear])
+    _reset(model)
+    oracle_backend.install(monkeypatch, M, hashing=False, sparse=True, dense=False)
+    want = _run_steps(model, ids, 110)
+    assert float((have - want).abs().max()) <= 2e-3 * max(float(want.abs().max()), 1.0)
+
+
 def test_cache_hash_state_after_prefill_and_decode(dev):
     """Codes and value norms written by the fused append equal the oracle's hash
     of the cached rows wherever the fp64 projection is clear of zero."""
