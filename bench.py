@@ -42,10 +42,14 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 BOX_CPU_SHARE = 16              # host cores a one-GPU job is given on the benchmark box
 
 # HBM bytes per launch of the scorer from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of `bench.py --only score` (see profiles/), keyed by workload; None until
-# a counter run for that workload has been recorded there.
-MEASURED_TRAFFIC_BYTES = {}
-MEASURED_TRAFFIC_SOURCE = None
+# runs of `bench.py --only score_grouped` (profiles/score_packed_c3_hbm_counters.txt
+# holds the commands, the raw counters and the calibration), keyed by workload;
+# None until a counter run for that workload has been recorded there.  The profiler
+# cannot run inside this process, so the figure is a recorded one and says so.
+MEASURED_TRAFFIC_BYTES = {"c3": int(187240 * 1024 * 2.000 + 65618 * 1024 * 1.000)}
+MEASURED_TRAFFIC_SOURCE = ("recorded, not measured in this run: rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated on a 1 GiB "
+                           "read stream of the same request width) + WRITE_SIZE (x1.000, device copy); "
+                           "profiles/score_packed_c3_hbm_counters.txt")
 
 
 def algorithmic_bytes(w, lens=None, budgets=None):
@@ -494,7 +498,7 @@ def main():
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--only", default=None,
                     choices=["score", "score_f32", "score_grouped", "select", "attend", "hash", "prefill_hash", "dense", "copy",
-                             "block_sparse", "step", "decode"])
+                             "block_sparse", "step", "decode", "read_probe"])
     ap.add_argument("--reference-table-layout", action="store_true",
                     help="feed the scorer q_probs as [B,Hq,L,R] instead of the grouped layout the soft-hash kernel writes")
     ap.add_argument("--no-cpu", action="store_true")
@@ -518,6 +522,13 @@ def main():
     torch.cuda.set_device(dev)
     if args.only == "block_sparse":
         block_sparse_bench(dev, max(args.steps, 1), args.warmup)
+        return
+    if args.only == "read_probe":
+        # a pure read stream of known size (1 GiB of bf16 weights through the matrix-vector
+        # kernel, 16-byte non-temporal loads): the calibration kernel for FETCH_SIZE when the
+        # kernel under study issues full-width read requests, as the scorer's code stream does
+        print(json.dumps({"only": "read_probe", "bytes_read": 131072 * 4096 * 2,
+                          "gbs": round(read_ceiling_gbs(dev), 1)}))
         return
     if args.only == "decode":
         print(json.dumps({"only": "decode", "ctx_128k": decode_tok_s(dev, 131072 - 128, 128)}))
