@@ -294,14 +294,17 @@ int socket_sparse_attention(const void* q, const void* k, const void* v, int dty
  * allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * The per-split partials go to a fixed array of SOCKET_STATIC_SCRATCH_BYTES in
- * device memory that belongs to the library's image (each GPU the library runs
- * on holds one copy until the process ends); a call whose
- * socket_sparse_attention_workspace_bytes(B, Hq, D, max_len) exceeds that size
- * returns SOCKET_ERR_WORKSPACE and launches nothing.  The call allocates and
- * frees nothing.  All calls on one GPU share the array: calls that overlap in
- * time on the same GPU (different streams or threads) race; serialise them.
- * Same results as socket_sparse_attention.
- * socket_static_scratch_init looks the array's device address up for the current
+ * device memory that belongs to the library's image, next to 65536 row counters
+ * (each GPU the library runs on holds one copy until the process ends); a call
+ * whose socket_sparse_attention_workspace_bytes(B, Hq, D, max_len) exceeds that
+ * size, or with more than 65536 (b, h) rows, returns SOCKET_ERR_WORKSPACE and
+ * launches nothing.  The call allocates and frees nothing, and it is ONE launch:
+ * the workgroup that completes a row's last split merges the row's splits (the
+ * counters are zero between calls: tickets are drawn with a wrapping increment).
+ * All calls on one GPU share the arrays: calls that overlap in time on the same
+ * GPU (different streams or threads) race; serialise them.
+ * Same results as socket_sparse_attention, bit for bit.
+ * socket_static_scratch_init looks the arrays' device addresses up for the current
  * device ahead of the first call (optional; the first call does it otherwise). */
 #define SOCKET_STATIC_SCRATCH_BYTES (4u << 20)
 size_t socket_static_scratch_bytes(void);

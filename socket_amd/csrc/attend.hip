@@ -27,6 +27,18 @@ constexpr int kUnroll = 4;
 
 __device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
 
+// Stores and loads that are coherent across the whole GPU without a fence: the
+// store is written through to where every compute die sees it, the load does not
+// take a copy from this die's caches.  (A device-scope fence instead writes back
+// everything dirty in the die's L2 -- the scores the scorer has just written
+// among it -- and made the one-launch attention slower than two launches.)
+__device__ __forceinline__ void store_coherent(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_coherent(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Merge (m, l, acc) pairs of an online softmax.
 template <int E>
 __device__ __forceinline__ void merge_state(float& m, float& l, float* acc, float m2, float l2,
@@ -42,7 +54,7 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* acc, floa
 
 // Final merge of the workgroup's states and the split's output.  Every lane
 // holds the state of (row slot, column chunk); GH heads per lane.
-template <int E, int LPR, int GH>
+template <int E, int LPR, int GH, bool COHERENT = false>
 __device__ __forceinline__ void finish_split(float (&m)[GH], float (&l)[GH], float (&acc)[GH][E],
                                              int G, float* mid_o_base, float* mid_lse_base,
                                              int64_t head_stride_o, int64_t head_stride_lse,
@@ -93,19 +105,122 @@ __device__ __forceinline__ void finish_split(float (&m)[GH], float (&l)[GH], flo
       val += rec[d] * sc;
     }
     const bool any = Lsum > 0.f;
-    mid_o_base[g * head_stride_o + d] = any ? val / Lsum : 0.f;
-    if (d == 0) mid_lse_base[g * head_stride_lse] = any ? M + logf(Lsum) : -INFINITY;
+    if (COHERENT) {
+      store_coherent(mid_o_base + g * head_stride_o + d, any ? val / Lsum : 0.f);
+      if (d == 0) store_coherent(mid_lse_base + g * head_stride_lse, any ? M + logf(Lsum) : -INFINITY);
+    } else {
+      mid_o_base[g * head_stride_o + d] = any ? val / Lsum : 0.f;
+      if (d == 0) mid_lse_base[g * head_stride_lse] = any ? M + logf(Lsum) : -INFINITY;
+    }
   }
 }
 
-template <class DT, int D>
+constexpr int kMergeThreads = 256;
+
+// Merge of the per-split partials of one (b, h) by a workgroup of 256 lanes: the
+// largest log-sum-exp first, then the lanes, four output coordinates each and
+// 256 / (D/4) splits side by side, add up weight * partial with independent
+// loads, and LDS folds the side-by-side groups.
+template <int D, bool COHERENT = false>
+__device__ __forceinline__ void merge_splits(const float* mo, const float* ml, int nblk, void* __restrict__ out,
+                                             int out_dtype, int64_t out_off) {
+  constexpr int LPD = D / 4;                    // lanes across the head dimension
+  constexpr int NG = kMergeThreads / LPD;       // splits handled side by side
+  constexpr int kW = kMergeThreads / SOCKET_WAVE;
+  __shared__ float red[kW];
+  __shared__ float part[NG][D + 4];
+  __shared__ float psum[NG];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+
+  float m = -INFINITY;
+  for (int s = tid; s < nblk; s += kMergeThreads) m = fmaxf(m, COHERENT ? load_coherent(ml + s) : ml[s]);
+#pragma unroll
+  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, SOCKET_WAVE));
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = red[0];
+#pragma unroll
+  for (int w = 1; w < kW; ++w) m = fmaxf(m, red[w]);
+
+  const int grp = tid / LPD, d4 = (tid % LPD) * 4;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float sum = 0.f;
+  for (int s = grp; s < nblk; s += NG) {
+    const float lse = COHERENT ? load_coherent(ml + s) : ml[s];
+    // a split without a live row has lse = -inf and weight 0; so has every split
+    // when nothing at all was attended (m = -inf), which leaves 0/0 below
+    const float w = (lse == -INFINITY) ? 0.f : fast_exp(lse - m);
+    float4 o;
+    if (COHERENT) {
+      const float* src = mo + (int64_t)s * D + d4;
+      o = make_float4(load_coherent(src), load_coherent(src + 1), load_coherent(src + 2), load_coherent(src + 3));
+    } else {
+      o = *reinterpret_cast<const float4*>(mo + (int64_t)s * D + d4);
+    }
+    acc.x += w * o.x;
+    acc.y += w * o.y;
+    acc.z += w * o.z;
+    acc.w += w * o.w;
+    sum += w;
+  }
+  part[grp][d4] = acc.x;
+  part[grp][d4 + 1] = acc.y;
+  part[grp][d4 + 2] = acc.z;
+  part[grp][d4 + 3] = acc.w;
+  if (d4 == 0) psum[grp] = sum;
+  __syncthreads();
+  if (tid < D) {
+    float a = 0.f, t = 0.f;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      a += part[g][tid];
+      t += psum[g];
+    }
+    const float r = a / t;  // 0/0 -> NaN when nothing was attended, as the reference
+    const int64_t o = out_off + tid;
+    if (out_dtype == SOCKET_F32) store_elem<DType_f32>(out, o, r);
+    else if (out_dtype == SOCKET_BF16) store_elem<DType_bf16>(out, o, r);
+    else store_elem<DType_f16>(out, o, r);
+  }
+}
+
+// One workgroup per (b, h): the merge as a launch of its own.
+template <int D>
+__global__ __launch_bounds__(kMergeThreads) void stage2_kernel(
+    const float* __restrict__ mid_o, const float* __restrict__ mid_lse,
+    const int32_t* __restrict__ sparse_len, int64_t len_sb, int64_t len_sh, void* __restrict__ out,
+    int out_dtype, int64_t out_sb, int64_t out_sh, int Hq, int nsplit, int block_seq) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int len = sparse_len[b * len_sb + h * len_sh];
+  // (a length beyond nsplit * block_seq is cut to the splits that exist)
+  int nblk = len <= 0 ? 0 : (len + block_seq - 1) / block_seq;
+  nblk = min(nblk, nsplit);
+  merge_splits<D>(mid_o + ((int64_t)b * Hq + h) * nsplit * D, mid_lse + ((int64_t)b * Hq + h) * nsplit, nblk, out,
+                  out_dtype, b * out_sb + h * out_sh);
+}
+
+// FINISH: the workgroup that completes a row's last outstanding split also merges
+// the splits (what stage2_kernel does), so the whole attention is one launch.
+// `arrive` holds one counter per row that is zero between launches: every split
+// with work takes a ticket with a wrapping increment after publishing its partial
+// result, the one that draws the last ticket finds the counter back at zero and
+// every other split's result visible.
+struct Stage1Finish {
+  unsigned int* arrive;
+  void* out;
+  int out_dtype;
+  int64_t out_sb, out_sh;
+};
+
+template <class DT, int D, bool FINISH>
 __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
     const void* __restrict__ q_, const void* __restrict__ k_, const void* __restrict__ v_,
     int64_t q_sb, int64_t q_sh, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb,
     int64_t v_sh, int64_t v_ss, const int32_t* __restrict__ sparse_list, int64_t list_sb,
     int64_t list_sh, const int32_t* __restrict__ sparse_len, int64_t len_sb, int64_t len_sh,
     float* __restrict__ mid_o, float* __restrict__ mid_lse, int Hq, int G, int kv_rows, int list_width,
-    int nsplit, int block_seq, float sm_scale) {
+    int nsplit, int block_seq, float sm_scale, Stage1Finish fin) {
   typedef typename DT::storage ST;
   constexpr int E = DT::kPer16B;
   constexpr int LPR = D / E;
@@ -117,6 +232,17 @@ __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
   const int len = min(sparse_len[b * len_sb + h * len_sh], list_width);
   const int lo = s * block_seq;
   const int hi = min(len, lo + block_seq);
+  if (FINISH && s == 0 && len <= 0) {
+    // nothing listed: no split runs for this row; the reference's 0/0
+    if (threadIdx.x < D) {
+      const int64_t o = b * fin.out_sb + h * fin.out_sh + threadIdx.x;
+      const float nan = __uint_as_float(0x7fc00000u);
+      if (fin.out_dtype == SOCKET_F32) store_elem<DType_f32>(fin.out, o, nan);
+      else if (fin.out_dtype == SOCKET_BF16) store_elem<DType_bf16>(fin.out, o, nan);
+      else store_elem<DType_f16>(fin.out, o, nan);
+    }
+    return;
+  }
   if (hi <= lo) return;
   const int kvh = h / G;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -187,78 +313,21 @@ __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
 
   float* mo = mid_o + (((int64_t)b * Hq + h) * nsplit + s) * D;
   float* ml = mid_lse + ((int64_t)b * Hq + h) * nsplit + s;
-  finish_split<E, LPR, 1>(m, l, acc, 1, mo, ml, 0, 0, lds);
-}
-
-constexpr int kMergeThreads = 256;
-
-// Merge of the per-split partials.  One workgroup of 256 lanes per (b, h): the
-// largest log-sum-exp first, then the lanes, four output coordinates each and
-// 256 / (D/4) splits side by side, add up weight * partial with independent
-// loads, and LDS folds the side-by-side groups.
-template <int D>
-__global__ __launch_bounds__(kMergeThreads) void stage2_kernel(
-    const float* __restrict__ mid_o, const float* __restrict__ mid_lse,
-    const int32_t* __restrict__ sparse_len, int64_t len_sb, int64_t len_sh, void* __restrict__ out,
-    int out_dtype, int64_t out_sb, int64_t out_sh, int Hq, int nsplit, int block_seq) {
-  // (a length beyond nsplit * block_seq is cut to the splits that exist, below)
-  constexpr int LPD = D / 4;                    // lanes across the head dimension
-  constexpr int NG = kMergeThreads / LPD;       // splits handled side by side
-  constexpr int kW = kMergeThreads / SOCKET_WAVE;
-  __shared__ float red[kW];
-  __shared__ float part[NG][D + 4];
-  __shared__ float psum[NG];
-  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int len = sparse_len[b * len_sb + h * len_sh];
-  int nblk = len <= 0 ? 0 : (len + block_seq - 1) / block_seq;
-  nblk = min(nblk, nsplit);
-  const float* mo = mid_o + ((int64_t)b * Hq + h) * nsplit * D;
-  const float* ml = mid_lse + ((int64_t)b * Hq + h) * nsplit;
-
-  float m = -INFINITY;
-  for (int s = tid; s < nblk; s += kMergeThreads) m = fmaxf(m, ml[s]);
-#pragma unroll
-  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, SOCKET_WAVE));
-  if (lane == 0) red[wave] = m;
-  __syncthreads();
-  m = red[0];
-#pragma unroll
-  for (int w = 1; w < kW; ++w) m = fmaxf(m, red[w]);
-
-  const int grp = tid / LPD, d4 = (tid % LPD) * 4;
-  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-  float sum = 0.f;
-  for (int s = grp; s < nblk; s += NG) {
-    const float lse = ml[s];
-    // a split without a live row has lse = -inf and weight 0; so has every split
-    // when nothing at all was attended (m = -inf), which leaves 0/0 below
-    const float w = (lse == -INFINITY) ? 0.f : fast_exp(lse - m);
-    const float4 o = *reinterpret_cast<const float4*>(mo + (int64_t)s * D + d4);
-    acc.x += w * o.x;
-    acc.y += w * o.y;
-    acc.z += w * o.z;
-    acc.w += w * o.w;
-    sum += w;
-  }
-  part[grp][d4] = acc.x;
-  part[grp][d4 + 1] = acc.y;
-  part[grp][d4 + 2] = acc.z;
-  part[grp][d4 + 3] = acc.w;
-  if (d4 == 0) psum[grp] = sum;
-  __syncthreads();
-  if (tid < D) {
-    float a = 0.f, t = 0.f;
-#pragma unroll
-    for (int g = 0; g < NG; ++g) {
-      a += part[g][tid];
-      t += psum[g];
-    }
-    const float r = a / t;  // 0/0 -> NaN when nothing was attended, as the reference
-    const int64_t o = b * out_sb + h * out_sh + tid;
-    if (out_dtype == SOCKET_F32) store_elem<DType_f32>(out, o, r);
-    else if (out_dtype == SOCKET_BF16) store_elem<DType_bf16>(out, o, r);
-    else store_elem<DType_f16>(out, o, r);
+  finish_split<E, LPR, 1, FINISH>(m, l, acc, 1, mo, ml, 0, 0, lds);
+  if (FINISH) {
+    __shared__ int last;
+    const int nblk = min((len + block_seq - 1) / block_seq, nsplit);   // splits of this row that run
+    // Every lane waits until its written-through stores of the partial result have been
+    // acknowledged, the barrier collects the lanes, and only then is the ticket drawn
+    // (an atomic at the same, device-wide, level): whoever draws a later ticket can read
+    // this split's result.  No fence: see store_coherent.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) last = atomicInc(&fin.arrive[b * Hq + h], (unsigned int)(nblk - 1)) == (unsigned int)(nblk - 1);
+    __syncthreads();
+    if (!last) return;
+    merge_splits<D, true>(mid_o + ((int64_t)b * Hq + h) * nsplit * D, mid_lse + ((int64_t)b * Hq + h) * nsplit,
+                          nblk, fin.out, fin.out_dtype, b * fin.out_sb + h * fin.out_sh);
   }
 }
 
@@ -397,11 +466,18 @@ template <class DT, int D>
 void launch_sparse_stage1(const AttArgs& a, const int32_t* list, int64_t list_sb, int64_t list_sh,
                           const int32_t* len, int64_t len_sb, int64_t len_sh, float* mid_o,
                           float* mid_lse, int B, int Hq, int Hkv, int kv_rows, int list_width,
-                          int nsplit, int block_seq, hipStream_t s) {
-  hipLaunchKernelGGL((sparse_stage1_kernel<DT, D>), dim3(nsplit, Hq, B), dim3(kAttThreads), 0, s,
-                     a.q, a.k, a.v, a.q_sb, a.q_sh, a.k_sb, a.k_sh, a.k_ss, a.v_sb, a.v_sh, a.v_ss,
-                     list, list_sb, list_sh, len, len_sb, len_sh, mid_o, mid_lse, Hq, Hq / Hkv,
-                     kv_rows, list_width, nsplit, block_seq, 1.0f / sqrtf((float)D));
+                          int nsplit, int block_seq, const Stage1Finish* fin, hipStream_t s) {
+#define SOCKET_S1_ARGS                                                                               \
+  a.q, a.k, a.v, a.q_sb, a.q_sh, a.k_sb, a.k_sh, a.k_ss, a.v_sb, a.v_sh, a.v_ss, list, list_sb, list_sh, \
+      len, len_sb, len_sh, mid_o, mid_lse, Hq, Hq / Hkv, kv_rows, list_width, nsplit, block_seq,      \
+      1.0f / sqrtf((float)D)
+  if (fin)
+    hipLaunchKernelGGL((sparse_stage1_kernel<DT, D, true>), dim3(nsplit, Hq, B), dim3(kAttThreads), 0, s,
+                       SOCKET_S1_ARGS, *fin);
+  else
+    hipLaunchKernelGGL((sparse_stage1_kernel<DT, D, false>), dim3(nsplit, Hq, B), dim3(kAttThreads), 0, s,
+                       SOCKET_S1_ARGS, Stage1Finish{});
+#undef SOCKET_S1_ARGS
 }
 
 template <class DT, int D>
@@ -452,15 +528,15 @@ int dense_rows_per_split(int B, int Hkv, int T) {
 
 }  // namespace
 
-extern "C" int socket_attend_stage1(const void* q, const void* k, const void* v, int dtype,
-                                    int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_b,
-                                    int64_t k_stride_h, int64_t k_stride_s, int64_t v_stride_b,
-                                    int64_t v_stride_h, int64_t v_stride_s,
-                                    const int32_t* sparse_list, int64_t list_stride_b,
-                                    int64_t list_stride_h, const int32_t* sparse_len,
-                                    int64_t len_stride_b, int64_t len_stride_h, float* mid_o,
-                                    float* mid_lse, int B, int Hq, int Hkv, int D, int kv_rows,
-                                    int list_width, int nsplit, int block_seq, void* stream) {
+namespace {
+
+int attend_stage1(const void* q, const void* k, const void* v, int dtype, int64_t q_stride_b,
+                  int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                  int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s, const int32_t* sparse_list,
+                  int64_t list_stride_b, int64_t list_stride_h, const int32_t* sparse_len,
+                  int64_t len_stride_b, int64_t len_stride_h, float* mid_o, float* mid_lse, int B, int Hq,
+                  int Hkv, int D, int kv_rows, int list_width, int nsplit, int block_seq,
+                  const Stage1Finish* fin, void* stream) {
   AttArgs a{q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h, k_stride_s,
             v_stride_b, v_stride_h, v_stride_s};
   int st = check_common(a, B, Hq, Hkv, D);
@@ -468,11 +544,12 @@ extern "C" int socket_attend_stage1(const void* q, const void* k, const void* v,
   SOCKET_REQUIRE(sparse_list && sparse_len && mid_o && mid_lse, SOCKET_ERR_NULL);
   SOCKET_REQUIRE(nsplit > 0 && nsplit <= 65535 * 32 && block_seq > 0 && kv_rows > 0 && list_width > 0,
                  SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(socket_aligned16(mid_o), SOCKET_ERR_ALIGN);
   hipStream_t s = (hipStream_t)stream;
 #define SOCKET_S1(DT, DD)                                                                          \
   launch_sparse_stage1<DT, DD>(a, sparse_list, list_stride_b, list_stride_h, sparse_len,           \
                                len_stride_b, len_stride_h, mid_o, mid_lse, B, Hq, Hkv, kv_rows,    \
-                               list_width, nsplit, block_seq, s)
+                               list_width, nsplit, block_seq, fin, s)
 #define SOCKET_S1_D(DD)                                    \
   do {                                                     \
     if (dtype == SOCKET_BF16) SOCKET_S1(DType_bf16, DD);   \
@@ -487,6 +564,23 @@ extern "C" int socket_attend_stage1(const void* q, const void* k, const void* v,
 #undef SOCKET_S1
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
+}
+
+}  // namespace
+
+extern "C" int socket_attend_stage1(const void* q, const void* k, const void* v, int dtype,
+                                    int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_b,
+                                    int64_t k_stride_h, int64_t k_stride_s, int64_t v_stride_b,
+                                    int64_t v_stride_h, int64_t v_stride_s,
+                                    const int32_t* sparse_list, int64_t list_stride_b,
+                                    int64_t list_stride_h, const int32_t* sparse_len,
+                                    int64_t len_stride_b, int64_t len_stride_h, float* mid_o,
+                                    float* mid_lse, int B, int Hq, int Hkv, int D, int kv_rows,
+                                    int list_width, int nsplit, int block_seq, void* stream) {
+  return attend_stage1(q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h, k_stride_s, v_stride_b,
+                       v_stride_h, v_stride_s, sparse_list, list_stride_b, list_stride_h, sparse_len,
+                       len_stride_b, len_stride_h, mid_o, mid_lse, B, Hq, Hkv, D, kv_rows, list_width, nsplit,
+                       block_seq, nullptr, stream);
 }
 
 extern "C" int socket_attend_stage2(const float* mid_o, const float* mid_lse,
@@ -575,23 +669,34 @@ extern "C" int socket_sparse_attention(const void* q, const void* k, const void*
 // image.  Every GPU the library runs on holds its own copy until the process ends.
 // ---------------------------------------------------------------------------
 static __device__ __align__(256) unsigned char scratch[SOCKET_STATIC_SCRATCH_BYTES];
+// One arrival counter per (b, h) row for the launch that also merges the splits.
+// Zero when the library is loaded and zero again after every call: the tickets are
+// drawn with a wrapping increment, so the split that completes a row leaves its
+// counter at zero.
+constexpr int kArriveRows = 65536;
+static __device__ unsigned int arrive_counters[kArriveRows];
 
 namespace {
 
 constexpr int kMaxDevices = 64;
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
+std::atomic<void*> g_arrive_ptr[kMaxDevices];
 
-// Device address of `scratch` on the current device (the array's name is only a
-// host-side handle).  Looked up once per device; no allocation.
-int static_scratch(void** out) {
+// Device addresses of `scratch` and `arrive_counters` on the current device (the
+// arrays' names are only host-side handles).  Looked up once per device; no allocation.
+int static_scratch(void** out, unsigned int** arrive) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return SOCKET_ERR_LAUNCH;
   void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
-  if (!p) {
+  void* c = g_arrive_ptr[dev].load(std::memory_order_acquire);
+  if (!p || !c) {
     if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return SOCKET_ERR_LAUNCH;
-    g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same address
+    if (hipGetSymbolAddress(&c, HIP_SYMBOL(arrive_counters)) != hipSuccess || !c) return SOCKET_ERR_LAUNCH;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // every thread finds the same addresses
+    g_arrive_ptr[dev].store(c, std::memory_order_release);
   }
   *out = p;
+  *arrive = (unsigned int*)c;
   return SOCKET_OK;
 }
 
@@ -601,7 +706,8 @@ extern "C" size_t socket_static_scratch_bytes(void) { return (size_t)SOCKET_STAT
 
 extern "C" int socket_static_scratch_init(void) {
   void* p = nullptr;
-  return static_scratch(&p);
+  unsigned int* c = nullptr;
+  return static_scratch(&p, &c);
 }
 
 extern "C" int socket_sparse_attention_static(const void* q, const void* k, const void* v, int dtype,
@@ -615,18 +721,26 @@ extern "C" int socket_sparse_attention_static(const void* q, const void* k, cons
                                               int Hkv, int D, int kv_rows, int max_len, void* stream) {
   SOCKET_REQUIRE(out, SOCKET_ERR_NULL);
   SOCKET_REQUIRE(max_len > 0 && B > 0 && Hq > 0 && D > 0, SOCKET_ERR_SHAPE);
-  // the partials of this call must fit the fixed array
+  // the partials of this call must fit the fixed array, its rows the counters
   SOCKET_REQUIRE(socket_sparse_attention_workspace_bytes(B, Hq, D, max_len) <= (size_t)SOCKET_STATIC_SCRATCH_BYTES,
                  SOCKET_ERR_WORKSPACE);
+  SOCKET_REQUIRE((int64_t)B * Hq <= kArriveRows, SOCKET_ERR_WORKSPACE);
   void* ws = nullptr;
-  const int st = static_scratch(&ws);
+  unsigned int* arrive = nullptr;
+  const int st = static_scratch(&ws, &arrive);
   if (st != SOCKET_OK) return st;
-  // Nothing in the array has to start at zero: stage 1 writes every split stage 2
-  // reads (the first ceil(len / split size) of a row); older contents are never read.
-  return sparse_attention_on(ws, q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h,
-                             k_stride_s, v_stride_b, v_stride_h, v_stride_s, sparse_list, list_stride_b,
-                             list_stride_h, sparse_len, len_stride_b, len_stride_h, out, out_stride_b,
-                             out_stride_h, B, Hq, Hkv, D, kv_rows, max_len, stream);
+  // Nothing in the partials array has to start at zero: a row's merge reads only the
+  // splits the same launch wrote (the first ceil(len / split size) of the row).  One
+  // launch: the workgroup that finishes a row's last split merges the row.
+  const int bs = socket_sparse_attention_block_seq(B, Hq, max_len);
+  const int nsplit = (max_len + bs - 1) / bs;
+  float* mid_o = (float*)ws;
+  float* mid_lse = mid_o + (size_t)B * Hq * nsplit * D;
+  const Stage1Finish fin{arrive, out, dtype, out_stride_b, out_stride_h};
+  return attend_stage1(q, k, v, dtype, q_stride_b, q_stride_h, k_stride_b, k_stride_h, k_stride_s, v_stride_b,
+                       v_stride_h, v_stride_s, sparse_list, list_stride_b, list_stride_h, sparse_len,
+                       len_stride_b, len_stride_h, mid_o, mid_lse, B, Hq, Hkv, D, kv_rows, max_len, nsplit, bs,
+                       &fin, stream);
 }
 
 extern "C" size_t socket_dense_decode_workspace_bytes(int B, int Hq, int D, int T) {

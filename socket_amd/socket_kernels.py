@@ -150,8 +150,9 @@ def sparse_attention_fwd_static(query: torch.Tensor, key: torch.Tensor, value: t
                                 sparse_list: torch.Tensor, sparse_len: torch.Tensor,
                                 out: torch.Tensor) -> torch.Tensor:
     """`sparse_attention_fwd` into a caller-provided `out` [B,H,D] without allocating
-    anything: the per-split partials live in a fixed array inside the library
-    (one per GPU, shared by every call on it: calls that overlap on one GPU race).
+    anything, as one launch: the per-split partials live in a fixed array inside the
+    library and the workgroup that finishes a row's last split merges the row
+    (one array per GPU, shared by every call on it: calls that overlap on one GPU race).
     `sparse_list` / `sparse_len` must already be int32.  Raises RuntimeError when
     the call needs more than the array holds."""
     assert query.is_cuda and key.is_cuda and value.is_cuda and sparse_list.is_cuda and sparse_len.is_cuda
@@ -171,6 +172,13 @@ def sparse_attention_fwd_static(query: torch.Tensor, key: torch.Tensor, value: t
         ptr(out), out.stride(0), out.stride(1),
         B, H, key.shape[1], D, key.shape[2], width, stream_ptr(query.device)))
     return out
+
+
+def fits_static_scratch(B: int, H: int, D: int, width: int) -> bool:
+    """True if `sparse_attention_fwd_static` takes a call of this shape."""
+    L = lib()
+    return (width > 0 and B * H <= 65536 and
+            L.socket_sparse_attention_workspace_bytes(B, H, D, width) <= L.socket_static_scratch_bytes())
 
 
 @torch.no_grad()

@@ -1,8 +1,9 @@
 """socket_sparse_attention_static (the entry point that allocates nothing: its
-per-split partials live in a fixed array inside the library) against
-socket_sparse_attention on the same inputs, through the C ABI.  Both run the
-same kernels with the same split, so the outputs must be identical bit for bit.
-Two calls in a row share the array; the second is smaller than the first."""
+per-split partials and row counters live in fixed arrays inside the library, and
+the last split of a row merges the row in the same launch) against
+socket_sparse_attention on the same inputs, through the C ABI.  Both use the same
+split and the same merge arithmetic, so the outputs must be identical bit for bit.
+Calls in a row share the arrays; later ones are smaller than the first."""
 import pytest
 import torch
 
@@ -21,6 +22,8 @@ def _case(dev, seed, B, Hq, Hkv, T, width, dtype):
     ln = torch.randint(1, width + 1, (B, Hq), generator=g, dtype=torch.int32)
     ln[0, 0] = width
     sl[0, 1, :3] = -1            # skipped entries
+    ln[-1, -1] = 0               # nothing listed: the reference's 0/0
+    ln[-1, 0] = 1
     return q, k, v, sl.to(dev), ln.to(dev)
 
 
@@ -40,8 +43,15 @@ def test_static_scratch_variant_equals_the_workspace_variant(dev):
         got = socket_kernels.sparse_attention_fwd_static(q, k, v, sl, ln, out)
         assert torch.cuda.memory_stats()["allocation.all.allocated"] == allocs   # no allocation through torch either
         torch.cuda.synchronize()
+        assert torch.isnan(want[-1, -1]).all() and torch.isnan(got[-1, -1]).all()
+        want[-1, -1] = 0
+        got[-1, -1] = 0
         assert torch.isfinite(want.float()).all()
         assert torch.equal(got, want), f"case {seed}: max diff {(got.float() - want.float()).abs().max()}"
+    # the row counters are back at zero: the same call again gives the same result
+    again = socket_kernels.sparse_attention_fwd_static(q, k, v, sl, ln, torch.empty_like(got))
+    again[-1, -1] = 0
+    assert torch.equal(again, got)
 
 
 def test_static_scratch_variant_refuses_what_does_not_fit(dev):
