@@ -78,12 +78,39 @@ def algorithmic_bytes(w, lens=None, budgets=None):
     }
 
 
+SETTLE_MS = 60.0
+
+
+def settle(run, ms=None):
+    """Keeps the GPU busy with `run` for about `ms` milliseconds, untimed, and returns
+    how many times it ran.  A burst that starts on an idle GPU runs in a transient
+    power state: the scorer of the 128k workload takes 95-114 us per launch in the
+    first milliseconds after an idle gap and 88-89 us once the card has been busy
+    for some tens of milliseconds, which is the state of a decode loop (32 layers
+    back to back, token after token).  Timed regions therefore follow a settle
+    phase; the figure without one is reported beside the step's."""
+    ms = SETTLE_MS if ms is None else ms
+    if ms <= 0:
+        return 0
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    run()
+    e1.record()
+    e1.synchronize()
+    n = int(min(20000, max(1, ms / max(e0.elapsed_time(e1), 1e-3))))
+    for _ in range(n):
+        run()
+    return n + 1
+
+
 def time_graph(fn, iters, warmup=2, per_graph=10):
     """Average device time in microseconds of one call of `fn`: `per_graph` calls are
     recorded into one HIP graph and the graph is replayed between two HIP events, so
     the figure is kernel time plus the in-graph launch gap, without the Python and
     ctypes cost of an eager call (which is several microseconds, more than some of
-    these kernels take).  Falls back to eager launches if capture fails."""
+    these kernels take).  The timed replays (at least 100 calls) follow a settle
+    phase.  Falls back to eager launches if capture fails."""
     try:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -98,7 +125,8 @@ def time_graph(fn, iters, warmup=2, per_graph=10):
                 fn()
         g.replay()
         torch.cuda.synchronize()
-        reps = max(1, (iters + per_graph - 1) // per_graph)
+        reps = max(1, (max(iters, 100) + per_graph - 1) // per_graph)
+        settle(g.replay)
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -385,19 +413,28 @@ def timed_graph_steps(step_fn, steps, warmup, eager=False):
             print(f"bench: HIP graph capture unavailable ({e}); timing eager launches", file=sys.stderr)
             graph, ok = None, None
     run = graph.replay if graph is not None else step_fn
-    for _ in range(warmup):
-        run()
+
+    def timed():
+        for _ in range(warmup):
+            run()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps, (time.perf_counter() - t0) * 1e3
+
+    # once from an idle GPU (reported beside the result), then after the settle phase
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    return e0.elapsed_time(e1) / steps, wall_ms, "hip graph replay" if graph is not None else "eager", ok
+    time.sleep(0.05)
+    after_idle_ms, _ = timed()
+    settled = settle(run)
+    ms_per_step, wall_ms = timed()
+    return (ms_per_step, wall_ms, "hip graph replay" if graph is not None else "eager", ok,
+            {"settle_steps_untimed": settled, "settle_ms": SETTLE_MS, "us_per_step_from_idle": round(after_idle_ms * 1e3, 2)})
 
 
 def measure_workload(w, dev, steps, warmup, args, full):
@@ -426,7 +463,7 @@ def measure_workload(w, dev, steps, warmup, args, full):
     ab = st.abytes
     kernels = {k: {"us": round(v, 2), "algorithmic_MB": round(ab[k] / 1e6, 2), "gbs": round(ab[k] / v / 1e3, 1),
                    "hbm_frac": round(ab[k] / v / 1e3 / HBM_PEAK_GBS, 4)} for k, v in per.items()}
-    ms_per_step, wall_ms, launch, replay_ok = timed_graph_steps(st.step, steps, warmup, eager=args.eager)
+    ms_per_step, wall_ms, launch, replay_ok, power_state = timed_graph_steps(st.step, steps, warmup, eager=args.eager)
     sparse_us = ms_per_step * 1e3
     sparse_bytes = ab["score"] + ab["select"] + ab["attend"]
     kernel_sum_us = per["score"] + per["select"] + per["attend"]
@@ -440,7 +477,9 @@ def measure_workload(w, dev, steps, warmup, args, full):
         "step_us": round(sparse_us, 2),
         "ms_per_step": ms_per_step,
         "launch": launch,
-        "kernel_timing": "HIP-graph replay of 10 launches between two HIP events (kernel time + in-graph launch gap)",
+        "power_state": power_state,
+        "kernel_timing": "HIP-graph replay of 10 launches between two HIP events (kernel time + in-graph launch gap), "
+                         f">= 100 launches timed after {SETTLE_MS:.0f} ms of untimed replays",
         "kernels": kernels,
         "sparse_total": {"algorithmic_MB": round(sparse_bytes / 1e6, 2), "kernel_sum_us": round(kernel_sum_us, 2),
                          "hbm_frac_of_kernel_sum": round(sparse_bytes / kernel_sum_us / 1e3 / HBM_PEAK_GBS, 4),
@@ -501,12 +540,15 @@ def main():
                              "block_sparse", "step", "decode", "read_probe"])
     ap.add_argument("--reference-table-layout", action="store_true",
                     help="feed the scorer q_probs as [B,Hq,L,R] instead of the grouped layout the soft-hash kernel writes")
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
+                    help="untimed GPU-busy time before each timed region (0: time from whatever state the GPU is in)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the other workloads' sub-records and the end-to-end decode runs")
     ap.add_argument("--eager", action="store_true", help="time plain launches instead of a recorded HIP graph")
     args = ap.parse_args()
+    globals()["SETTLE_MS"] = args.settle_ms
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every (sequence, kv head) "
               "pair is independent; see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
@@ -560,6 +602,7 @@ def main():
         fn = {"score": st.k_score_ref, "score_f32": st.k_score_f32, "score_grouped": st.k_score_grouped,
               "select": lambda: st.k_select(scores, rng), "attend": lambda: st.k_attend(sl, ln), "hash": st.k_hash,
               "dense": st.k_dense, "step": st.step}[args.only]
+        settle(fn)
         us = time_launches(fn, iters, warmup=args.warmup)
         key = args.only.replace("_grouped", "")
         nbytes = st.abytes[key] if key in st.abytes else st.abytes["score"] + st.abytes["select"] + st.abytes["attend"]
@@ -595,6 +638,7 @@ def main():
                      "traffic_source": MEASURED_TRAFFIC_SOURCE if MEASURED_TRAFFIC_BYTES.get(w.name) else None},
         "kernels": rec["kernels"],
         "kernel_timing": rec["kernel_timing"],
+        "power_state": rec["power_state"],
         "sparse_total": rec["sparse_total"],
         "hash_prefill": rec["hash_prefill"],
         "copy_ceiling_gbs": round(ceiling, 1),

@@ -155,7 +155,21 @@ int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
  * socket_score_prefers_grouped: which layout a producer should write for this
  * shape (T = the context length the scorer will be called with): 1 = grouped,
  * 0 = [B,Hq,L,R] (the shapes the scorer serves one head per workgroup, see
- * socket_score_packed), -1 = invalid shape.  Either layout is always accepted. */
+ * socket_score_packed), -1 = invalid shape.  Either layout is always accepted.
+ * socket_score_plan_query: the launch shape the scorer would use for a table in the
+ * given layout (tokens per workgroup; whether table slices are copied global ->
+ * LDS directly; whether a workgroup serves one head with its table resident) and
+ * the cost model's estimate of the launch in microseconds.  The model prices a
+ * shape from table bytes per workgroup, LDS slices, lookups per tile, entry width
+ * and workgroups against compute units; it ranks shapes, it is not a timing promise. */
+int socket_score_plan_query(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R, int grouped,
+                            int* tile, int* direct_copy, int* one_head, float* cost_us);
+/* The same estimate for one given shape (tile 8192, 4096, 2048 or 1024), with the
+ * LDS slices per workgroup and the waves per workgroup it was priced on;
+ * SOCKET_ERR_UNSUPPORTED if that shape cannot be launched for this table.
+ * socket_score_plan_query returns the cheapest of these. */
+int socket_score_shape_cost(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R, int grouped,
+                            int tile, int direct_copy, int one_head, int* slices, int* waves, float* cost_us);
 int socket_group_shape(int Hq, int Hkv, int* parts, int* width);
 int socket_score_prefers_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);
 int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);

@@ -46,6 +46,10 @@ SIGNATURES = {
     "socket_score_packed": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
     "socket_soft_hash_collision": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "socket_soft_hash_score_f16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "socket_score_plan_query": (_I, [_I, _I, _I, _I, _I, _I, _I, _I, _I, POINTER(c_int), POINTER(c_int),
+                                     POINTER(c_int), POINTER(c_float)]),
+    "socket_score_shape_cost": (_I, [_I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, POINTER(c_int), POINTER(c_int),
+                                     POINTER(c_float)]),
     "socket_group_shape": (_I, [_I, _I, POINTER(c_int), POINTER(c_int)]),
     "socket_score_prefers_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "socket_score_range_parts_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),

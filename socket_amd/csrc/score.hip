@@ -21,6 +21,10 @@
 //  * collision_i16_kernel: the reference's own operand layout (int16 codes per
 //    query head), for drop-in callers.
 #include <type_traits>
+#ifdef SOCKET_SCORE_PLAN_OVERRIDE
+#include <cstdio>
+#include <cstdlib>
+#endif
 
 #include "socket_common.h"
 
@@ -769,6 +773,39 @@ struct ScoreArgs {
   int grouped;  // table layout: 0 = [B,Hq,L,R], 1 = [B*Hkv*parts, L, R, group width]
 };
 
+// How a workgroup's table passes through LDS: buffers, packed words per slice.
+// Shared by the launch and by the cost model, so that both see the same slices.
+struct SliceLayout {
+  int nbuf, chunk_words;
+  bool ok;
+};
+
+SliceLayout slice_layout(bool dma, size_t bytes_per_word, size_t slots_per_word, int NW, size_t lds_budget) {
+  SliceLayout s{2, 1, true};
+  if (dma) {
+    if (bytes_per_word * NW <= lds_budget) {
+      // the whole table at once: one copy, no slices
+      s.nbuf = 1;
+      s.chunk_words = NW;
+    } else {
+      // two buffers, as many words per slice as LDS holds (no register staging to fit)
+      if (2 * bytes_per_word > lds_budget) s.ok = false;
+      while (s.ok && s.chunk_words < NW && 2 * bytes_per_word * (s.chunk_words + 1) <= lds_budget) ++s.chunk_words;
+    }
+  } else if (2 * bytes_per_word <= lds_budget && slots_per_word <= 1024) {
+    // Double-buffered when one word's tables fit twice in LDS and in the staging
+    // registers (1024 vector slots per workgroup); as many words per slice as that
+    // allows.  Otherwise a single buffer filled in place.
+    while (s.chunk_words < NW && 2 * bytes_per_word * (s.chunk_words + 1) <= lds_budget / 2 &&
+           slots_per_word * (s.chunk_words + 1) <= 1024)
+      ++s.chunk_words;
+  } else {
+    s.nbuf = 1;
+    if (bytes_per_word > lds_budget) s.ok = false;
+  }
+  return s;
+}
+
 template <int GP, class TT, int KT4, int THREADS, int PT, int MODE>
 int launch_score_packed(const ScoreArgs& a) {
   typedef typename TT::elem TE;
@@ -781,31 +818,12 @@ int launch_score_packed(const ScoreArgs& a) {
   const size_t slots_per_word = (size_t)cpw * a.R / EPV;
   constexpr bool DMA = MODE == 2;
   const size_t lds_budget = (size_t)lim.max_lds_per_block - kScoreScratchBytes;
-  int nbuf = 2, chunk_words = 1;
-  if (DMA) {
-    // The slice copy needs the table block of a workgroup contiguous: the grouped
-    // layout, or any layout when a workgroup serves one head.
-    if (!(a.grouped || GP == 1) || (a.grouped && GP == 1 && G != 1)) return SOCKET_ERR_UNSUPPORTED;
-    if (bytes_per_word * NW <= lds_budget) {
-      // the whole table at once: one copy, no slices
-      nbuf = 1;
-      chunk_words = NW;
-    } else {
-      // two buffers, as many words per slice as LDS holds (no register staging to fit)
-      if (2 * bytes_per_word > lds_budget) return SOCKET_ERR_UNSUPPORTED;
-      while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= lds_budget) ++chunk_words;
-    }
-  } else if (2 * bytes_per_word <= lds_budget && slots_per_word <= 1024) {
-    // Double-buffered when one word's tables fit twice in LDS and in the staging
-    // registers (1024 vector slots per workgroup); as many words per slice as that
-    // allows.  Otherwise a single buffer filled in place.
-    while (chunk_words < NW && 2 * bytes_per_word * (chunk_words + 1) <= lds_budget / 2 &&
-           slots_per_word * (chunk_words + 1) <= 1024)
-      ++chunk_words;
-  } else {
-    nbuf = 1;
-    if (bytes_per_word > lds_budget) return SOCKET_ERR_UNSUPPORTED;
-  }
+  // The slice copy needs the table block of a workgroup contiguous: the grouped
+  // layout, or any layout when a workgroup serves one head.
+  if (DMA && (!(a.grouped || GP == 1) || (a.grouped && GP == 1 && G != 1))) return SOCKET_ERR_UNSUPPORTED;
+  const SliceLayout sl = slice_layout(DMA, bytes_per_word, slots_per_word, NW, lds_budget);
+  if (!sl.ok) return SOCKET_ERR_UNSUPPORTED;
+  const int nbuf = sl.nbuf, chunk_words = sl.chunk_words;
   const size_t table_bytes = bytes_per_word * chunk_words * nbuf;
   const size_t lds_bytes = table_bytes + kScoreScratchBytes;
 
@@ -856,75 +874,90 @@ struct ScorePlan {
   float cost;  // rough time estimate, for comparing plans only
 };
 
-// Launch shapes and what they cost (microseconds measured at L60 x P10 bf16
-// tables on this GPU; only their ratios are used, to choose between shapes):
-//  * grouped / direct: G heads per gather, table slices copied global -> LDS.
-//    8192-token tiles: ~53 per round of workgroups on a full chip, ~40 when the
-//    workgroups cover only part of it (a workgroup's time hardly depends on how
-//    many others there are); 4096 / 2048 / 1024-token tiles (16-bit entries):
-//    ~29 / 20 / 20 per round -- every workgroup pulls the whole table through LDS,
-//    so small tiles pay off only while they add CUs, not rounds;
-//  * slices staged through registers: 8192-token tiles ~57 per round (~50 on a part
-//    of the chip, ~73 with 32-bit entries); smaller tiles
-//    (4096 / 2048 / 1024, chosen so that every CU has a workgroup) ~45 per round
-//    from the reference layout and ~62 from the grouped one -- every workgroup
-//    still pulls the whole table through LDS, one exposed latency per slice;
-//  * solo: ONE query head per workgroup, its whole table (L*R elements, if that
-//    fits LDS) copied in once, no barriers; the G workgroups of a kv head share its
-//    code stream through the XCD's L2.  ~5 + 31 * (tile / 8192) per round, but G
-//    times the workgroups: it wins while those still fit one round (short
-//    contexts, few kv heads) and loses to the grouped shape beyond.
-// Solo needs the [B,Hq,L,R] layout, the direct copy the grouped one: score_plan
-// prices the layout it is given, socket_score_prefers_grouped compares the two.
-ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_elem_bytes, int L, int P, int R) {
+// Cost model of a launch shape.  A workgroup's time on its CU is priced from what it
+// does, and a round of workgroups from that and from the HBM stream they share:
+//
+//   t_cu   = a + s * slices + r * (table KB per wave) + c[entry bytes] * lookups
+//   t_mem  = workgroups in the round * tokens per tile * HBM bytes per token / kStreamGBs
+//   round  = (t_cu^3 + t_mem^3)^(1/3)        (the two overlap, imperfectly)
+//   launch = rounds * round
+//
+//   slices         LDS slices a tile walks (slice_layout: the launch's own arithmetic)
+//   table KB/wave  the table block every tile pulls through LDS, shared out over its waves
+//   lookups        tokens per tile * tables: the LDS gathers of a workgroup
+//   entry bytes    heads per lookup * element size: what one gather returns
+//
+// with one set of coefficients per kernel variant (they are different kernels:
+// direct global -> LDS copies, slices staged through registers from either table
+// layout, one head per workgroup with its table resident).  The coefficients are
+// a non-negative least-squares fit to 1008 timed launches on one MI355X: every
+// variant and tile size forced in turn on 8 table geometries (L60xP10 with 1, 2
+// and 4 heads per kv head in bf16 and with 4 in fp32; L48xP10 with 4 and 7; L32xP8
+// in bf16 and fp32) times 7 batch / context shapes from B1 x 32768 to B16 x 65536.
+// Choosing by the model costs 1% on average and at most 31% over the best
+// measured shape of a layout (the hand-written table it replaces: 14% / 125%).
+// Its error between variants is larger than within one, so the layout preference
+// asks for a margin (kLayoutMargin).
+struct VariantCost {
+  float a, s, r;      // us; us per slice; us per table KB per wave
+  float c[4];         // picoseconds per lookup for entries of 2, 4, 8, 16 bytes
+};
+constexpr VariantCost kCostDirect = {3.331f, 0.535f, 0.068f, {64.2f, 63.2f, 64.6f, 112.1f}};
+constexpr VariantCost kCostStagedRef = {0.536f, 0.0f, 0.102f, {63.4f, 68.8f, 91.1f, 145.1f}};
+constexpr VariantCost kCostStagedGrouped = {0.670f, 0.668f, 0.284f, {49.9f, 70.2f, 95.7f, 143.7f}};
+constexpr VariantCost kCostSolo = {0.0f, 0.0f, 0.222f, {63.6f, 53.3f, 53.3f, 53.3f}};
+constexpr float kStreamGBs = 6000.f;   // what the code stream and the score stores get when every CU pulls
+constexpr float kLayoutMargin = 1.3f;  // the grouped layout is preferred unless the other is this much cheaper
+
+int threads_of(int tile, bool dma) {
+  if (dma) return tile >= 4096 ? 1024 : tile == 2048 ? 512 : 256;
+  return tile == 8192 ? 1024 : tile >= 2048 ? 512 : 256;
+}
+
+// Estimated microseconds of a launch of the given shape; < 0 if the shape cannot be launched.
+float shape_cost(int B, int Hkv, int G, int T, int grouped, size_t eb, int L, int P, int R, int tile, bool dma,
+                 bool solo, int* slices_out = nullptr, int* waves_out = nullptr) {
   const SocketDeviceLimits& lim = socket_device_limits();
-  const int width = G == 1 ? 1 : G == 2 ? 2 : 4;
-  const int64_t pairs = (int64_t)B * Hkv * ((G + width - 1) / width);  // groups of 5..8 heads go as two workgroups
-  auto tiles = [&](int tw) { return (int64_t)((T + tw - 1) / tw); };
-  auto rounds = [&](int64_t wgs) { return (float)((wgs + lim.cu_count - 1) / lim.cu_count); };
-  const int64_t big = pairs * tiles(8192);  // workgroups of the 8192-token shapes
-  const size_t bytes_per_word = P > 0 ? (size_t)(32 / P) * R * width * table_elem_bytes : 0;
-  const bool slices_fit_twice = P > 0 && 2 * bytes_per_word + kScoreScratchBytes <= (size_t)lim.max_lds_per_block;
-  // staged tiles: the largest that gives every CU a workgroup
-  ScorePlan staged{1024, false, false, (grouped ? 62.f : 45.f) * rounds(pairs * tiles(1024))};
-  for (int tw = 8192; tw > 1024; tw >>= 1)
-    if (pairs * tiles(tw) >= lim.cu_count) {
-      staged = {tw, false, false, (tw == 8192 ? 57.f : grouped ? 62.f : 45.f) * rounds(pairs * tiles(tw))};
-      break;
+  if (P < 1 || P > 16 || L < 1) return -1.f;
+  const int cpw = 32 / P, NW = (L + cpw - 1) / cpw;
+  const int width = (G == 1 || solo) ? 1 : G == 2 ? 2 : 4;
+  const int hsplit = solo ? G : (G + width - 1) / width;
+  if (solo && (grouped || G == 1 || !dma)) return -1.f;
+  if (dma && !solo && !(grouped || G == 1)) return -1.f;
+  const size_t bytes_per_word = (size_t)cpw * R * width * eb;
+  const size_t slots_per_word = (size_t)cpw * R / (16 / eb);
+  const size_t budget = (size_t)lim.max_lds_per_block - kScoreScratchBytes;
+  const SliceLayout sl = slice_layout(dma, bytes_per_word, slots_per_word, NW, budget);
+  if (!sl.ok) return -1.f;
+  if (solo && sl.nbuf != 1) return -1.f;   // one head per workgroup only with its whole table resident
+  const int waves = threads_of(tile, dma) / SOCKET_WAVE;
+  const int slices = (NW + sl.chunk_words - 1) / sl.chunk_words;
+  if (slices_out) *slices_out = slices;
+  if (waves_out) *waves_out = waves;
+  const int64_t wgs = (int64_t)B * Hkv * hsplit * ((T + tile - 1) / tile);
+  const int64_t rounds = (wgs + lim.cu_count - 1) / lim.cu_count;
+  const int64_t active = wgs < lim.cu_count ? wgs : lim.cu_count;
+  const VariantCost& v = solo ? kCostSolo : dma ? kCostDirect : grouped ? kCostStagedGrouped : kCostStagedRef;
+  const size_t entry = (size_t)width * eb;
+  const float c = v.c[entry <= 2 ? 0 : entry <= 4 ? 1 : entry <= 8 ? 2 : 3];
+  const float table_kb = (float)((size_t)L * R * width * eb) / 1e3f;
+  const float t_cu = v.a + v.s * slices + v.r * table_kb / waves + c * 1e-6f * (float)tile * L;
+  // HBM bytes per token of a workgroup: codes + norm (shared through the L2 by the G
+  // workgroups of a kv head when each serves one head) + the scores it stores
+  const float bpt = (NW * 4.f + 2.f) / (solo ? G : 1) + 4.f * width;
+  const float t_mem = (float)active * tile * bpt / (kStreamGBs * 1e3f);
+  return (float)rounds * cbrtf(t_cu * t_cu * t_cu + t_mem * t_mem * t_mem);
+}
+
+// The cheapest launchable shape for a table in the given layout.
+ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_elem_bytes, int L, int P, int R) {
+  ScorePlan best{1024, false, false, -1.f};
+  for (int tile = 8192; tile >= 1024; tile >>= 1)
+    for (int variant = 0; variant < 3; ++variant) {
+      const bool dma = variant != 1, solo = variant == 2;
+      const float cost = shape_cost(B, Hkv, G, T, grouped, table_elem_bytes, L, P, R, tile, dma, solo);
+      if (cost >= 0.f && (best.cost < 0.f || cost < best.cost)) best = {tile, dma, solo, cost};
     }
-  if (grouped) {
-    if (slices_fit_twice) {
-      ScorePlan best = {1024 * 4 * kDmaKT4, true, false, big >= lim.cu_count ? 53.f * rounds(big) : 40.f};
-      if (table_elem_bytes == 2) {
-        // smaller tiles (16-bit entries: the variants whose code prefetch runs ahead):
-        // a round of them on a full chip / on a part of it
-        const int tw[3] = {4096, 2048, 1024};
-        const float full[3] = {29.f, 20.f, 20.f}, part[3] = {25.f, 19.f, 20.f};
-        for (int i = 0; i < 3; ++i) {
-          const int64_t wgs = pairs * tiles(tw[i]);
-          const float cost = wgs >= lim.cu_count ? full[i] * rounds(wgs) : part[i];
-          if (cost < best.cost) best = {tw[i], true, false, cost};
-        }
-      }
-      return best;
-    }
-    return staged;
-  }
-  ScorePlan best = staged;
-  // 8192-token tiles on a part of the chip (16-bit entries ~50, 32-bit ~73)
-  const float big_part = table_elem_bytes == 2 ? 50.f : 73.f;
-  if (slices_fit_twice && big < lim.cu_count && big_part < best.cost) best = {8192, false, false, big_part};
-  if (G > 1 && (size_t)L * R * table_elem_bytes + kScoreScratchBytes <= (size_t)lim.max_lds_per_block) {
-    const int64_t heads = (int64_t)B * Hkv * G;
-    int tw = 1024;
-    for (int t = 8192; t > 1024; t >>= 1)
-      if (heads * tiles(t) >= lim.cu_count) {
-        tw = t;
-        break;
-      }
-    const float cost = (5.f + 31.f * (float)tw / 8192.f) * rounds(heads * tiles(tw));
-    if (cost < best.cost) best = {tw, true, true, cost};
-  }
   return best;
 }
 
@@ -945,7 +978,13 @@ int dispatch_tile(const ScoreArgs& a, const ScorePlan& plan) {
 template <class TT>
 int dispatch_g(const ScoreArgs& a) {
   const int G = a.Hq / a.Hkv;
-  const ScorePlan plan = score_plan(a.B, a.Hkv, G, a.T, a.grouped, sizeof(typename TT::elem), a.L, a.P, a.R);
+  ScorePlan plan = score_plan(a.B, a.Hkv, G, a.T, a.grouped, sizeof(typename TT::elem), a.L, a.P, a.R);
+#ifdef SOCKET_SCORE_PLAN_OVERRIDE
+  if (const char* f = getenv("SOCKET_SCORE_FORCE")) {  // "tile,dma,solo" (measurement builds only)
+    int t = 0, d = 0, so = 0;
+    if (sscanf(f, "%d,%d,%d", &t, &d, &so) == 3) plan = {t, d != 0, so != 0, 0.f};
+  }
+#endif
   if (G == 1 || plan.solo) return dispatch_tile<1, TT>(a, plan);
   if (G == 2) return dispatch_tile<2, TT>(a, plan);
   return dispatch_tile<4, TT>(a, plan);
@@ -1035,7 +1074,34 @@ extern "C" int socket_score_prefers_grouped(int B, int Hq, int Hkv, int T, int q
   const size_t eb = q_dtype == SOCKET_F32 ? 4 : 2;
   const ScorePlan ref = score_plan(B, Hkv, Hq / Hkv, T, 0, eb, L, P, R);
   const ScorePlan grp = score_plan(B, Hkv, Hq / Hkv, T, 1, eb, L, P, R);
-  return grp.cost <= ref.cost ? 1 : 0;
+  if (grp.cost < 0.f) return 0;
+  if (ref.cost < 0.f) return 1;
+  return grp.cost <= ref.cost * kLayoutMargin ? 1 : 0;
+}
+
+extern "C" int socket_score_plan_query(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R, int grouped,
+                                       int* tile, int* direct_copy, int* one_head, float* cost_us) {
+  if (range_parts_of(B, Hq, Hkv, T, q_dtype, L, P, R, grouped) == 0) return SOCKET_ERR_SHAPE;
+  if (Hq / Hkv > 8) return SOCKET_ERR_UNSUPPORTED;
+  const ScorePlan plan = score_plan(B, Hkv, Hq / Hkv, T, grouped, q_dtype == SOCKET_F32 ? 4 : 2, L, P, R);
+  if (plan.cost < 0.f) return SOCKET_ERR_UNSUPPORTED;
+  if (tile) *tile = plan.tile;
+  if (direct_copy) *direct_copy = plan.dma ? 1 : 0;
+  if (one_head) *one_head = plan.solo ? 1 : 0;
+  if (cost_us) *cost_us = plan.cost;
+  return SOCKET_OK;
+}
+
+extern "C" int socket_score_shape_cost(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R, int grouped,
+                                       int tile, int direct_copy, int one_head, int* slices, int* waves,
+                                       float* cost_us) {
+  if (range_parts_of(B, Hq, Hkv, T, q_dtype, L, P, R, grouped) == 0) return SOCKET_ERR_SHAPE;
+  if (Hq / Hkv > 8 || (tile != 8192 && tile != 4096 && tile != 2048 && tile != 1024)) return SOCKET_ERR_UNSUPPORTED;
+  const float cost = shape_cost(B, Hkv, Hq / Hkv, T, grouped, q_dtype == SOCKET_F32 ? 4 : 2, L, P, R, tile,
+                                direct_copy != 0, one_head != 0, slices, waves);
+  if (cost < 0.f) return SOCKET_ERR_UNSUPPORTED;
+  if (cost_us) *cost_us = cost;
+  return SOCKET_OK;
 }
 
 extern "C" int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {

@@ -116,9 +116,104 @@ def test_sizes_helpers(lib):
     assert lib.socket_score_prefers_grouped(1, 32, 8, 32768, 1, 60, 10, 1024) == 1
     assert lib.socket_score_range_parts_grouped(1, 32, 8, 131072, 1, 60, 10, 1024) == 32   # 4096-token tiles fill the chip
     assert lib.socket_score_range_parts_grouped(1, 32, 8, 65536, 1, 60, 10, 1024) == 32    # 2048-token tiles
-    assert lib.socket_score_range_parts_grouped(1, 32, 8, 65536, 0, 60, 10, 1024) == 8     # fp32 entries stay at 8192
+    assert lib.socket_score_range_parts_grouped(1, 32, 8, 65536, 0, 60, 10, 1024) == 32    # fp32 entries too
     assert lib.socket_score_prefers_grouped(1, 32, 8, 65536, 0, 60, 10, 1024) == 1     # fp32: a head's table exceeds LDS
     assert lib.socket_score_prefers_grouped(1, 5, 2, 100, 1, 60, 10, 1024) == -1
+
+
+def _plan(lib, B, Hq, Hkv, T, dt, L, P, grouped):
+    from ctypes import byref, c_float, c_int
+    tile, direct, one_head, cost = c_int(), c_int(), c_int(), c_float()
+    rc = lib.socket_score_plan_query(B, Hq, Hkv, T, dt, L, P, 1 << P, grouped, byref(tile), byref(direct),
+                                     byref(one_head), byref(cost))
+    return rc, tile.value, direct.value, one_head.value, cost.value
+
+
+def _shape_cost(lib, B, Hq, Hkv, T, dt, L, P, grouped, tile, direct, one_head):
+    from ctypes import byref, c_float, c_int
+    slices, waves, cost = c_int(), c_int(), c_float()
+    rc = lib.socket_score_shape_cost(B, Hq, Hkv, T, dt, L, P, 1 << P, grouped, tile, direct, one_head, byref(slices),
+                                     byref(waves), byref(cost))
+    return rc, slices.value, waves.value, cost.value
+
+
+SCORE_GEOMETRIES = [(32, 8, 60, 10), (28, 4, 48, 10), (32, 8, 32, 8), (16, 8, 60, 10), (16, 16, 60, 10), (32, 8, 16, 12)]
+
+
+@pytest.mark.parametrize("Hq,Hkv,L,P", SCORE_GEOMETRIES)
+@pytest.mark.parametrize("dt", [0, 1])
+def test_score_plan_is_the_cheapest_launchable_shape(Hq, Hkv, L, P, dt):
+    from socket_amd._lib import lib as load
+    lib = load()
+    for grouped in (0, 1):
+        for B, T in ((1, 8192), (1, 65536), (4, 131072), (16, 57344)):
+            rc, tile, direct, one_head, cost = _plan(lib, B, Hq, Hkv, T, dt, L, P, grouped)
+            assert rc == 0 and tile in (1024, 2048, 4096, 8192) and cost > 0
+            costs = {}
+            for t in (8192, 4096, 2048, 1024):
+                for d, o in ((1, 0), (0, 0), (1, 1)):
+                    rc, slices, waves, c = _shape_cost(lib, B, Hq, Hkv, T, dt, L, P, grouped, t, d, o)
+                    if rc == 0:
+                        assert slices >= 1 and waves in (4, 8, 16) and c > 0
+                        costs[(t, d, o)] = c
+            assert (tile, direct, one_head) in costs
+            assert cost == min(costs.values()) == costs[(tile, direct, one_head)]
+            # one head per workgroup only on the [B,Hq,L,R] layout of a grouped-query model
+            assert not (one_head and (grouped or Hq == Hkv))
+            # the row ranges the scorer writes are per tile of the planned shape
+            parts = (lib.socket_score_range_parts_grouped if grouped else lib.socket_score_range_parts)(
+                B, Hq, Hkv, T, dt, L, P, 1 << P)
+            assert parts == -(-T // tile)
+
+
+@pytest.mark.parametrize("Hq,Hkv,L,P", SCORE_GEOMETRIES)
+def test_score_plan_cost_never_falls_with_more_work(Hq, Hkv, L, P):
+    """More tokens, more sequences, more tables or wider entries never make the
+    estimate cheaper: each shape's price is monotone in them, so their minimum is."""
+    from socket_amd._lib import lib as load
+    lib = load()
+    for grouped in (0, 1):
+        for dt in (0, 1):
+            prev = 0.0
+            for T in (1000, 4096, 8192, 20000, 32768, 65536, 100000, 131072, 262144, 1 << 20):
+                cost = _plan(lib, 2, Hq, Hkv, T, dt, L, P, grouped)[4]
+                assert cost >= prev, (grouped, dt, T)
+                prev = cost
+            prev = 0.0
+            for B in (1, 2, 3, 4, 8, 16, 64):
+                cost = _plan(lib, B, Hq, Hkv, 65536, dt, L, P, grouped)[4]
+                assert cost >= prev, (grouped, dt, B)
+                prev = cost
+            prev = 0.0
+            for tables in (L // 4, L // 2, L, 2 * L):
+                cost = _plan(lib, 4, Hq, Hkv, 65536, dt, tables, P, grouped)[4]
+                assert cost >= prev, (grouped, dt, tables)
+                prev = cost
+        # fp32 entries are never priced below bf16 entries of the same table
+        assert _plan(lib, 4, Hq, Hkv, 131072, 0, L, P, grouped)[4] >= _plan(lib, 4, Hq, Hkv, 131072, 1, L, P, grouped)[4]
+
+
+def test_score_plan_on_the_benchmark_shapes():
+    from socket_amd._lib import lib as load
+    lib = load()
+    # B4 x 128k, L60 x P10, bf16 grouped table: two rounds of 8192-token tiles, slices copied straight into LDS
+    rc, tile, direct, one_head, cost = _plan(lib, 4, 32, 8, 131072, 1, 60, 10, 1)
+    assert (rc, tile, direct, one_head) == (0, 8192, 1, 0) and 60 < cost < 140
+    # batch 1 at 32k: a quarter of the tile so that the chip is filled
+    assert _plan(lib, 1, 32, 8, 32768, 1, 60, 10, 1)[1:4] == (2048, 1, 0)
+    # short context on the [B,Hq,L,R] layout: one head per workgroup, table resident
+    assert _plan(lib, 1, 32, 8, 8192, 1, 60, 10, 0)[3] == 1
+    # fp32 entries: a head's table (60 x 1024 x 4 B) no longer fits LDS, so never one head per workgroup
+    assert _plan(lib, 1, 32, 8, 8192, 0, 60, 10, 0)[3] == 0
+    # the layout a producer is told to write is the cheaper one, with a margin in favour of the grouped one
+    for B, Hq, Hkv, T, dt, L, P in ((1, 32, 8, 8192, 1, 60, 10), (4, 32, 8, 131072, 1, 60, 10), (16, 28, 4, 57344, 1, 48, 10),
+                                    (1, 32, 8, 65536, 0, 60, 10), (2, 16, 8, 30000, 1, 32, 8)):
+        grp, ref = _plan(lib, B, Hq, Hkv, T, dt, L, P, 1)[4], _plan(lib, B, Hq, Hkv, T, dt, L, P, 0)[4]
+        assert lib.socket_score_prefers_grouped(B, Hq, Hkv, T, dt, L, P, 1 << P) == int(grp <= 1.3 * ref)
+    # bad shapes are refused, not priced
+    assert _plan(lib, 1, 5, 2, 100, 1, 60, 10, 1)[0] != 0
+    assert _shape_cost(lib, 1, 32, 8, 8192, 1, 60, 10, 1, 3000, 1, 0)[0] != 0       # not a tile the kernels have
+    assert _shape_cost(lib, 1, 32, 8, 8192, 1, 60, 10, 1, 2048, 1, 1)[0] != 0       # one head per workgroup on a grouped table
 
 
 def test_python_api_keeps_reference_signatures():
