@@ -335,7 +335,10 @@ int socket_sparse_attention_static(const void* q, const void* k, const void* v, 
 /* Dense split-K flash-decode over rows [0, len(b)) of the cache (the
  * comparator the sparse path is timed against; the reference's dense decode is
  * Attention.forward, GPT-FAST/model.py:562-589).  K/V rows are read once per kv
- * head and shared by its G query heads. */
+ * head and shared by its G = Hq / Hkv query heads.  bf16 / fp16 caches with D = 128
+ * run on the matrix cores (G <= 16; probabilities are rounded to the cache's type
+ * before the value product, as flash attention kernels do); other head dims and
+ * fp32 caches on the vector ALU (G <= 8).  SOCKET_ERR_UNSUPPORTED beyond that. */
 size_t socket_dense_decode_workspace_bytes(int B, int Hq, int D, int T);
 int socket_dense_decode(const void* q, const void* k, const void* v, int dtype,
                         int64_t q_stride_b, int64_t q_stride_h,

@@ -30,6 +30,7 @@ FLAGS = [
 # parks them in the accumulator file and moves them back and forth).
 FILE_FLAGS = {
     "block_sparse.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "attend.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],     # the MFMA dense flash-decode, for the same reason
 }
 
 

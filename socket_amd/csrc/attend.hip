@@ -52,6 +52,38 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* acc, floa
   m = nm;
 }
 
+// The split's output from the waves' states in LDS, records [wave][head] of D
+// accumulators (not yet divided by the sum), the running maximum and the sum:
+// acc / sum and max + log(sum) per head, as kernels/socket_triton_kernels.py:82-95.
+template <int D, int GH, bool COHERENT>
+__device__ __forceinline__ void combine_waves(const float* lds, int G, float* mid_o_base, float* mid_lse_base,
+                                              int64_t head_stride_o, int64_t head_stride_lse) {
+  constexpr int REC = D + 2;
+  for (int o = threadIdx.x; o < GH * D; o += kAttThreads) {
+    const int g = o / D, d = o % D;
+    if (g >= G) continue;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kAttWaves; ++w) M = fmaxf(M, lds[(w * GH + g) * REC + D]);
+    float Lsum = 0.f, val = 0.f;
+#pragma unroll
+    for (int w = 0; w < kAttWaves; ++w) {
+      const float* rec = lds + (w * GH + g) * REC;
+      const float sc = (rec[D] == M) ? 1.f : fast_exp(rec[D] - M);
+      Lsum += rec[D + 1] * sc;
+      val += rec[d] * sc;
+    }
+    const bool any = Lsum > 0.f;
+    if (COHERENT) {
+      store_coherent(mid_o_base + g * head_stride_o + d, any ? val / Lsum : 0.f);
+      if (d == 0) store_coherent(mid_lse_base + g * head_stride_lse, any ? M + logf(Lsum) : -INFINITY);
+    } else {
+      mid_o_base[g * head_stride_o + d] = any ? val / Lsum : 0.f;
+      if (d == 0) mid_lse_base[g * head_stride_lse] = any ? M + logf(Lsum) : -INFINITY;
+    }
+  }
+}
+
 // Final merge of the workgroup's states and the split's output.  Every lane
 // holds the state of (row slot, column chunk); GH heads per lane.
 template <int E, int LPR, int GH, bool COHERENT = false>
@@ -90,29 +122,7 @@ __device__ __forceinline__ void finish_split(float (&m)[GH], float (&l)[GH], flo
     }
   }
   __syncthreads();
-  for (int o = tid; o < GH * D; o += kAttThreads) {
-    const int g = o / D, d = o % D;
-    if (g >= G) continue;
-    float M = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < kAttWaves; ++w) M = fmaxf(M, lds[(w * GH + g) * REC + D]);
-    float Lsum = 0.f, val = 0.f;
-#pragma unroll
-    for (int w = 0; w < kAttWaves; ++w) {
-      const float* rec = lds + (w * GH + g) * REC;
-      const float sc = (rec[D] == M) ? 1.f : fast_exp(rec[D] - M);
-      Lsum += rec[D + 1] * sc;
-      val += rec[d] * sc;
-    }
-    const bool any = Lsum > 0.f;
-    if (COHERENT) {
-      store_coherent(mid_o_base + g * head_stride_o + d, any ? val / Lsum : 0.f);
-      if (d == 0) store_coherent(mid_lse_base + g * head_stride_lse, any ? M + logf(Lsum) : -INFINITY);
-    } else {
-      mid_o_base[g * head_stride_o + d] = any ? val / Lsum : 0.f;
-      if (d == 0) mid_lse_base[g * head_stride_lse] = any ? M + logf(Lsum) : -INFINITY;
-    }
-  }
+  combine_waves<D, GH, COHERENT>(lds, G, mid_o_base, mid_lse_base, head_stride_o, head_stride_lse);
 }
 
 constexpr int kMergeThreads = 256;
@@ -438,6 +448,314 @@ __global__ __launch_bounds__(kAttThreads) void dense_stage1_kernel(
   finish_split<E, LPR, GP>(m, l, acc, G, mo, ml, (int64_t)nsplit * D, (int64_t)nsplit, lds);
 }
 
+// ---------------------------------------------------------------------------
+// Dense flash-decode on the matrix cores: 16-bit K/V, D = 128, up to 16 query
+// heads per kv head.
+//
+// The lane-per-row kernel above spends, per K/V row, G dot products of 128 terms,
+// their cross-lane sums and G x 128 multiply-adds on the vector ALU; from four
+// heads per kv head on, that -- not the K/V stream -- is what bounds it (0.63 of
+// the HBM peak at G = 4, 0.25 at G = 7).  Here both products are MFMAs in the transposed orientation, with the query head as
+// the N index (lane x holds head x % 16 in every accumulator, heads past G are
+// zero columns):
+//   S^T[key, head] = K . Q^T      v_mfma_f32_16x16x32   A = 16 keys x 32 dims
+//   O^T[dim, head] = V^T . P^T    v_mfma_f32_16x16x16   A = 16 dims x 16 keys
+// so a head's running maximum and sum are over a lane's own registers and the
+// three other lane quarters, the rescale factor is per lane, and the
+// probabilities a lane computed (keys 4q..4q+3 of the block, q = lane / 16) are
+// the B operand it has to supply for those keys.
+//
+// A wave walks its own 16-key blocks (blocks wave, wave + 4, ... of the split);
+// K and V rows go global -> LDS directly, 1 KB (four whole rows) per
+// instruction, into the wave's private ring of STAGES blocks, so no barrier sits
+// in the loop and STAGES - 1 blocks per wave are in flight while one is
+// consumed.  The lane that copies 16-byte piece c of row r writes it to position
+// c ^ r of the row's 16 places: the K fragment reads (16 rows, same piece) and
+// the V reads (dwords of 4 rows x 16 neighbouring pieces) then hit 64 different
+// banks.  V^T is never materialised: a dword of V holds dims 2x and 2x + 1 of one
+// key, four such dwords (keys 4q..4q+3) split into their low and high halves are
+// the A operands of the two 16-dim blocks {2x + 32p} and {2x + 1 + 32p}, x < 16.
+// ---------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 att_bf16x8;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 att_f16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 att_f16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short att_s16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float att_f32x4;
+
+template <class DT>
+struct MmaType;
+template <>
+struct MmaType<DType_bf16> {
+  static __device__ __forceinline__ att_f32x4 qk(const uint4& a, const uint4& b, att_f32x4 c) {
+    union {
+      uint4 u;
+      att_bf16x8 v;
+    } x, y;
+    x.u = a;
+    y.u = b;
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x.v, y.v, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ att_f32x4 pv(const uint2& a, const uint2& b, att_f32x4 c) {
+    union {
+      uint2 u;
+      att_s16x4 v;
+    } x, y;
+    x.u = a;
+    y.u = b;
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(x.v, y.v, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    union {
+      bf2 v;
+      uint32_t u;
+    } r;
+    r.v = __builtin_convertvector(f2{lo, hi}, bf2);
+    return r.u;
+  }
+};
+template <>
+struct MmaType<DType_f16> {
+  static __device__ __forceinline__ att_f32x4 qk(const uint4& a, const uint4& b, att_f32x4 c) {
+    union {
+      uint4 u;
+      att_f16x8 v;
+    } x, y;
+    x.u = a;
+    y.u = b;
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(x.v, y.v, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ att_f32x4 pv(const uint2& a, const uint2& b, att_f32x4 c) {
+    union {
+      uint2 u;
+      att_f16x4 v;
+    } x, y;
+    x.u = a;
+    y.u = b;
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(x.v, y.v, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    union {
+      h2 v;
+      uint32_t u;
+    } r;
+    r.v = __builtin_convertvector(f2{lo, hi}, h2);
+    return r.u;
+  }
+};
+
+constexpr int kMmaKeys = 16;                            // keys per block of a wave
+constexpr int kMmaTileBytes = kMmaKeys * 128 * 2;       // one K or V tile
+constexpr int kMmaStageBytes = 2 * kMmaTileBytes;
+constexpr int kMmaHeads = 16;
+constexpr int kMmaMaxFlatBatch = SOCKET_WAVE;           // sequences one wave can scan
+
+// s_waitcnt vmcnt(N), also a compiler barrier for the LDS reads that follow
+template <int N>
+__device__ __forceinline__ void wait_copies() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Grid: one workgroup per (kv head, sequence, split), flattened.  With `flat`
+// (B <= 64) the splits that exist -- ceil(len_b / rows_per_split) per sequence --
+// are numbered consecutively from the lengths, so a ragged batch occupies the
+// first sum-of-splits workgroups and the rest of the grid (sized for the longest
+// possible sequence, the lengths live on the device) exits at once; otherwise the
+// grid is the rectangle B x nsplit.
+template <class DT, int STAGES>
+__global__ __launch_bounds__(kAttThreads) void dense_mma_kernel(
+    const uint16_t* __restrict__ q_, const uint16_t* __restrict__ k_, const uint16_t* __restrict__ v_,
+    int64_t q_sb, int64_t q_sh, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh,
+    int64_t v_ss, const int32_t* __restrict__ lens, float* __restrict__ mid_o, float* __restrict__ mid_lse,
+    int B, int Hq, int Hkv, int G, int T, int nsplit, int rows_per_split, float scale_log2, int flat) {
+  constexpr int D = 128;
+  extern __shared__ __attribute__((aligned(16))) unsigned char att_lds[];
+  __shared__ int item[3];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int prow = lane & 15, quarter = lane >> 4;
+
+  const int kvh = blockIdx.x % Hkv;
+  const int t = blockIdx.x / Hkv;
+  int b, s;
+  if (flat) {
+    if (wave == 0) {
+      const int n = lane < B ? (min(lens[lane], T) + rows_per_split - 1) / rows_per_split : 0;
+      int incl = n;
+#pragma unroll
+      for (int d = 1; d < SOCKET_WAVE; d <<= 1) {
+        const int up = __shfl_up(incl, d, SOCKET_WAVE);
+        if (lane >= d) incl += up;
+      }
+      if (t >= incl - n && t < incl) {
+        item[0] = lane;
+        item[1] = t - (incl - n);
+      }
+      if (lane == SOCKET_WAVE - 1) item[2] = incl;
+    }
+    __syncthreads();
+    if (t >= item[2]) return;
+    b = item[0];
+    s = item[1];
+  } else {
+    b = t / nsplit;
+    s = t % nsplit;
+  }
+  const int len = min(lens[b], T);
+  const int lo = s * rows_per_split;
+  const int hi = min(len, lo + rows_per_split);
+  if (hi <= lo) return;
+
+  const uint16_t* kbase = k_ + b * k_sb + kvh * k_sh;
+  const uint16_t* vbase = v_ + b * v_sb + kvh * v_sh;
+  // Q^T fragments (B operand): head prow, dims 32 ks + 8 quarter .. + 7
+  uint4 qf[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) qf[ks] = make_uint4(0, 0, 0, 0);
+  if (prow < G) {
+    const uint16_t* q = q_ + b * q_sb + (int64_t)(kvh * G + prow) * q_sh;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qf[ks] = *reinterpret_cast<const uint4*>(q + (4 * ks + quarter) * 8);
+  }
+
+  // The fragments must have arrived before the first copy is issued: the compiler
+  // counts the loads it knows of, not the LDS copies below, and would otherwise
+  // wait for "its" loads inside the loop with a count that drains every copy in
+  // flight, on every trip.
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].y), "v"(qf[ks].z), "v"(qf[ks].w));
+
+  unsigned char* ring = att_lds + wave * STAGES * kMmaStageBytes;
+  const int nblk = (hi - lo + kMmaKeys - 1) / kMmaKeys;
+  const int mine = nblk > wave ? (nblk - wave + kAttWaves - 1) / kAttWaves : 0;
+  // Block j of this wave into a ring stage.  Rows past the split's end are fetched
+  // from its last row (a live row, so the copy count per block is constant and
+  // nothing outside the split is touched); their scores are masked below.
+  // The walk starts at a block that differs from workgroup to workgroup and wraps
+  // (the softmax does not care about order): splits are a power-of-two number of
+  // bytes apart in a cache whose length is a power of two, and workgroups that
+  // start together would otherwise sweep the same few memory channels in step.
+  const int rot = (int)((blockIdx.x * 2654435761u) >> 8) % nblk;
+  auto block_of = [&](int j) {
+    const int i = wave + kAttWaves * j + rot;
+    return i >= nblk ? i - nblk : i;
+  };
+  auto fetch = [&](int j, int stage) {
+    const int key0 = lo + (j < mine ? block_of(j) : nblk) * kMmaKeys;
+    unsigned char* dst = ring + stage * kMmaStageBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = 4 * i + quarter;
+      const int key = min(key0 + r, hi - 1);
+      const int piece = prow ^ r;
+      lds_dma16(kbase + (int64_t)key * k_ss + piece * 8, dst + i * 1024);
+      lds_dma16(vbase + (int64_t)key * v_ss + piece * 8, dst + kMmaTileBytes + i * 1024);
+    }
+  };
+
+  float m_i = -INFINITY, l_part = 0.f;
+  att_f32x4 o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = att_f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int j = 0; j < STAGES - 1; ++j) fetch(j, j);
+  for (int j = 0; j < mine; ++j) {
+    fetch(j + STAGES - 1, (j + STAGES - 1) % STAGES);
+    wait_copies<(STAGES - 1) * 8>();
+    const unsigned char* st = ring + (j % STAGES) * kMmaStageBytes;
+    const uint4* kt = reinterpret_cast<const uint4*>(st);
+    const uint32_t* vt = reinterpret_cast<const uint32_t*>(st + kMmaTileBytes);
+
+    // ---- S^T: register i = key 4 quarter + i of the block against head prow
+    att_f32x4 sc = att_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) sc = MmaType<DT>::qk(kt[prow * 16 + ((4 * ks + quarter) ^ prow)], qf[ks], sc);
+    const int key0 = lo + block_of(j) * kMmaKeys + 4 * quarter;
+    float m_blk = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sc[i] = (key0 + i < hi) ? sc[i] : -INFINITY;
+      m_blk = fmaxf(m_blk, sc[i]);
+    }
+    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, SOCKET_WAVE));
+    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, SOCKET_WAVE));
+    // The maximum is kept on the raw dot products and the (positive) scale applied
+    // to the difference, in base 2: the largest score of a block then gives exactly
+    // exp2(0) whatever its magnitude, which scaling first and subtracting the rounded
+    // maximum afterwards does not guarantee.
+    const float m_new = fmaxf(m_i, m_blk);
+    const bool blind = m_new == -INFINITY;
+    const float alpha = blind ? 1.f : __builtin_amdgcn_exp2f((m_i - m_new) * scale_log2);
+    const float ref = blind ? 0.f : m_new;
+    float p[4], psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      p[i] = __builtin_amdgcn_exp2f((sc[i] - ref) * scale_log2);
+      psum += p[i];
+    }
+    l_part = l_part * alpha + psum;
+    m_i = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        o[i][0] *= alpha;
+        o[i][1] *= alpha;
+        o[i][2] *= alpha;
+        o[i][3] *= alpha;
+      }
+    }
+    // ---- O^T += V^T . P^T
+    const uint2 pf = make_uint2(MmaType<DT>::pack2(p[0], p[1]), MmaType<DT>::pack2(p[2], p[3]));
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp) {
+      uint32_t w[4];
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int r = 4 * quarter + jj;
+        w[jj] = vt[r * 64 + (((4 * pp + (prow >> 2)) ^ r) << 2) + (prow & 3)];
+      }
+      const uint2 lo2 = make_uint2(__builtin_amdgcn_perm(w[1], w[0], 0x05040100u),
+                                   __builtin_amdgcn_perm(w[3], w[2], 0x05040100u));
+      const uint2 hi2 = make_uint2(__builtin_amdgcn_perm(w[1], w[0], 0x07060302u),
+                                   __builtin_amdgcn_perm(w[3], w[2], 0x07060302u));
+      o[2 * pp] = MmaType<DT>::pv(lo2, pf, o[2 * pp]);
+      o[2 * pp + 1] = MmaType<DT>::pv(hi2, pf, o[2 * pp + 1]);
+    }
+  }
+
+  // the copies still under way (fetched past the wave's last block) must land
+  // before the ring is reused for the waves' records
+  wait_copies<0>();
+  float l = l_part;
+  l += __shfl_xor(l, 16, SOCKET_WAVE);
+  l += __shfl_xor(l, 32, SOCKET_WAVE);
+  __syncthreads();
+  constexpr int REC = D + 2;
+  float* lds = reinterpret_cast<float*>(att_lds);
+  if (prow < G) {
+    float* rec = lds + (wave * kMmaHeads + prow) * REC;
+    // register i of accumulator 2 pp + e: dim 8 quarter + 2 i + 32 pp + e
+#pragma unroll
+    for (int pp = 0; pp < 4; ++pp)
+#pragma unroll
+      for (int e = 0; e < 2; ++e)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rec[8 * quarter + 2 * i + 32 * pp + e] = o[2 * pp + e][i];
+    if (quarter == 0) {
+      rec[D] = m_i * (scale_log2 * 0.6931471805599453f);   // the records hold scaled scores, natural base
+      rec[D + 1] = l;
+    }
+  }
+  __syncthreads();
+  const int h0 = kvh * G;
+  combine_waves<D, kMmaHeads, false>(lds, G, mid_o + (((int64_t)b * Hq + h0) * nsplit + s) * D,
+                                     mid_lse + ((int64_t)b * Hq + h0) * nsplit + s, (int64_t)nsplit * D,
+                                     (int64_t)nsplit);
+}
+
 struct AttArgs {
   const void *q, *k, *v;
   int dtype;
@@ -498,6 +816,42 @@ int launch_dense_stage1(const AttArgs& a, const int32_t* lens, float* mid_o, flo
   return SOCKET_OK;
 }
 
+// Two ring stages per wave (64 KB per workgroup, two workgroups per CU) and splits
+// of at least 1024 rows measured best from one sequence of 32k rows to 16 ragged
+// ones; deeper rings (one workgroup per CU) lose at batch 1 and gain nothing at
+// the large shapes.  Measured at 5.4-5.9 TB/s for 1 to 8 heads per kv head, which
+// is above the lane-per-row kernel at every group size, so every 16-bit D = 128
+// cache takes this path.
+constexpr int kMmaStages = 2;
+constexpr int kMmaMinRows = 1024;
+
+bool dense_uses_mma(int dtype, int D, int G) {
+  return (dtype == SOCKET_BF16 || dtype == SOCKET_F16) && D == 128 && G <= kMmaHeads;
+}
+
+template <class DT>
+int launch_dense_mma(const AttArgs& a, const int32_t* lens, float* mid_o, float* mid_lse, int B, int Hq,
+                     int Hkv, int T, int nsplit, int rows_per_split, hipStream_t s) {
+  auto kern = dense_mma_kernel<DT, kMmaStages>;
+  constexpr size_t ring = (size_t)kAttWaves * kMmaStages * kMmaStageBytes;
+  constexpr size_t records = (size_t)kAttWaves * kMmaHeads * (128 + 2) * sizeof(float);
+  constexpr size_t lds = ring > records ? ring : records;
+  static std::atomic<bool> ready{false};
+  if (!ready.load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)lds) != hipSuccess)
+      return SOCKET_ERR_LAUNCH;
+    ready.store(true, std::memory_order_release);
+  }
+  SOCKET_REQUIRE((int64_t)B * nsplit * Hkv < (int64_t)1 << 31, SOCKET_ERR_SHAPE);
+  const float scale_log2 = 1.4426950408889634f / sqrtf(128.f);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(B * nsplit * Hkv)), dim3(kAttThreads), lds, s, (const uint16_t*)a.q,
+                     (const uint16_t*)a.k, (const uint16_t*)a.v, a.q_sb, a.q_sh, a.k_sb, a.k_sh, a.k_ss, a.v_sb,
+                     a.v_sh, a.v_ss, lens, mid_o, mid_lse, B, Hq, Hkv, Hq / Hkv, T, nsplit, rows_per_split,
+                     scale_log2, B <= kMmaMaxFlatBatch ? 1 : 0);
+  return SOCKET_OK;
+}
+
 int launch_stage2(const float* mid_o, const float* mid_lse, const int32_t* len, int64_t len_sb,
                   int64_t len_sh, void* out, int out_dtype, int64_t out_sb, int64_t out_sh, int B,
                   int Hq, int D, int nsplit, int block_seq, hipStream_t s) {
@@ -514,15 +868,15 @@ int launch_stage2(const float* mid_o, const float* mid_lse, const int32_t* len, 
   return SOCKET_OK;
 }
 
-int dense_rows_per_split(int B, int Hkv, int T) {
-  // Aim at >= 8 workgroups per CU over the whole grid, splits of >= 256 rows.
+int dense_rows_per_split(int B, int Hkv, int T, int min_rows = 256) {
+  // Aim at >= 8 workgroups per CU over the whole grid, splits of >= min_rows rows.
   const SocketDeviceLimits& lim = socket_device_limits();
   const int want = 8 * lim.cu_count;
   int nsplit = (want + B * Hkv - 1) / (B * Hkv);
   if (nsplit < 1) nsplit = 1;
   int rows = (T + nsplit - 1) / nsplit;
   rows = (rows + 63) / 64 * 64;
-  if (rows < 256) rows = 256;
+  if (rows < min_rows) rows = min_rows;
   return rows;
 }
 
@@ -768,7 +1122,8 @@ extern "C" int socket_dense_decode(const void* q, const void* k, const void* v, 
   SOCKET_REQUIRE(workspace_bytes >= socket_dense_decode_workspace_bytes(B, Hq, D, T),
                  SOCKET_ERR_WORKSPACE);
   SOCKET_REQUIRE(socket_aligned16(workspace), SOCKET_ERR_ALIGN);
-  const int rows = dense_rows_per_split(B, Hkv, T);
+  const bool mma = dense_uses_mma(dtype, D, Hq / Hkv);
+  const int rows = dense_rows_per_split(B, Hkv, T, mma ? kMmaMinRows : 256);
   const int nsplit = (T + rows - 1) / rows;
   float* mid_o = (float*)workspace;
   float* mid_lse = mid_o + (size_t)B * Hq * nsplit * D;
@@ -779,7 +1134,10 @@ extern "C" int socket_dense_decode(const void* q, const void* k, const void* v, 
     else if (dtype == SOCKET_F16) st = launch_dense_stage1<DType_f16, DD>(a, lens, mid_o, mid_lse, B, Hq, Hkv, T, nsplit, rows, s); \
     else st = launch_dense_stage1<DType_f32, DD>(a, lens, mid_o, mid_lse, B, Hq, Hkv, T, nsplit, rows, s); \
   } while (0)
-  if (D == 128) SOCKET_DENSE_D(128);
+  if (mma)
+    st = dtype == SOCKET_BF16 ? launch_dense_mma<DType_bf16>(a, lens, mid_o, mid_lse, B, Hq, Hkv, T, nsplit, rows, s)
+                              : launch_dense_mma<DType_f16>(a, lens, mid_o, mid_lse, B, Hq, Hkv, T, nsplit, rows, s);
+  else if (D == 128) SOCKET_DENSE_D(128);
   else if (D == 64) SOCKET_DENSE_D(64);
   else if (D == 32) SOCKET_DENSE_D(32);
   else SOCKET_DENSE_D(16);

@@ -423,6 +423,53 @@ def test_dense_decode_ragged(dev):
     assert (got.cpu().double() - want).abs().max() <= 2e-2
 
 
+@pytest.mark.parametrize("dtype,B,Hq,Hkv,T,strided", [
+    (torch.bfloat16, 2, 8, 2, 3000, False),     # G = 4
+    (torch.bfloat16, 3, 10, 2, 2500, True),     # G = 5, K/V as [B,T,Hkv,D] views
+    (torch.float16, 2, 14, 2, 1111, False),     # G = 7, half precision
+    (torch.bfloat16, 1, 16, 1, 4097, False),    # G = 16: every column of the tile is a head
+    (torch.bfloat16, 1, 12, 1, 600, False),     # G = 12
+    (torch.bfloat16, 70, 8, 1, 300, False),     # more sequences than one wave can scan: rectangular grid
+])
+def test_dense_decode_matrix_core_path(dev, dtype, B, Hq, Hkv, T, strided):
+    """16-bit caches with four or more heads per kv head run the MFMA dense
+    kernel: ragged lengths down to one row, lengths off the 16-key block and off
+    the split, scores that must be masked, and rows after a sequence's end holding
+    huge values that must never be read into a result."""
+    g = torch.Generator().manual_seed(B * 1000 + Hq)
+    D = 128
+    q = torch.randn(B, Hq, D, generator=g).to(dtype)
+    k = torch.randn(B, Hkv, T, D, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, T, D, generator=g).to(dtype)
+    lens = torch.randint(1, T + 1, (B,), generator=g, dtype=torch.int32)
+    lens[0] = T
+    if B > 1:
+        lens[1] = 1
+    if B > 2:
+        lens[2] = 17
+    big = 3e4 if dtype == torch.bfloat16 else 100.0       # (4 * big must stay finite in the cache's type)
+    for b in range(B):                      # poison what lies beyond each sequence
+        k[b, :, int(lens[b]):] = big
+        v[b, :, int(lens[b]):] = -big
+    if strided:
+        kd = k.to(dev).transpose(1, 2).contiguous().transpose(1, 2)      # [B,Hkv,T,D] view of [B,T,Hkv,D]
+        vd = v.to(dev).transpose(1, 2).contiguous().transpose(1, 2)
+        assert not kd.is_contiguous()
+    else:
+        kd, vd = k.to(dev), v.to(dev)
+    got = socket_kernels.dense_decode_fwd(q.to(dev), kd, vd, lens.to(dev))
+    want = orc.dense_attend(q, k, v, lens)
+    assert torch.isfinite(got.float()).all()
+    assert (got.cpu().double() - want).abs().max() <= 2e-2
+    # sharply peaked rows: one key dominates (scores of the order of 1e11 where the
+    # query was taken from a poisoned row), the result is that key's value row
+    q2 = (k[:, :, 5].repeat_interleave(Hq // Hkv, 1).float() * 4).to(dtype)
+    lens2 = torch.full((B,), min(T, 64), dtype=torch.int32)
+    got2 = socket_kernels.dense_decode_fwd(q2.to(dev), kd, vd, lens2.to(dev))
+    want2 = orc.dense_attend(q2, k, v, lens2)
+    assert (got2.cpu().double() - want2).abs().max() <= 2e-2
+
+
 # ---------------------------------------------------------------- K1 hash
 @pytest.mark.parametrize("dtype,L,P,S,D", [(torch.bfloat16, 60, 10, 1000, 128), (torch.float32, 32, 8, 333, 128),
                                            (torch.float16, 7, 5, 65, 128), (torch.bfloat16, 48, 10, 1, 128),
