@@ -72,7 +72,6 @@ def algorithmic_bytes(w, lens=None, budgets=None):
         "score_f32_table": w.Hkv * tok * (wc + 2 + 4 * G),
         "score_reference_layout": w.Hkv * tok * (wc + 2 + 4 * G),
         "select": sel,
-        "select_own_range": sel,
         "attend": w.Hq * kt * (4 * w.D + 4) + w.B * w.Hq * 4 * w.D,
         "dense": w.Hkv * tok * 4 * w.D,
     }
@@ -323,11 +322,11 @@ class Step:
 
     def k_score_ref(self):
         return self.hc.score_packed(self.q_table, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
-                                    out=self.scores_buf, with_range=True)
+                                    out=self.scores_buf)
 
     def k_score_grouped(self):
         return self.hc.score_packed(self.q_table_grouped, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
-                                    out=self.scores_buf, with_range=True, n_heads=self.w.Hq)
+                                    out=self.scores_buf, n_heads=self.w.Hq)
 
     def k_score_f32(self):
         return self.hc.score_packed(self.q_table_f32, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
@@ -336,9 +335,9 @@ class Step:
     def k_score(self):
         return self.k_score_grouped() if self.use_grouped else self.k_score_ref()
 
-    def k_select(self, scores, rng=None):
+    def k_select(self, scores):
         w = self.w
-        return self.sp.select_list(scores, w.sink, w.window, w.M, lens=self.lens, budgets=self.budgets, row_range=rng)
+        return self.sp.select_list(scores, w.sink, w.window, w.M, lens=self.lens, budgets=self.budgets)
 
     def k_attend(self, sl, ln):
         return self.sk.sparse_attention_fwd(self.inp.q, self.inp.k, self.inp.v, sl, ln)
@@ -443,8 +442,8 @@ def measure_workload(w, dev, steps, warmup, args, full):
     the parity gates (the headline workload)."""
     st = Step(w, dev, reference_table_layout=args.reference_table_layout)
     prefill_us = time_launches(st.prefill_hash, 3, warmup=1)
-    scores, rng = st.k_score()
-    sl, ln = st.k_select(scores, rng)
+    scores = st.k_score()
+    sl, ln = st.k_select(scores)
     out = st.k_attend(sl, ln)
     torch.cuda.synchronize()
     iters = max(steps, 1)
@@ -452,14 +451,13 @@ def measure_workload(w, dev, steps, warmup, args, full):
     per = {
         "hash": time_graph(st.k_hash, iters),
         "score": time_graph(st.k_score, iters),
-        "select": time_graph(lambda: st.k_select(scores, rng), iters),
+        "select": time_graph(lambda: st.k_select(scores), iters),
         "attend": time_graph(lambda: st.k_attend(sl, ln), iters),
         "dense": time_graph(st.k_dense, max(iters // 2, 5), per_graph=5),
     }
     if full:
         per["score_reference_layout"] = time_graph(st.k_score_ref, iters)
         per["score_f32_table"] = time_graph(st.k_score_f32, iters)
-        per["select_own_range"] = time_graph(lambda: st.k_select(scores), iters)
     ab = st.abytes
     kernels = {k: {"us": round(v, 2), "algorithmic_MB": round(ab[k] / 1e6, 2), "gbs": round(ab[k] / v / 1e3, 1),
                    "hbm_frac": round(ab[k] / v / 1e3 / HBM_PEAK_GBS, 4)} for k, v in per.items()}
@@ -500,6 +498,51 @@ def measure_workload(w, dev, steps, warmup, args, full):
         "new_keys_hashed_per_step": w.B * w.Hkv * w.new_keys,
     }
     return rec, st, per
+
+
+def drop_in_operator(st):
+    """`sparse.build_sparse_list_decode` on the reference's own operands
+    (GPT-FAST/kernels/sparse.py:16-95: q_probs [B,H,L,R] in the model's type,
+    int16 codes per QUERY head [B,H,L,T], fp16 value norms and a boolean mask per
+    query head) at this workload's size: what a caller that keeps the reference's
+    cache layout pays.  Eager launches, torch's relayouts included, as the
+    reference's call site runs it; the collision kernel alone beside it."""
+    from socket_amd import sparse
+    w = st.w
+    G = w.Hq // w.Hkv
+    T = w.T
+    k_hard = st.hc.unpack_codes(st.codes, w.L, w.P, 0, T).repeat_interleave(G, dim=1).contiguous()      # [B,H,L,T] int16
+    v_norm = st.v_norm[:, :, :T].repeat_interleave(G, dim=1).contiguous()
+    pos = torch.arange(T, device=st.dev)
+    lens = st.lens if st.lens is not None else torch.full((w.B,), T, dtype=torch.int32, device=st.dev)
+    allowed = (pos[None, None, :] < lens[:, None, None]).expand(w.B, w.Hq, T).contiguous()
+    q_probs = st.q_table                                                                                 # [B,H,L,R] bf16
+
+    def op():
+        return sparse.build_sparse_list_decode(q_probs, k_hard, v_norm, allowed, w.sink, w.window, w.M)
+
+    ext = sparse._get_soft_hash_ext()
+    q32 = q_probs.float().unsqueeze(2).contiguous()
+    a_ext, v_ext = allowed.unsqueeze(2).contiguous(), v_norm.float().unsqueeze(2).contiguous()
+    sl, ln = op()
+    # the packed path's selection for the same step (its bf16-table sums may differ from
+    # this fp32-table kernel's in the last place, so near-ties at the cut may swap)
+    want_sl, want_ln = st.k_select(st.k_score())
+    overlap = 1.0
+    for b in (0, w.B - 1):
+        for h in (0, w.Hq - 1):
+            a = set(sl[b, h, :int(ln[b, h])].tolist())
+            c = set(want_sl[b, h, :int(want_ln[b, h])].tolist())
+            overlap = min(overlap, len(a & c) / max(len(c), 1))
+    settle(op, 20.0)
+    total = time_launches(op, 10, warmup=2)
+    kern = time_graph(lambda: ext.soft_hash_collision(q32, k_hard, a_ext, v_ext), 20)
+    nbytes = w.B * w.Hq * T * (2 * w.L + 1 + 4 + 4)         # int16 codes, mask byte, fp32 norm, fp32 score per (head, token)
+    return {"operator_us": round(total, 1), "collision_kernel_us": round(kern, 1),
+            "collision_kernel_algorithmic_MB": round(nbytes / 1e6, 1),
+            "collision_kernel_gbs": round(nbytes / kern / 1e3, 1),
+            "list_overlap_with_packed_path_min": round(overlap, 4),
+            "operands": "q_probs bf16 [B,H,L,R], int16 codes [B,H,L,T] per query head, fp16 norms, bool mask"}
 
 
 def decode_tok_s(dev, prompt_len, new_tokens, n_layer=None, kinds=("sparse", "dense")):
@@ -596,11 +639,11 @@ def main():
                               "mfma_tflops": round(2.0 * rows * w.D * w.L * w.P / us / 1e6, 1)}))
             return
         st.prefill_hash()
-        scores, rng = st.k_score()
-        sl, ln = st.k_select(scores, rng)
+        scores = st.k_score()
+        sl, ln = st.k_select(scores)
         torch.cuda.synchronize()
         fn = {"score": st.k_score_ref, "score_f32": st.k_score_f32, "score_grouped": st.k_score_grouped,
-              "select": lambda: st.k_select(scores, rng), "attend": lambda: st.k_attend(sl, ln), "hash": st.k_hash,
+              "select": lambda: st.k_select(scores), "attend": lambda: st.k_attend(sl, ln), "hash": st.k_hash,
               "dense": st.k_dense, "step": st.step}[args.only]
         settle(fn)
         us = time_launches(fn, iters, warmup=args.warmup)
@@ -649,6 +692,8 @@ def main():
         "input_generation_s": rec["input_generation_s"],
     }
 
+    if not args.no_extra and w.name == "c3":
+        result["drop_in_operator"] = drop_in_operator(st)
     if not args.no_cpu:
         T, Hkv, Hq = w.T, w.Hkv, w.Hq
         lens, budgets = st.lens, st.budgets
@@ -672,6 +717,8 @@ def main():
             for k in ("ms_per_step", "parity", "input_generation_s", "kernel_timing"):
                 r.pop(k, None)
             r["steps"] = sub_steps
+            if name == "c2":
+                r["drop_in_operator"] = drop_in_operator(s2)
             result[name] = r
             del s2
             torch.cuda.empty_cache()

@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libsocket_hip.so")
-SOURCES = ["common.hip", "score.hip", "topk.hip", "attend.hip", "hash.hip", "softhash.hip", "decode_ops.hip", "block_sparse.hip"]
+SOURCES = ["common.hip", "score.hip", "collide.hip", "topk.hip", "attend.hip", "hash.hip", "softhash.hip", "decode_ops.hip", "block_sparse.hip"]
 ARCH = "gfx950"
 # Packed-FP32 VALU ops are switched off for every device translation unit.
 FLAGS = [

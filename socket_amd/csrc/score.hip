@@ -18,8 +18,8 @@
 //    A table given in the grouped layout (the LDS image itself, written by the
 //    soft-hash kernel) is copied rather than interleaved, and for large launches
 //    the copy is global_load_lds: global memory straight into LDS.
-//  * collision_i16_kernel: the reference's own operand layout (int16 codes per
-//    query head), for drop-in callers.
+// (The reference's own operand layout, int16 codes per query head, is served by
+// collide.hip.)
 #include <type_traits>
 #ifdef SOCKET_SCORE_PLAN_OVERRIDE
 #include <cstdio>
@@ -990,70 +990,6 @@ int dispatch_g(const ScoreArgs& a) {
   return dispatch_tile<4, TT>(a, plan);
 }
 
-// ---------------------------------------------------------------------------
-// reference-layout scorer (int16 codes per query head)
-// ---------------------------------------------------------------------------
-__device__ __forceinline__ float table_to_f32(float x) { return x; }
-__device__ __forceinline__ float table_to_f32(uint16_t x) { return f16_bits_to_f32(x); }
-
-// One thread per token; tables staged in LDS in slices of `ct` tables
-// (ct == 0: R too large for LDS, gather from global memory instead).
-template <typename QT, int THREADS>
-__global__ __launch_bounds__(THREADS) void collision_i16_kernel(
-    const QT* __restrict__ q_probs, const int16_t* __restrict__ key_buckets,
-    const uint8_t* __restrict__ allowed, const QT* __restrict__ v_hist, float* __restrict__ out,
-    int L, int R, int T, int ct) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  QT* table = reinterpret_cast<QT*>(lds_raw);
-  const int bh = blockIdx.y;
-  const int t = blockIdx.x * THREADS + threadIdx.x;
-  const bool in = t < T;
-  const QT* qp = q_probs + (int64_t)bh * L * R;
-  const int16_t* kb = key_buckets + (int64_t)bh * L * T;
-  float sum = 0.f;
-  if (ct == 0) {
-    if (in) {
-      for (int l = 0; l < L; ++l) {
-        const int r = (int)kb[(int64_t)l * T + t];
-        if (r >= 0 && r < R) sum += table_to_f32(qp[(int64_t)l * R + r]);
-      }
-    }
-  } else {
-    for (int l0 = 0; l0 < L; l0 += ct) {
-      const int nt = min(ct, L - l0);
-      __syncthreads();
-      for (int i = threadIdx.x; i < nt * R; i += THREADS) table[i] = qp[(int64_t)l0 * R + i];
-      __syncthreads();
-      if (in) {
-        for (int l = 0; l < nt; ++l) {
-          const int r = (int)kb[(int64_t)(l0 + l) * T + t];
-          if (r >= 0 && r < R) sum += table_to_f32(table[l * R + r]);
-        }
-      }
-    }
-  }
-  if (in) {
-    const int64_t o = (int64_t)bh * T + t;
-    out[o] = allowed[o] ? sum * table_to_f32(v_hist[o]) : -INFINITY;
-  }
-}
-
-template <typename QT>
-int launch_collision_i16(const QT* q_probs, const int16_t* key_buckets, const uint8_t* allowed,
-                         const QT* v_hist, float* out, int B, int H, int L, int R, int T,
-                         hipStream_t stream) {
-  constexpr int THREADS = 256;
-  const size_t per_table = (size_t)R * sizeof(QT);
-  int ct = (int)((48 * 1024) / per_table);
-  if (ct > L) ct = L;
-  const size_t lds = (size_t)ct * per_table;
-  dim3 grid((T + THREADS - 1) / THREADS, B * H);
-  hipLaunchKernelGGL((collision_i16_kernel<QT, THREADS>), grid, dim3(THREADS), lds, stream, q_probs,
-                     key_buckets, allowed, v_hist, out, L, R, T, ct);
-  SOCKET_LAUNCH_CHECK();
-  return SOCKET_OK;
-}
-
 }  // namespace
 
 namespace {
@@ -1202,22 +1138,3 @@ extern "C" int socket_group_q_probs(const void* q_probs, int q_dtype, void* q_ta
   return SOCKET_OK;
 }
 
-extern "C" int socket_soft_hash_collision(const float* q_probs, const int16_t* key_buckets,
-                                          const uint8_t* allowed, const float* v_hist, float* out,
-                                          int B, int H, int L, int R, int T, void* stream) {
-  SOCKET_REQUIRE(q_probs && key_buckets && allowed && v_hist && out, SOCKET_ERR_NULL);
-  SOCKET_REQUIRE(B > 0 && H > 0 && L > 0 && R > 0 && T > 0, SOCKET_ERR_SHAPE);
-  SOCKET_REQUIRE((int64_t)B * H <= 65535, SOCKET_ERR_SHAPE);
-  return launch_collision_i16<float>(q_probs, key_buckets, allowed, v_hist, out, B, H, L, R, T,
-                                     (hipStream_t)stream);
-}
-
-extern "C" int socket_soft_hash_score_f16(const uint16_t* q_probs, const int16_t* key_buckets,
-                                          const uint16_t* v_norm, const uint8_t* allowed, float* out,
-                                          int B, int H, int L, int R, int T, void* stream) {
-  SOCKET_REQUIRE(q_probs && key_buckets && allowed && v_norm && out, SOCKET_ERR_NULL);
-  SOCKET_REQUIRE(B > 0 && H > 0 && L > 0 && R > 0 && T > 0, SOCKET_ERR_SHAPE);
-  SOCKET_REQUIRE((int64_t)B * H <= 65535, SOCKET_ERR_SHAPE);
-  return launch_collision_i16<uint16_t>(q_probs, key_buckets, allowed, v_norm, out, B, H, L, R, T,
-                                        (hipStream_t)stream);
-}

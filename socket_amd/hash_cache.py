@@ -281,8 +281,11 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     q [B,Hq,D]; q_probs [B,Hq,L,R]; T = number of cached tokens to consider (an
     upper bound when `lens` gives per-sequence lengths).  Returns out [B,Hq,D].
     """
-    scores, rng = score_packed(q_probs, codes, v_norm, T, P, lens=lens, with_range=True, n_heads=q.shape[1])
-    sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets, row_range=rng)
+    # (no per-tile key ranges from the scorer: the selection draws its threshold from a
+    # sample of the row and only a row whose sample misleads it falls back to a pass
+    # that would use them; tracking them costs the scorer more than that pass saves)
+    scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens, n_heads=q.shape[1])
+    sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets)
     B, Hq, D = q.shape
     if fits_static_scratch(B, Hq, D, sparse_list.shape[-1]):
         # one launch (the last split of a row merges it) on the library's own scratch array;

@@ -110,21 +110,31 @@ def test_score_packed_collision_counts(dev):
     assert got[0, 2, 17] == 120.0 and got[0, 0, 99] >= 60.0
 
 
-@pytest.mark.parametrize("L,R,T", [(32, 256, 777), (60, 1024, 4096), (3, 32768, 100)])
+@pytest.mark.parametrize("L,R,T", [(32, 256, 777), (60, 1024, 4096), (3, 32768, 100), (60, 1024, 9000),
+                                   (17, 1024, 10001), (5, 8192, 2056), (40, 2048, 16384)])
 def test_reference_layout_scorer(dev, L, R, T):
+    """Rows on and off the 16-byte grid, one to several table slices in LDS, more
+    than one tile of tokens per row, codes outside [0, R) (they add nothing)."""
     g = torch.Generator().manual_seed(L + T)
     B, H = 2, 3
     q_probs = torch.rand(B, H, L, R, generator=g)
     codes = torch.randint(0, R, (B, H, L, T), generator=g, dtype=torch.int32).to(torch.int16)
+    if R < 32768:
+        stray = torch.rand(B, H, L, T, generator=g)
+        codes[stray < 0.01] = -1
+        codes[stray > 0.99] = R
     allowed = torch.rand(B, H, T, generator=g) > 0.2
     v_hist = torch.rand(B, H, T, generator=g) * 5
     ext = load_soft_hash_collision(3)
     got = ext.soft_hash_collision(q_probs.unsqueeze(2).contiguous().to(dev), codes.to(dev),
                                   allowed.unsqueeze(2).contiguous().to(dev),
                                   v_hist.unsqueeze(2).contiguous().to(dev)).squeeze(2).cpu()
-    assert torch.equal(got, orc.collision_score(q_probs, codes, allowed, v_hist))
+    # the oracle sees the strays as hits of an extra all-zero bucket (x + 0.0 == x)
+    padded = torch.cat([q_probs, torch.zeros(B, H, L, 1)], -1)
+    mapped = torch.where((codes < 0) | (codes.int() >= R), torch.full_like(codes.int(), R), codes.int())
+    assert torch.equal(got, orc.collision_score(padded, mapped, allowed, v_hist))
     got16 = soft_hash_score(q_probs.half().to(dev), codes.to(dev), v_hist.half().to(dev), allowed.to(dev)).cpu()
-    assert torch.equal(got16, orc.collision_score_vnorm16(q_probs.half(), codes, v_hist.half(), allowed))
+    assert torch.equal(got16, orc.collision_score_vnorm16(padded.half(), mapped, v_hist.half(), allowed))
 
 
 REF_SO = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle", "_ref", "libref_scorer.so")
