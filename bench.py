@@ -441,7 +441,8 @@ def measure_workload(w, dev, steps, warmup, args, full):
     workload.  `full`: also the scorer's other table layouts, the prefill hash and
     the parity gates (the headline workload)."""
     st = Step(w, dev, reference_table_layout=args.reference_table_layout)
-    prefill_us = time_launches(st.prefill_hash, 3, warmup=1)
+    settle(st.prefill_hash)
+    prefill_us = time_launches(st.prefill_hash, 10, warmup=2)
     scores = st.k_score()
     sl, ln = st.k_select(scores)
     out = st.k_attend(sl, ln)
@@ -633,6 +634,7 @@ def main():
     if args.only:
         st = Step(w, dev, reference_table_layout=args.reference_table_layout)
         if args.only == "prefill_hash":
+            settle(st.prefill_hash)
             us = time_launches(st.prefill_hash, iters, warmup=args.warmup)
             rows = w.B * w.Hkv * w.T
             print(json.dumps({"only": "prefill_hash", "workload": w.name, "us": round(us, 1), "rows": rows,
