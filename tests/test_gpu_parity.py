@@ -480,6 +480,34 @@ def test_dense_decode_matrix_core_path(dev, dtype, B, Hq, Hkv, T, strided):
     assert (got2.cpu().double() - want2).abs().max() <= 2e-2
 
 
+@pytest.mark.parametrize("draw", range(12))
+def test_dense_decode_random_shapes(dev, draw):
+    """Drawn geometries for the MFMA dense kernel: 1 to 16 heads per kv head, 1 to 5
+    sequences of 1 to 6000 rows (one to several splits, blocks and waves with
+    nothing to do), both 16-bit types, contiguous caches and `[B,T,Hkv,D]` views."""
+    import random
+    rnd = random.Random(7000 + draw)
+    G = rnd.choice([1, 2, 3, 4, 6, 7, 8, 11, 16])
+    Hkv = rnd.choice([1, 2, 3])
+    B = rnd.randint(1, 5)
+    T = rnd.choice([1, 15, 16, 17, 63, 64, 65, 500, 1023, 1025, 2500, 6000])
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    g = torch.Generator().manual_seed(7000 + draw)
+    q = torch.randn(B, Hkv * G, 128, generator=g).to(dtype)
+    k = torch.randn(B, Hkv, T, 128, generator=g).to(dtype)
+    v = torch.randn(B, Hkv, T, 128, generator=g).to(dtype)
+    lens = torch.randint(1, T + 1, (B,), generator=g, dtype=torch.int32)
+    lens[rnd.randrange(B)] = T
+    print(f"G{G} Hkv{Hkv} B{B} T{T} {dtype} lens {lens.tolist()}", flush=True)
+    kd, vd = k.to(dev), v.to(dev)
+    if rnd.random() < 0.5:
+        kd = kd.transpose(1, 2).contiguous().transpose(1, 2)
+        vd = vd.transpose(1, 2).contiguous().transpose(1, 2)
+    got = socket_kernels.dense_decode_fwd(q.to(dev), kd, vd, lens.to(dev))
+    want = orc.dense_attend(q, k, v, lens)
+    assert (got.cpu().double() - want).abs().max() <= 2e-2
+
+
 # ---------------------------------------------------------------- K1 hash
 @pytest.mark.parametrize("dtype,L,P,S,D", [(torch.bfloat16, 60, 10, 1000, 128), (torch.float32, 32, 8, 333, 128),
                                            (torch.float16, 7, 5, 65, 128), (torch.bfloat16, 48, 10, 1, 128),
