@@ -9,12 +9,16 @@ configuration 3 (batch 4, 32/8 heads, head dim 128, 131072-token bf16 cache,
 L=60 x P=10, top-k 2048 + 4 sink + 256 window).
 
 Prints one JSON line.  `value` is microseconds per layer per step of the sparse
-path on configuration 3, exactly --steps graph replays after --warmup; `roofline`
+path on configuration 3, exactly --steps graph replays after --warmup, taken
+in the sustained power state of a decode loop (a settle phase of untimed
+replays comes first; the figure of a burst that starts on an idle GPU is
+reported beside it as `power_state.us_per_step_from_idle`); `roofline`
 prices the scorer (the kernel moving the most bytes) against HBM peak; `kernels`
 does the same for every kernel of the step and for the dense flash-decode
 comparator on the same GPU (each timed as a HIP-graph replay of ten launches, so
 small kernels are not priced at the cost of an eager Python call); `c2` and `c5`
-are the same records for configurations 2 and 5; `decode_tok_s` is the end-to-end
+are the same records for configurations 2 and 5; `drop_in_operator` times
+`build_sparse_list_decode` on the reference's own operand layout; `decode_tok_s` is the end-to-end
 greedy decode of the 32-layer Llama-3.1-8B-shaped model, sparse and dense, at
 128k context and at configuration 4's 65536-token prompt; `cpu_baseline` is the
 CPU oracle timed on the host's cores on a slice of configuration 3.
