@@ -361,7 +361,12 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
     const int32_t* __restrict__ pos_b, int t0, int Hkv, int S, int L, int P, int NW, int64_t Tcap,
     int tiles_per_row, int n_tiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (the wave index as a scalar: every address that depends on it -- this wave's
+  // words of the code cache above all -- then stays out of the vector registers;
+  // with it in a VGPR the kernel spilled three registers, and each reload in the
+  // middle of a tile came with a vmcnt(0) that also waited for the NEXT tile's
+  // copies, so the copies never overlapped the contraction)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int prow = lane & 15, quarter = lane >> 4;
   const int cpw = 32 / P;
   const bool with_values = v_ != nullptr;

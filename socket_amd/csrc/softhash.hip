@@ -17,6 +17,8 @@
 // then every lane owns runs of four buckets and makes three sweeps over them
 // (maximum, sum of exponentials, normalised write), recomputing the K-term
 // logits each time rather than holding R/64 of them per head in registers.
+#include <type_traits>
+
 #include "socket_common.h"
 
 namespace {
@@ -78,9 +80,9 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* qs = lds;
   float* ps = qs + G * D;
-  float* ts = ps + K * (D + 1);
-  float* red = ts + G * K;
-  float* protos_lds = lds + ((G * D + K * (D + 1) + G * K + kSHWaves * GC + 3) / 4) * 4;
+  float* ts = ps + ((K * (D + 1) + 3) / 4) * 4;   // (16-byte aligned when G * D is a multiple of 4: read as float4)
+  float* red = ts + ((G * K + 3) / 4) * 4;
+  float* protos_lds = lds + ((G * D + ((K * (D + 1) + 3) / 4) * 4 + ((G * K + 3) / 4) * 4 + kSHWaves * GC + 3) / 4) * 4;
   const int DP = D + 1;
   const int l = blockIdx.x, pair = blockIdx.y;
   const int b = pair / Hkv, kvh = pair % Hkv;
@@ -198,8 +200,31 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
       }
     };
     if constexpr (direct) {
+      // the G x K scaled projections as a handful of 16-byte broadcast reads instead
+      // of one LDS read per (head, plane) term
+      if ((G * D) % 4 == 0) {
+        constexpr int NV = (GC * (KC > 0 ? KC : 1) + 3) / 4;
+        float tv[NV * 4];
 #pragma unroll
-      for (int k = 0; k < KC; ++k) add_plane(k, pk[k]);
+        for (int i = 0; i < NV; ++i) {
+          const float4 t4 = (i * 4 < G * K) ? *reinterpret_cast<const float4*>(ts + i * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+          tv[4 * i] = t4.x, tv[4 * i + 1] = t4.y, tv[4 * i + 2] = t4.z, tv[4 * i + 3] = t4.w;
+        }
+#pragma unroll
+        for (int g = 0; g < GC; ++g) {
+          if (g < G) {
+#pragma unroll
+            for (int k = 0; k < KC; ++k) {
+              const float t = tv[g * KC + k];
+#pragma unroll
+              for (int i = 0; i < 4; ++i) lg[g][i] += t * pk[k][i];
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < KC; ++k) add_plane(k, pk[k]);
+      }
     } else {
       for (int k = 0; k < K; ++k) {
         float pr[4];
@@ -296,35 +321,48 @@ __global__ __launch_bounds__(kSHThreads) void soft_hash_kernel(
         }
       }
     } else {
-      // grouped layout [B*Hkv*parts, L, R, width]: the scorer's LDS image
-      for (int part = 0; part < parts; ++part) {
-        const int64_t o = ((((int64_t)pair * parts + part) * L + l) * R + r0) * width;
-        float v[16];  // [bucket][head of this part]: 4 * width consecutive elements of the table
+      // grouped layout [B*Hkv*parts, L, R, width]: the scorer's LDS image.  Width and
+      // part are compile-time in each instance below, so v[] is indexed statically
+      // (with a runtime width the compiler kept it in scratch memory).
+      auto write_part = [&](auto width_c, auto part_c) {
+        constexpr int W = decltype(width_c)::value, PART = decltype(part_c)::value;
+        if constexpr (PART * W < GC) {
+          const int64_t o = ((((int64_t)pair * parts + PART) * L + l) * R + r0) * W;
+          float v[4 * W];  // [bucket][head of this part]: 4 * W consecutive elements of the table
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+          for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int g = 0; g < GC; ++g) {
-            const int gg = g - part * width;
-            if (gg >= 0 && gg < width) v[i * width + gg] = lg[g][i];
-          }
-        if (out_dtype == SOCKET_F32) {
-          for (int c = 0; c < width; ++c)
-            *reinterpret_cast<float4*>((float*)out + o + 4 * c) = make_float4(v[4 * c], v[4 * c + 1], v[4 * c + 2], v[4 * c + 3]);
-        } else {
-          uint32_t w[8];
+            for (int gg = 0; gg < W; ++gg) v[i * W + gg] = lg[PART * W + gg][i];
+          if (out_dtype == SOCKET_F32) {
 #pragma unroll
-          for (int c = 0; c < 8; ++c)
-            w[c] = (uint32_t)f32_to_bf16_bits(v[2 * c]) | ((uint32_t)f32_to_bf16_bits(v[2 * c + 1]) << 16);
-          uint16_t* dst = (uint16_t*)out + o;
-          if (width == 4) {
-            *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
-            *reinterpret_cast<uint4*>(dst + 8) = make_uint4(w[4], w[5], w[6], w[7]);
-          } else if (width == 2) {
-            *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+            for (int c = 0; c < W; ++c)
+              *reinterpret_cast<float4*>((float*)out + o + 4 * c) =
+                  make_float4(v[4 * c], v[4 * c + 1], v[4 * c + 2], v[4 * c + 3]);
           } else {
-            *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
+            uint32_t w[2 * W];
+#pragma unroll
+            for (int c = 0; c < 2 * W; ++c)
+              w[c] = (uint32_t)f32_to_bf16_bits(v[2 * c]) | ((uint32_t)f32_to_bf16_bits(v[2 * c + 1]) << 16);
+            uint16_t* dst = (uint16_t*)out + o;
+            if constexpr (W == 4) {
+              *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+              *reinterpret_cast<uint4*>(dst + 8) = make_uint4(w[4], w[5], w[6], w[7]);
+            } else if constexpr (W == 2) {
+              *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+            } else {
+              *reinterpret_cast<uint2*>(dst) = make_uint2(w[0], w[1]);
+            }
           }
         }
+      };
+      using std::integral_constant;
+      if (width == 4) {
+        write_part(integral_constant<int, 4>{}, integral_constant<int, 0>{});
+        if (parts > 1) write_part(integral_constant<int, 4>{}, integral_constant<int, 1>{});
+      } else if (width == 2) {
+        write_part(integral_constant<int, 2>{}, integral_constant<int, 0>{});
+      } else {
+        write_part(integral_constant<int, 1>{}, integral_constant<int, 0>{});
       }
     }
   }
@@ -367,7 +405,8 @@ int soft_hash_entry(const void* q, int dtype, int64_t q_stride_b, int64_t q_stri
   const size_t protos_bytes = (size_t)K * R * sizeof(float);
   const int protos_in_lds = (!direct && protos_bytes <= 64 * 1024) ? 1 : 0;
   const int GC = G <= 4 ? 4 : 8;
-  const size_t head_floats = (((size_t)G * D + (size_t)K * (D + 1) + (size_t)G * K + kSHWaves * GC + 3) / 4) * 4;
+  const size_t head_floats = (((size_t)G * D + (((size_t)K * (D + 1) + 3) / 4) * 4 + (((size_t)G * K + 3) / 4) * 4 +
+                               kSHWaves * GC + 3) / 4) * 4;
   const size_t dyn_lds = head_floats * sizeof(float) + (protos_in_lds ? protos_bytes : 0);
 #define SOCKET_SH_LAUNCH(DT, GCV, KCV)                                                                     \
   do {                                                                                                     \
