@@ -373,7 +373,9 @@ __device__ __forceinline__ void score_tile(
 #pragma unroll
           for (int g = 0; g < GP; ++g) {
             const int i = tid + (k * GP + g) * THREADS;
-            if (i < nslots * GP) stage[k][g] = src[i];
+            // (unconditional assignment: an element left unwritten on one path made
+            // the compiler keep the whole array in scratch memory)
+            stage[k][g] = (i < nslots * GP) ? src[i] : make_uint4(0, 0, 0, 0);
           }
         return;
       }
