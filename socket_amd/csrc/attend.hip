@@ -582,7 +582,7 @@ __global__ __launch_bounds__(kAttThreads) void dense_mma_kernel(
   int b, s;
   if (flat) {
     if (wave == 0) {
-      const int n = lane < B ? (min(lens[lane], T) + rows_per_split - 1) / rows_per_split : 0;
+      const int n = lane < B ? (max(0, min(lens[lane], T)) + rows_per_split - 1) / rows_per_split : 0;
       int incl = n;
 #pragma unroll
       for (int d = 1; d < SOCKET_WAVE; d <<= 1) {

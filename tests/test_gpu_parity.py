@@ -480,6 +480,22 @@ def test_dense_decode_matrix_core_path(dev, dtype, B, Hq, Hkv, T, strided):
     assert (got2.cpu().double() - want2).abs().max() <= 2e-2
 
 
+def test_dense_decode_with_empty_sequences(dev):
+    """A sequence of length zero (or a negative length) takes no split; its
+    neighbours' splits are still numbered and attended correctly."""
+    g = torch.Generator().manual_seed(77)
+    B, Hq, Hkv, T = 5, 8, 2, 3000
+    q = torch.randn(B, Hq, 128, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, T, 128, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, T, 128, generator=g).to(torch.bfloat16)
+    lens = torch.tensor([0, 2500, -7, 1, 3000], dtype=torch.int32)
+    got = socket_kernels.dense_decode_fwd(q.to(dev), k.to(dev), v.to(dev), lens.to(dev)).cpu()
+    live = [1, 3, 4]
+    want = orc.dense_attend(q[live], k[live], v[live], lens[live])
+    assert (got[live].double() - want).abs().max() <= 2e-2
+    assert torch.isnan(got[[0, 2]].float()).all()        # nothing attended: 0 / 0, as the sparse path's empty list
+
+
 @pytest.mark.parametrize("draw", range(12))
 def test_dense_decode_random_shapes(dev, draw):
     """Drawn geometries for the MFMA dense kernel: 1 to 16 heads per kv head, 1 to 5
