@@ -346,7 +346,7 @@ __device__ __forceinline__ void score_tile(
     // workgroup has.  There it serves the direct copies and the double-buffered
     // register staging alike.)
     constexpr bool kFlat = GP > 1 && std::is_same<TT, TabBF16>::value;
-    constexpr int kPrefetch = kFlat ? (DMA ? (KT4 == 1 ? 8 : 4) : 3) : DMA ? 4 : 3;
+    constexpr int kPrefetch = kFlat ? (DMA ? (KT4 == 1 ? 8 : 4) : (KT4 == 2 && THREADS == 1024 ? 2 : 3)) : DMA ? 4 : 3;
     uint4 ring[kPrefetch][KT4];
 #pragma unroll
     for (int d = 0; d < kPrefetch; ++d)
