@@ -599,7 +599,7 @@ def main():
     globals()["SETTLE_MS"] = args.settle_ms
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every (sequence, kv head) "
-              "pair is independent; see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
+              "pair is independent, so the path shards over sequences or kv heads without exchange). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py needs a HIP device", file=sys.stderr)
@@ -729,7 +729,7 @@ def main():
             del s2
             torch.cuda.empty_cache()
         # the metric's second half: decode tokens per second at 128k context (prompt
-        # 130944 + 128 new tokens = the model's block_size), and configuration 4 as BASELINE
+        # 130944 + 128 new tokens = the model's block_size), and configuration 4 as its definition
         # states it (65536-token prompt, 256 greedy tokens)
         result["decode_tok_s"] = {"ctx_128k": decode_tok_s(dev, 131072 - 128, 128),
                                   "c4_prompt_65536": decode_tok_s(dev, 65536, 256)}

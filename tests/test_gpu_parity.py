@@ -795,7 +795,7 @@ def test_soft_hash_strided_queries_and_argument_checks(dev):
 # ---------------------------------------------------------------- whole step
 @pytest.mark.parametrize("name,T", [("c1", 4096), ("c2", 8192)])
 def test_decode_step_end_to_end(dev, name, T):
-    """hash -> score -> select -> attend on a BASELINE configuration (C2 with a
+    """hash -> score -> select -> attend on a benchmark configuration (C2 with a
     shorter context so the oracle finishes in seconds)."""
     w = scaled(WORKLOADS[name], T=T, M=min(WORKLOADS[name].M, T // 8))
     inp = make_inputs(w, device="cpu")
