@@ -142,11 +142,10 @@ __global__ __launch_bounds__(THREADS) void collision_i16_kernel(
       } else {
         load_partial(o, t0, sum);
       }
-      // the codes of kAhead tables are requested before the first of them is used:
-      // one 16-byte load in flight per lane leaves the stream waiting on latency
-      // A ring of kAhead code words per lane stays in flight: slot a always holds
-      // table lb + a (the loop is unrolled by the ring's depth, so a slot is a fixed
-      // set of registers and the wait before its use counts the loads behind it).
+      // A ring of kAhead code words per lane stays in flight (one 16-byte load per lane
+      // would leave the stream waiting on latency): slot a always holds table lb + a;
+      // the loop is unrolled by the ring's depth, so a slot is a fixed set of registers
+      // and the wait before its use counts exactly the loads behind it.
       uint4 ring[kAhead];
 #pragma unroll
       for (int a = 0; a < kAhead; ++a) ring[a] = codes_of(l0 + min(a, nt - 1), t0);
