@@ -111,7 +111,10 @@ def test_score_packed_collision_counts(dev):
 
 
 @pytest.mark.parametrize("L,R,T", [(32, 256, 777), (60, 1024, 4096), (3, 32768, 100), (60, 1024, 9000),
-                                   (17, 1024, 10001), (5, 8192, 2056), (40, 2048, 16384)])
+                                   (17, 1024, 10001), (5, 8192, 2056), (40, 2048, 16384),
+                                   # rows long enough for several tiles per workgroup under each table slice,
+                                   # one table per slice: the sums wait in the output between slices
+                                   (3, 32768, 1400000), (3, 32768, 1400001)])
 def test_reference_layout_scorer(dev, L, R, T):
     """Rows on and off the 16-byte grid, one to several table slices in LDS, more
     than one tile of tokens per row, codes outside [0, R) (they add nothing)."""
