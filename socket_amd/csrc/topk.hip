@@ -619,7 +619,11 @@ __global__ __launch_bounds__(kLocThreads) void select_local_kernel(
 // ---------------------------------------------------------------------------
 // rows
 // ---------------------------------------------------------------------------
-template <bool VEC>
+// REGPOOL: the pooled composites stay in registers, eight per lane, instead of in
+// LDS.  Possible whenever the slices have run: a row then either brings a compact
+// list of at most kPoolCap entries or is itself that short.  Without the 64 KB
+// pool the kernel needs 72 KB of LDS and two rows share a CU.
+template <bool VEC, bool REGPOOL>
 __global__ __launch_bounds__(kThreads) void select_list_kernel(
     const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
     const int32_t* __restrict__ budgets, const uint32_t* __restrict__ row_range, int range_parts,
@@ -631,8 +635,8 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   u64* buf = reinterpret_cast<u64*>(lds_raw);  // winners                  [cap_above]
   u64* cand = buf + cap_above;                 // entries of the k-th bin  [kCandCap]
-  u64* pool = cand + kCandCap;                 // pooled composites        [kPoolCap] if use_pool
-  u64* tmp = pool + (use_pool ? kPoolCap : 0); // counting placement       [2*cap_above] if counting_ok
+  u64* pool = cand + kCandCap;                 // pooled composites        [kPoolCap] if use_pool and not REGPOOL
+  u64* tmp = pool + ((use_pool && !REGPOOL) ? kPoolCap : 0);  // counting placement [2*cap_above] if counting_ok
 
   const int rowi = blockIdx.x;
   const int b = rowi / Hq;
@@ -659,19 +663,33 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     }
     int total = -1;  // uniform; stays -1 when no pool could be formed
     uint32_t kmin = 0xffffffffu, kmax = 0u;  // key range of what this lane pooled
+    constexpr int U = kPoolCap / kThreads;
+    u64 pv[REGPOOL ? U : 1];                 // REGPOOL: entry tid + u * kThreads of the pool
     if (n <= kPoolCap) {  // the whole row
-      for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
-        const uint32_t k = score_to_key(x);
-        kmin = min(kmin, k);
-        kmax = max(kmax, k);
-        pool[i] = composite(k, i);
-      });
+      if (REGPOOL) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = tid + u * kThreads;
+          const uint32_t k = score_to_key(i < n ? row[i] : 0.f);
+          if (i < n) {
+            kmin = min(kmin, k);
+            kmax = max(kmax, k);
+          }
+          pv[REGPOOL ? u : 0] = composite(k, i);
+        }
+      } else {
+        for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
+          const uint32_t k = score_to_key(x);
+          kmin = min(kmin, k);
+          kmax = max(kmax, k);
+          pool[i] = composite(k, i);
+        });
+      }
       total = n;
     } else if (loc) {  // what the slices found above the sampled threshold
       // The row's list is compact; its length and its entries are requested
       // together (entries past the length are stale and never used), so the
       // gather costs one memory latency.
-      constexpr int U = kPoolCap / kThreads;
       const u64* src = loc + (int64_t)rowi * kPoolCap;
       const int sum = row_count[rowi];
       u64 v[U];
@@ -684,11 +702,12 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
             const uint32_t k = (uint32_t)(v[u] >> 32);
             kmin = min(kmin, k);
             kmax = max(kmax, k);
-            pool[tid + u * kThreads] = v[u];
+            if (REGPOOL) pv[REGPOOL ? u : 0] = v[u];
+            else pool[tid + u * kThreads] = v[u];
           }
         total = sum;
       }
-    } else if (sampling_ok(m)) {  // one workgroup: threshold from the sample, one pass
+    } else if (!REGPOOL && sampling_ok(m)) {  // one workgroup: threshold from the sample, one pass
       const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
       for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
         const uint32_t k = score_to_key(x);
@@ -733,9 +752,17 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         const int shift = range_shift(lo, hi);
         for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
         __syncthreads();
-        for (int i = tid; i < total; i += kThreads) {
-          const u64 v = pool[i];
-          if (v >= lo && v <= hi) atomicAdd(&hist[(int)((v - lo) >> shift)], 1u);
+        if (REGPOOL) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const u64 v = pv[REGPOOL ? u : 0];
+            if (tid + u * kThreads < total && v >= lo && v <= hi) atomicAdd(&hist[(int)((v - lo) >> shift)], 1u);
+          }
+        } else {
+          for (int i = tid; i < total; i += kThreads) {
+            const u64 v = pool[i];
+            if (v >= lo && v <= hi) atomicAdd(&hist[(int)((v - lo) >> shift)], 1u);
+          }
         }
         __syncthreads();
         find_bin<kThreads>(hist, need_in, 1, sh, tid);
@@ -752,10 +779,20 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
       }
       const u64 blo = sh.lo, bhi = sh.hi;
       const int need = sh.need;
-      for (int i = tid; i < total; i += kThreads) {
-        const u64 v = pool[i];
-        wave_append(v > bhi, v, &sh.fill_above, buf, cap_above);
-        wave_append(v >= blo && v <= bhi, v, &sh.fill_cand, cand, kCandCap);
+      if (REGPOOL) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const u64 v = pv[REGPOOL ? u : 0];
+          const bool have = tid + u * kThreads < total;
+          wave_append(have && v > bhi, v, &sh.fill_above, buf, cap_above);
+          wave_append(have && v >= blo && v <= bhi, v, &sh.fill_cand, cand, kCandCap);
+        }
+      } else {
+        for (int i = tid; i < total; i += kThreads) {
+          const u64 v = pool[i];
+          wave_append(v > bhi, v, &sh.fill_above, buf, cap_above);
+          wave_append(v >= blo && v <= bhi, v, &sh.fill_cand, cand, kCandCap);
+        }
       }
       __syncthreads();
       order_and_write(buf, m - need, cand, min(sh.fill_cand, kCandCap), need, lo0, shift0, tmp, hist, sh,
@@ -961,8 +998,15 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
 
   // extras as LDS allows: the pool (where a pooled select can apply at all), then
   // counting placement (2 * cap_above more slots)
+  // With slices the pool lives in registers (a row brings at most kPoolCap entries or
+  // is that short itself) and costs no LDS.
   int use_pool = 0, counting_ok = 0;
-  if ((T <= kPoolCap || sampling_ok(m_max)) && lds + (size_t)kPoolCap * sizeof(u64) + lds_static <= lds_max) {
+  int S = 0;
+  const bool pool_applies = T <= kPoolCap || sampling_ok(m_max);
+  const bool slices = workspace && pool_applies && use_slices(T, m_max, &S);
+  if (slices) {
+    use_pool = 1;
+  } else if (pool_applies && lds + (size_t)kPoolCap * sizeof(u64) + lds_static <= lds_max) {
     use_pool = 1;
     lds += (size_t)kPoolCap * sizeof(u64);
   }
@@ -970,8 +1014,6 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
     counting_ok = 1;
     lds += (size_t)2 * cap_above * sizeof(u64);
   }
-  int S = 0;
-  const bool slices = workspace && use_pool && use_slices(T, m_max, &S);
 
   const u64* loc = nullptr;
   const int32_t* loc_count = nullptr;
@@ -1000,7 +1042,8 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
     loc_count = count_w;
   }
 
-  auto kern = vec ? select_list_kernel<true> : select_list_kernel<false>;
+  auto kern = slices ? (vec ? select_list_kernel<true, true> : select_list_kernel<false, true>)
+                     : (vec ? select_list_kernel<true, false> : select_list_kernel<false, false>);
   if (lds > 32 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
