@@ -371,6 +371,28 @@ int socket_rope_append(const void* qkv, int dtype, int64_t qkv_stride_b, const v
                        int64_t cache_stride_s, int32_t* lens, void* k_new, void* v_new, int B, int Hq, int Hkv,
                        int D, int64_t Tcap, void* stream);
 
+/* The head of a single-token decode step in ONE launch: what socket_rope_append,
+ * socket_hash_keys on the new key and socket_soft_hash (out_dtype / grouped as
+ * socket_soft_hash_grouped when grouped != 0) do in three, with the same results bit
+ * for bit -- rotary embedding of the new token's q and k from the fused projection
+ * qkv [B, (Hq + 2*Hkv) * D], K/V rows written at pos, lens[b] = pos + 1, packed
+ * codes and value norm of the new key written at pos (planes_words as for
+ * socket_hash_keys, P = K), q_out [B,Hq,D], and the rotated queries' bucket
+ * probabilities in q_table ([B,Hq,L,R], or the grouped layout).  Arguments as in
+ * those three entry points.  Written for dtype = SOCKET_BF16, D = 128, K = 10,
+ * R <= 1024, Hq / Hkv <= 8, 16-byte aligned operands and strides that are
+ * multiples of 8 elements: anything else returns SOCKET_ERR_UNSUPPORTED /
+ * SOCKET_ERR_ALIGN and the caller uses the three entry points.
+ * Replaces GPT-FAST/model.py:433-451 (rotary, KVCache.update, hard_hash_keys of
+ * the new key, value norm) and :392-401 (soft_hash) for one new token. */
+int socket_decode_prologue(const void* qkv, int dtype, int64_t qkv_stride_b, const void* freqs_cis,
+                           int freqs_dtype, int64_t n_pos, const int64_t* pos, int pos_stride, void* q_out,
+                           void* k_cache, void* v_cache, int64_t cache_stride_b, int64_t cache_stride_h,
+                           int64_t cache_stride_s, int32_t* lens, const void* planes_words, void* codes,
+                           void* v_norm, const void* planes, const void* protos_T, void* q_table, int out_dtype,
+                           int grouped, int B, int Hq, int Hkv, int D, int L, int K, int R, int64_t Tcap,
+                           float tanh_scale, float inv_temperature, void* stream);
+
 /* h = x + residual (residual may be NULL: h = x), rounded to `dtype`;
  * y = round(h * rsqrt(mean(h^2) + eps)) * weight.  x, residual, h_out (may be
  * NULL), y_out: [rows, dim] contiguous; weight [dim].

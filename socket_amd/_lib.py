@@ -61,6 +61,8 @@ SIGNATURES = {
     "socket_select_list": (_I, [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _P, _Z, _P]),
     "socket_rope_append": (_I, [_P, _I, _L, _P, _I, _L, _P, _I, _P, _P, _P, _L, _L, _L, _P, _P, _P, _I, _I, _I, _I,
                                 _L, _P]),
+    "socket_decode_prologue": (_I, [_P, _I, _L, _P, _I, _L, _P, _I, _P, _P, _P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _P,
+                                    _I, _I, _I, _I, _I, _I, _I, _I, _I, _L, c_float, c_float, _P]),
     "socket_add_rmsnorm": (_I, [_P, _P, _P, _P, _P, _I, _L, _I, c_float, _P]),
     "socket_silu_mul": (_I, [_P, _P, _P, _I, _L, _P]),
     "socket_gemv_bf16": (_I, [_P, _L, _P, _P, _P, _L, _I, _I, _I, _P]),

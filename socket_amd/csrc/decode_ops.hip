@@ -63,16 +63,6 @@ __device__ __forceinline__ void store16<DType_f16>(void* base, int64_t idx, cons
   *reinterpret_cast<uint4*>((uint16_t*)base + idx) = w;
 }
 
-// (x0 + i x1) * (c + i s) with separately rounded products, as the reference's
-// elementwise multiplies, subtraction and addition round: no contraction into
-// fused multiply-adds here.
-__device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s, float& re, float& im) {
-#pragma clang fp contract(off)
-  const float a = x0 * c, b = x1 * s, cc = x1 * c, d = x0 * s;
-  re = a - b;
-  im = cc + d;
-}
-
 // One workgroup per (head of the fused projection, sequence); lane i owns the
 // pair (2i, 2i+1).  Heads [0,Hq) are queries, [Hq,Hq+Hkv) keys, the rest values.
 template <class DT, class FT>

@@ -121,6 +121,16 @@ __device__ __forceinline__ void store_elem<DType_f16>(void* base, int64_t idx, f
   ((uint16_t*)base)[idx] = f32_to_f16_bits(v);
 }
 
+// (x0 + i x1) * (c + i s) with separately rounded products, as the reference's
+// elementwise multiplies, subtraction and addition round (apply_rotary_emb,
+// GPT-FAST/model.py:626-639): no contraction into fused multiply-adds here.
+__device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s, float& re, float& im) {
+#pragma clang fp contract(off)
+  const float a = x0 * c, b = x1 * s, cc = x1 * c, d = x0 * s;
+  re = a - b;
+  im = cc + d;
+}
+
 // 16 bytes per lane from global memory straight into LDS: lane i's bytes land at
 // lds_dst + 16 * i (lds_dst is the same for the whole wave).  Written as assembly
 // so that the compiler does not serialise later LDS reads behind it; M0, which

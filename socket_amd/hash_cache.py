@@ -219,6 +219,61 @@ def soft_hash(queries_bhd: torch.Tensor, planes_lkd: torch.Tensor, protos_T: tor
     return out
 
 
+def decode_prologue_fits(qkv: torch.Tensor, head_dim: int, K: int, R: int, n_heads: int, n_kv_heads: int) -> bool:
+    """Whether `decode_prologue` takes these operands (else: rope_append, hash_keys_into
+    and soft_hash, three launches with the same results)."""
+    return (qkv.is_cuda and qkv.dtype == torch.bfloat16 and head_dim == HASH_DIM and K == 10 and R % 4 == 0 and
+            4 <= R <= 1024 and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 8)
+
+
+@torch.no_grad()
+def decode_prologue(qkv: torch.Tensor, freqs_cis: torch.Tensor, input_pos: torch.Tensor, k_cache: torch.Tensor,
+                    v_cache: torch.Tensor, lens: Optional[torch.Tensor], planes_words: torch.Tensor,
+                    codes: torch.Tensor, v_norm: torch.Tensor, planes_lkd: torch.Tensor, protos_T: torch.Tensor,
+                    n_heads: int, n_kv_heads: int, temperature: float = 1.0, grouped: bool = False):
+    """The head of a single-token decode step in one launch: rotary embedding of the
+    new q and k (from the fused projection qkv [B,(Hq+2Hkv)*D]), K/V append at
+    input_pos, `lens` raised, hash + value norm of the new key into `codes` /
+    `v_norm`, and the soft hash of the rotated queries (GPT-FAST/model.py:433-451 and
+    :392-401).  Returns (q [B,Hq,D], q_probs in the reference's or the grouped
+    layout).  Same results as decode_ops.rope_append + hash_keys_into + soft_hash."""
+    B = qkv.shape[0]
+    q2 = qkv.reshape(B, -1)
+    D = k_cache.shape[-1]
+    L, K, D2 = planes_lkd.shape
+    K2, R = protos_T.shape
+    assert decode_prologue_fits(q2, D, K, R, n_heads, n_kv_heads) and D2 == D and K2 == K
+    assert q2.stride(-1) == 1 and q2.shape[1] == (n_heads + 2 * n_kv_heads) * D
+    assert k_cache.shape == v_cache.shape and k_cache.stride() == v_cache.stride() and k_cache.stride(-1) == 1
+    assert k_cache.dtype == q2.dtype and k_cache.shape[0] == B and k_cache.shape[1] == n_kv_heads
+    assert input_pos.dtype == torch.int64 and input_pos.is_cuda and input_pos.numel() in (1, B)
+    assert freqs_cis.is_contiguous() and freqs_cis.shape[1:] == (D // 2, 2)
+    Tcap = k_cache.shape[2]
+    NW = words_per_key(L, K)
+    assert codes.dtype == torch.int32 and codes.is_contiguous() and tuple(codes.shape) == (B, n_kv_heads, NW, Tcap)
+    assert v_norm.dtype == torch.float16 and v_norm.is_contiguous() and tuple(v_norm.shape) == (B, n_kv_heads, Tcap)
+    assert planes_words.dtype == torch.bfloat16 and planes_words.is_contiguous()
+    assert tuple(planes_words.shape) == (NW * 32, HASH_DIM)
+    if lens is not None:
+        assert lens.dtype == torch.int32 and lens.numel() == B
+    planes_lkd = planes_lkd.to(q2.dtype).contiguous()
+    protos_T = protos_T.to(q2.dtype).contiguous()
+    q_out = torch.empty((B, n_heads, D), dtype=q2.dtype, device=q2.device)
+    if grouped:
+        parts, width = group_shape(n_heads, n_kv_heads)
+        table = torch.empty((B, n_kv_heads * parts, L, R, width), dtype=q2.dtype, device=q2.device)
+    else:
+        table = torch.empty((B, n_heads, L, R), dtype=q2.dtype, device=q2.device)
+    check("socket_decode_prologue", lib().socket_decode_prologue(
+        ptr(q2), dtype_enum(q2.dtype), q2.stride(0), ptr(freqs_cis), dtype_enum(freqs_cis.dtype), freqs_cis.shape[0],
+        ptr(input_pos), 0 if input_pos.numel() == 1 else 1, ptr(q_out), ptr(k_cache), ptr(v_cache),
+        k_cache.stride(0), k_cache.stride(1), k_cache.stride(2), ptr(lens), ptr(planes_words), ptr(codes),
+        ptr(v_norm), ptr(planes_lkd), ptr(protos_T), ptr(table), dtype_enum(q2.dtype), int(bool(grouped)), B,
+        n_heads, n_kv_heads, D, L, K, R, Tcap, 1.0 / max(math.sqrt(D), 1e-6), 1.0 / float(temperature),
+        stream_ptr(q2.device)))
+    return q_out, table
+
+
 @torch.no_grad()
 def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
                  lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,

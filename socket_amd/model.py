@@ -211,6 +211,22 @@ def _soft_hash(q_bhd: Tensor, planes: Tensor, protos_T: Tensor, n_kv_heads: int,
     return hash_cache.soft_hash(q_bhd, planes, protos_T, 1.0, n_kv_heads, grouped=grouped)
 
 
+def _decode_prologue(qkv: Tensor, freqs_table: Tensor, input_pos: Tensor, cache: KVCache, planes: Tensor,
+                     protos_T: Tensor, n_heads: int, n_kv_heads: int):
+    """Rotary + append + hash of the new key + soft hash of the new query in one
+    launch; None when the shapes are not the ones that launch is written for."""
+    D = cache.k_cache.size(-1)
+    if cache.planes_words is None or not hash_cache.decode_prologue_fits(qkv, D, cache.K, protos_T.shape[1], n_heads,
+                                                                         n_kv_heads):
+        return None
+    T = cache.k_cache.size(2)
+    grouped = hash_cache._prefers_grouped(qkv.shape[0], n_heads, n_kv_heads, T, hash_cache.dtype_enum(qkv.dtype),
+                                          cache.L, cache.K, int(protos_T.shape[1]))
+    return hash_cache.decode_prologue(qkv, freqs_table, input_pos, cache.k_cache, cache.v_cache, cache.lens,
+                                      cache.planes_words, cache.codes, cache.v_norm, planes, protos_T, n_heads,
+                                      n_kv_heads, grouped=grouped)
+
+
 def _planes_to_words(planes: Tensor) -> Tensor:
     return hash_cache.permute_planes(planes)
 
@@ -449,12 +465,17 @@ class Attention(nn.Module):
         cache = self.kv_cache
         qkv = decode_ops.linear_rows(x, self.wqkv.weight)
         if sparse:
-            q_bhd, k_new, v_new = decode_ops.rope_append(qkv, step.freqs_table, input_pos, cache.k_cache,
-                                                         cache.v_cache, cache.lens, self.n_head,
-                                                         self.n_local_heads, return_new=True)
-            _hash_rows(cache, k_new, v_new, pos_b=step.pos_b)
             cfg = self.config
-            q_probs = _soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, cache.k_cache.size(2))
+            fused = _decode_prologue(qkv, step.freqs_table, input_pos, cache, self.planes, self.protos_T,
+                                     self.n_head, self.n_local_heads)
+            if fused is not None:
+                q_bhd, q_probs = fused
+            else:
+                q_bhd, k_new, v_new = decode_ops.rope_append(qkv, step.freqs_table, input_pos, cache.k_cache,
+                                                             cache.v_cache, cache.lens, self.n_head,
+                                                             self.n_local_heads, return_new=True)
+                _hash_rows(cache, k_new, v_new, pos_b=step.pos_b)
+                q_probs = _soft_hash(q_bhd, self.planes, self.protos_T, self.n_local_heads, cache.k_cache.size(2))
             out_bhd = _sparse_step(q_bhd, q_probs, cache, cache.k_cache.size(2), int(cfg.sink_size),
                                    int(cfg.window_size), int(self.heavy_const))
         else:

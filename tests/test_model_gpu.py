@@ -263,6 +263,62 @@ def test_rope_append_equals_the_torch_chain(dev, dtype):
     assert lens.tolist() == [3, 0, 10] and not kc[1].any() and kc[0, :, 2].any() and kc[2, :, 9].any()
 
 
+@pytest.mark.parametrize("Hq,Hkv,L,grouped,ftype", [(32, 8, 60, True, torch.bfloat16), (32, 8, 60, False, torch.float32),
+                                                    (28, 4, 48, True, torch.bfloat16), (8, 8, 7, False, torch.bfloat16),
+                                                    (16, 8, 33, True, torch.float32)])
+def test_decode_prologue_equals_the_three_launches(dev, Hq, Hkv, L, grouped, ftype):
+    """rope_append + hash of the new key + soft hash in one launch: every output
+    bit for bit what the three launches leave (queries, K/V rows, lengths, packed
+    codes, value norms, the probability table in either layout), rows elsewhere in
+    the cache untouched, and positions outside the cache or the rotary table
+    handled as the three launches handle them."""
+    from socket_amd import decode_ops, hash_cache
+    g = torch.Generator().manual_seed(100 + Hq + L)
+    B, D, K, R, Tcap, n_pos = 4, 128, 10, 1024, 72, 70
+    dt = torch.bfloat16
+    qkv = (torch.randn(B, 1, (Hq + 2 * Hkv) * D, generator=g) * 2).to(dt).to(dev)
+    table = M.precompute_freqs_cis(n_pos, D, 10000).to(ftype).to(dev)
+    planes = (torch.randn(L, K, D, generator=g) * 0.3).to(dt).to(dev)
+    protos_T = torch.randn(K, R, generator=g).to(dt).to(dev)
+    words = hash_cache.permute_planes(planes)
+    NW = hash_cache.words_per_key(L, K)
+
+    def fresh():
+        gg = torch.Generator().manual_seed(5)
+        kc = torch.randn(B, Hkv, Tcap, D, generator=gg).to(dt).to(dev)
+        vc = torch.randn(B, Hkv, Tcap, D, generator=gg).to(dt).to(dev)
+        codes = torch.randint(0, 2 ** 31 - 1, (B, Hkv, NW, Tcap), generator=gg, dtype=torch.int32).to(dev)
+        vn = torch.rand(B, Hkv, Tcap, generator=gg).to(torch.float16).to(dev)
+        lens = torch.tensor([3, 10, 70, 1], dtype=torch.int32, device=dev)
+        return kc, vc, codes, vn, lens
+
+    # one position for all; one each, with one beyond the cache (72) and one inside the
+    # cache but beyond the rotary table (70, 71)
+    for ip in (torch.tensor([17], device=dev), torch.tensor([0, 69, 72, 71], device=dev),
+               torch.tensor([5, -1, 33, 70], device=dev)):
+        a, b = fresh(), fresh()
+        q_a, kn, vn_new = decode_ops.rope_append(qkv, table, ip, a[0], a[1], a[4], Hq, Hkv, return_new=True)
+        hash_cache.hash_keys_into(kn, vn_new, words, a[2], a[3], L, K, pos_b=ip.to(torch.int32).expand(B).contiguous(),
+                                  layout="bshd")
+        t_a = hash_cache.soft_hash(q_a, planes, protos_T, 1.0, Hkv, grouped=grouped)
+        q_b, t_b = hash_cache.decode_prologue(qkv, table, ip, b[0], b[1], b[4], words, b[2], b[3], planes, protos_T,
+                                              Hq, Hkv, grouped=grouped)
+        assert torch.equal(q_a, q_b), ip.tolist()
+        assert t_a.shape == t_b.shape and torch.equal(t_a, t_b), ip.tolist()
+        for x, y, name in zip(a, b, ("k_cache", "v_cache", "codes", "v_norm", "lens")):
+            assert torch.equal(x, y), (name, ip.tolist())
+    # and the new key's codes are the hard hash of the rotated key (GPT-FAST/model.py:403-413)
+    ip = torch.tensor([9], device=dev)
+    kc, vc, codes, vn, lens = fresh()
+    hash_cache.decode_prologue(qkv, table, ip, kc, vc, lens, words, codes, vn, planes, protos_T, Hq, Hkv)
+    got = hash_cache.unpack_codes(codes, L, K, 9, 1, layout="bhlt")[..., 0].cpu()          # [B,Hkv,L]
+    proj = torch.einsum("bhd,lkd->bhlk", kc[:, :, 9].double().cpu(), planes.double().cpu())
+    want = ((proj >= 0).long() * (1 << torch.arange(K - 1, -1, -1))).sum(-1)
+    decided = proj.abs().min(-1).values > 1e-3
+    assert torch.equal(got.long()[decided], want[decided]) and float(decided.float().mean()) > 0.9
+    assert torch.allclose(vn[:, :, 9].float().cpu(), vc[:, :, 9].float().norm(dim=-1).cpu(), rtol=1e-3)
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 1e-2), (torch.float32, 1e-6)])
 def test_add_rmsnorm_and_silu_mul_equal_the_torch_chain(dev, dtype, tol):
     from socket_amd import decode_ops
