@@ -708,15 +708,98 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         total = sum;
       }
     } else if (!REGPOOL && sampling_ok(m)) {  // one workgroup: threshold from the sample, one pass
-      const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
-      for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
-        const uint32_t k = score_to_key(x);
-        if (k >= tau) {
+      if (VEC) {
+        // The row in batches of 16 scores per lane (four 16-byte loads, all in
+        // flight together); the first two batches are requested before the threshold is
+        // worked out, each further one two batches ahead of the one being filtered.  A wave
+        // counts what passes in its batch, reserves a stretch of the pool with one
+        // LDS atomic and writes its entries there: no barrier in the loop.
+        constexpr int kLoads = 4, kStep = kThreads * 4 * kLoads;
+        const int n4 = n & ~3;
+        auto fetch = [&](int base, float4 (&x)[kLoads]) {
+#pragma unroll
+          for (int u = 0; u < kLoads; ++u) {
+            // (past the end: the row's last four, fetched and ignored -- a load under a
+            // condition would make every wait in the loop a wait for all loads)
+            const int i0 = min(base + (u * kThreads + tid) * 4, n4 - 4);
+            x[u] = *reinterpret_cast<const float4*>(row + i0);
+          }
+        };
+        // What passes in one batch of one lane, as a bit per score.  The test is made
+        // on the floats (one compare per score; keys only for the pool): x passes
+        // when it is not below the float whose key is tau.  A tau above +inf's key or
+        // below -inf's is no float's key and is widened to that infinity (the pool
+        // only has to hold everything at or above tau; more is allowed).
+        auto filter = [&](int base, const float4 (&x)[kLoads], float tau_f) {
+          if (base >= n4) return;  // uniform
+          uint32_t taken = 0;      // bit u * 4 + c: score c of load u passes
+#pragma unroll
+          for (int u = 0; u < kLoads; ++u) {
+            const float xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+            const bool in = base + (u * kThreads + tid) * 4 < n4;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) taken |= (in && !(xs[c] < tau_f)) ? (1u << (u * 4 + c)) : 0u;
+          }
+          const int cnt = __popc(taken);
+          const int incl = wave_incl_scan(cnt, lane);
+          int at = 0;
+          if (lane == 63 && incl) at = atomicAdd(&sh.fill_pool, incl);
+          at = __shfl(at, 63, SOCKET_WAVE) + incl - cnt;
+          if (taken) {
+#pragma unroll
+            for (int u = 0; u < kLoads; ++u) {
+              const float xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+#pragma unroll
+              for (int c = 0; c < 4; ++c) {
+                if (taken & (1u << (u * 4 + c))) {   // (the score as it is: keys are made afterwards)
+                  if (at < kPoolCap) pool[at] = composite(__float_as_uint(xs[c]), base + (u * kThreads + tid) * 4 + c);
+                  ++at;
+                }
+              }
+            }
+          }
+        };
+        float4 b0[kLoads], b1[kLoads], b2[kLoads];
+        fetch(0, b0);
+        fetch(kStep, b1);
+        const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
+        const float tau_f = tau >= 0xff800000u ? INFINITY : tau <= 0x007fffffu ? -INFINITY
+                            : __uint_as_float((tau & 0x80000000u) ? (tau & 0x7fffffffu) : ~tau);
+        for (int base = 0; base < n4; base += 3 * kStep) {
+          fetch(base + 2 * kStep, b2);
+          filter(base, b0, tau_f);
+          fetch(base + 3 * kStep, b0);
+          filter(base + kStep, b1, tau_f);
+          fetch(base + 4 * kStep, b1);
+          filter(base + 2 * kStep, b2, tau_f);
+        }
+        // the last one to three scores of a row whose length is no multiple of four
+        if (wave == 0) {
+          const int i = n4 + lane;
+          const float x = i < n ? row[i] : 0.f;
+          wave_append(i < n && !(x < tau_f), composite(__float_as_uint(x), i), &sh.fill_pool, pool, kPoolCap);
+        }
+        __syncthreads();
+        // the pooled scores become keys, eight entries a lane at most
+        const int got = min(sh.fill_pool, kPoolCap);
+        for (int i = tid; i < got; i += kThreads) {
+          const u64 e = pool[i];
+          const uint32_t k = score_to_key(__uint_as_float((uint32_t)(e >> 32)));
           kmin = min(kmin, k);
           kmax = max(kmax, k);
+          pool[i] = ((u64)k << 32) | (e & 0xffffffffull);
         }
-        wave_append(k >= tau, composite(k, i), &sh.fill_pool, pool, kPoolCap);
-      });
+      } else {
+        const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
+        for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
+          const uint32_t k = score_to_key(x);
+          if (k >= tau) {
+            kmin = min(kmin, k);
+            kmax = max(kmax, k);
+          }
+          wave_append(k >= tau, composite(k, i), &sh.fill_pool, pool, kPoolCap);
+        });
+      }
       __syncthreads();
       const int got = sh.fill_pool;
       if (got >= m && got <= kPoolCap) total = got;
@@ -936,12 +1019,17 @@ int next_pow2(int x) {
   return p;
 }
 
-// Slices pay off once a row is several of them long; otherwise one workgroup per
-// row does everything.
-bool use_slices(int T, int m_max, int* S_out) {
+// One workgroup per row does everything (threshold from the sample, one streaming
+// pass, select) in about 19 + 1.47 us per slice length of its row; with slices the
+// three launches cost about 27.5 us + 3.2 us per (rows x slices / CU).  Slices
+// therefore pay off for few, long rows only (measured on 256 CUs, top-k 2048:
+// 32 rows from 131072 scores up, 64 rows from about 200000, 128 rows never).
+bool use_slices(int rows, int T, int m_max, int* S_out) {
   const int S = (T + kSliceLen - 1) / kSliceLen;
   *S_out = S;
-  return S >= 4 && S <= kMaxSlices && m_max > 0 && sampling_ok(m_max);
+  if (!(S >= 4 && S <= kMaxSlices && m_max > 0 && sampling_ok(m_max))) return false;
+  const float cus = (float)socket_device_limits().cu_count;
+  return (float)S * (1.467f - 3.2f * (float)rows / cus) > 8.2f;
 }
 
 struct SplitLayout {
@@ -969,7 +1057,7 @@ SplitLayout split_layout(int rows) {
 extern "C" size_t socket_select_workspace_bytes(int B, int Hq, int T, int M) {
   if (B <= 0 || Hq <= 0 || T <= 0 || M < 0) return 0;
   int S = 0;
-  if (!use_slices(T, M < T ? M : T, &S)) return 0;
+  if (!use_slices(B * Hq, T, M < T ? M : T, &S)) return 0;
   return split_layout(B * Hq).total;
 }
 
@@ -1003,7 +1091,7 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
   int use_pool = 0, counting_ok = 0;
   int S = 0;
   const bool pool_applies = T <= kPoolCap || sampling_ok(m_max);
-  const bool slices = workspace && pool_applies && use_slices(T, m_max, &S);
+  const bool slices = workspace && pool_applies && use_slices(rows, T, m_max, &S);
   if (slices) {
     use_pool = 1;
   } else if (pool_applies && lds + (size_t)kPoolCap * sizeof(u64) + lds_static <= lds_max) {

@@ -250,7 +250,7 @@ def test_select_random_scores(dev, T, M):
     _check_select(scores, 4, 64, M, dev)
 
 
-@pytest.mark.parametrize("T", [20000, 70001])
+@pytest.mark.parametrize("T", [20000, 70001, 140001])
 def test_select_ties_and_special_values(dev, T):
     g = torch.Generator().manual_seed(3)
     s = torch.randint(0, 50, (1, 6, T), generator=g).float()     # heavy ties, few distinct values
