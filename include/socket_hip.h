@@ -240,11 +240,18 @@ int socket_soft_hash_grouped(const void* q, int dtype, int64_t q_stride_b, int64
  * these scores, or NULL / 0 (then the kernel finds a row's range itself when it
  * needs it).
  * workspace: optional scratch of socket_select_workspace_bytes(B, Hq, T, M) bytes
- * (0 for short rows).  With it, long rows are first filtered slice by slice by
- * many workgroups; without it (NULL) one workgroup handles a whole row.  Same result.
+ * (0 where it would not help: short rows, or as many rows as the GPU has CUs).
+ * With it, a few long rows are each shared between several workgroups that
+ * exchange their candidates through it, in the same launch; without it (NULL) one
+ * workgroup handles a whole row.  Same result.  Its first
+ * socket_select_workspace_zero_bytes(B, Hq, T, M) bytes are arrival counters that
+ * must be zero when the call starts and are zero again when it has finished: zero
+ * them once, then the workspace can serve every later call of the same shape
+ * issued in order on one stream (calls that overlap on one workspace race).
  * Requires M <= SOCKET_TOPK_MAX_M, B*Hq <= 65535. */
 #define SOCKET_TOPK_MAX_M 16384
 size_t socket_select_workspace_bytes(int B, int Hq, int T, int M);
+size_t socket_select_workspace_zero_bytes(int B, int Hq, int T, int M);
 int socket_select_list(const float* scores, int64_t score_stride, const int32_t* lens,
                        const int32_t* budgets, const uint32_t* row_range, int range_parts,
                        int B, int Hq, int T, int M, int sink, int window, int write_base,

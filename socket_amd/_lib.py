@@ -58,6 +58,7 @@ SIGNATURES = {
     "socket_soft_hash_grouped": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),
     "socket_soft_hash": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),
     "socket_select_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "socket_select_workspace_zero_bytes": (_Z, [_I, _I, _I, _I]),
     "socket_select_list": (_I, [_P, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _L, _I, _P, _P, _Z, _P]),
     "socket_rope_append": (_I, [_P, _I, _L, _P, _I, _L, _P, _I, _P, _P, _P, _L, _L, _L, _P, _P, _P, _I, _I, _I, _I,
                                 _L, _P]),

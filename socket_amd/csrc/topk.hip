@@ -7,22 +7,21 @@
 // composite" is exactly "higher score, then lower index" and all composites of a
 // row are distinct.
 //
-// select_list_kernel, one workgroup (1024 lanes) per row, selects in two ways:
+// select_list_kernel, workgroups of 1024 lanes, selects in two ways:
 //  * pooled: a superset of the row's m winners, at most kPoolCap composites, is
-//    put into LDS and the m-th largest located there by range refinement -- a
-//    2048-bin LDS histogram over [lo, hi] (initially the pool's min / max, so the
-//    bins spread over the values that occur and LDS atomics rarely collide), then
-//    the bin holding the m-th becomes the new range, until it holds at most
-//    kCandCap entries.  Because the composites are distinct, ties need no special
-//    case.  The pool is the whole row when that fits; otherwise everything at or
-//    above a threshold estimated from a fixed sample of the row and aimed at
-//    about 2m entries.  For long rows select_tau_kernel finds the thresholds (one
-//    workgroup per row, only the sample is read) and select_local_kernel applies
-//    them, one 256-lane workgroup per slice of 16384 scores held in registers
-//    (one HBM read of the scores in all) and appending what passes to the row's
-//    list, in a stretch reserved with one atomic add; the row kernel reads that
-//    one compact list.  A pool that comes out shorter than m or longer
-//    than kPoolCap (the sample misjudged the row, or one key value is massively
+//    formed and the m-th largest located in it by range refinement -- a 2048-bin
+//    LDS histogram over [lo, hi] (initially the pool's min / max, so the bins
+//    spread over the values that occur and LDS atomics rarely collide), then the
+//    bin holding the m-th becomes the new range, until it holds at most kCandCap
+//    entries.  Because the composites are distinct, ties need no special case.
+//    The pool is the whole row when that fits; otherwise everything at or above a
+//    threshold estimated from a fixed sample of the row and aimed at about 2m
+//    entries, found in one streaming pass over the row (compacted in LDS, then
+//    held in registers).  Where CUs are to spare several workgroups share a row:
+//    each streams its share against the same threshold and appends what passes
+//    to the row's list in memory, and the last to arrive selects from that list,
+//    in the same launch.  A pool that comes out shorter than m or longer than
+//    kPoolCap (the sample misjudged the row, or one key value is massively
 //    repeated) is dropped and the row redone from scratch: the result is always
 //    exact, only the time differs.
 //  * from scratch: the same refinement over the row itself, one pass per level
@@ -47,12 +46,9 @@ constexpr int kBins = 2048;
 constexpr int kCandCap = 2048;           // entries of the k-th bin kept in LDS
 constexpr int kMaxBinForCounting = 128;  // larger bins are sorted, not rank-counted
 
-constexpr int kSliceLen = 16384;  // scores per select_local_kernel workgroup
-constexpr int kLocThreads = 256;
-constexpr int kLocWaves = kLocThreads / SOCKET_WAVE;
-constexpr int kLocPerLane = kSliceLen / kLocThreads;  // 64 keys in registers
-constexpr int kPoolCap = 8192;    // composites pooled per row in LDS
-constexpr int kMaxSlices = 64;
+constexpr int kBatch = kThreads * 16;  // scores a workgroup filters per batch (16 per lane)
+constexpr int kPoolCap = 8192;         // composites pooled per row
+constexpr int kMaxParts = 16;          // workgroups that share one row at most
 
 typedef unsigned long long u64;
 
@@ -68,6 +64,8 @@ struct SelectShared {
   int wsum[kWaves];
   int wflag[kWaves];
   uint32_t kmin, kmax;  // key range of the pool
+  int base;             // where this workgroup's entries go in the row's shared list
+  int last;             // this workgroup is the last of its row to arrive
 };
 
 __device__ __forceinline__ u64 composite(uint32_t key, int idx) {
@@ -517,128 +515,42 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
 }
 
 // ---------------------------------------------------------------------------
-// slices: everything at or above the row's sampled threshold
-// ---------------------------------------------------------------------------
-constexpr uint32_t kNoThreshold = 0xffffffffu;  // row is not filtered by slices (the row kernel does it all)
-
-// One workgroup per row: the sampled threshold of the row for the slice filter.
-template <bool VEC>
-__global__ __launch_bounds__(kThreads) void select_tau_kernel(
-    const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
-    const int32_t* __restrict__ budgets, int Hq, int T, int M, int sink, int window, int write_base,
-    int list_width, uint32_t* __restrict__ tau_out, int32_t* __restrict__ row_count) {
-  __shared__ uint32_t hist[kBins];
-  __shared__ SelectShared sh;
-  const int rowi = blockIdx.x, tid = threadIdx.x;
-  if (tid == 0) row_count[rowi] = 0;  // the slices add to it
-  int n, m, nbase;
-  row_shape(lens, budgets, rowi / Hq, T, M, sink, window, write_base, list_width, n, m, nbase);
-  // short rows are pooled whole by the row kernel; it also takes over when no
-  // threshold can be relied on
-  if (m == 0 || n <= kPoolCap || !sampling_ok(m)) {
-    if (tid == 0) tau_out[rowi] = kNoThreshold;
-    return;
-  }
-  const uint32_t tau = sample_threshold<kThreads, VEC>(scores + (int64_t)rowi * score_stride, n, m, hist, sh, tid);
-  // (a key of 0xffffffff is a NaN score; a threshold that high is as good as none)
-  if (tid == 0) tau_out[rowi] = tau;
-}
-
-// One workgroup of 256 lanes per slice of 16384 scores, in two halves of 32 keys
-// per lane held in registers between counting and writing.  What passes the
-// threshold goes to the ROW's list: a half's entries take a contiguous stretch
-// reserved with one atomic add on the row's counter, so the row kernel finds one
-// compact list (in no particular order; its result does not depend on it).  A
-// stretch that would run past the list's capacity is not written: the counter
-// then exceeds the capacity, which tells the row kernel to start from scratch.
-template <bool VEC>
-__global__ __launch_bounds__(kLocThreads) void select_local_kernel(
-    const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens, int Hq, int T,
-    const uint32_t* __restrict__ tau_in, u64* __restrict__ loc, int32_t* __restrict__ row_count) {
-  __shared__ int wsum[kLocWaves];
-  __shared__ int row_base;
-  const int s = blockIdx.x, rowi = blockIdx.y, tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int n = lens ? max(0, min(lens[rowi / Hq], T)) : T;
-  const int begin = s * kSliceLen, end = min(n, begin + kSliceLen);
-  const uint32_t tau = tau_in[rowi];
-  if (tau == kNoThreshold || end <= begin) return;
-  const float* row = scores + (int64_t)rowi * score_stride;
-  u64* my = loc + (int64_t)rowi * kPoolCap;
-  constexpr int kHalf = kLocPerLane / 2;
-  for (int half = 0; half < 2; ++half) {
-    // element e of lane t is index hbase + ((e / 4) * 256 + t) * 4 + e % 4; places past
-    // the row's end get key 0 and are excluded by their index
-    const int hbase = begin + half * (kSliceLen / 2);
-    uint32_t key[kHalf];
-#pragma unroll
-    for (int u = 0; u < kHalf / 4; ++u) {
-      const int i0 = hbase + (u * kLocThreads + tid) * 4;
-      float x[4] = {0.f, 0.f, 0.f, 0.f};
-      if (VEC && i0 + 4 <= end) {
-        const float4 v = *reinterpret_cast<const float4*>(row + i0);
-        x[0] = v.x;
-        x[1] = v.y;
-        x[2] = v.z;
-        x[3] = v.w;
-      } else {
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-          if (i0 + c < end) x[c] = row[i0 + c];
-      }
-#pragma unroll
-      for (int c = 0; c < 4; ++c) key[u * 4 + c] = score_to_key(x[c]);
-    }
-    auto index_of = [&](int e) { return hbase + ((e >> 2) * kLocThreads + tid) * 4 + (e & 3); };
-    int cnt = 0;
-#pragma unroll
-    for (int e = 0; e < kHalf; ++e) cnt += (key[e] >= tau && index_of(e) < end) ? 1 : 0;
-    const int incl = wave_incl_scan(cnt, lane);
-    __syncthreads();  // the earlier half's readers of wsum / row_base are done
-    if (lane == 63) wsum[wave] = incl;
-    __syncthreads();
-    int at = incl - cnt, total = 0;
-#pragma unroll
-    for (int w = 0; w < kLocWaves; ++w) {
-      if (w < wave) at += wsum[w];
-      total += wsum[w];
-    }
-    if (tid == 0) row_base = total ? atomicAdd(&row_count[rowi], total) : 0;
-    __syncthreads();
-    const int base = row_base;
-    if (base + total > kPoolCap) continue;  // (uniform) over capacity: see above
-    at += base;
-#pragma unroll
-    for (int e = 0; e < kHalf; ++e) {
-      const int i = index_of(e);
-      if (key[e] >= tau && i < end) my[at++] = composite(key[e], i);
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------
 // rows
 // ---------------------------------------------------------------------------
-// REGPOOL: the pooled composites stay in registers, eight per lane, instead of in
-// LDS.  Possible whenever the slices have run: a row then either brings a compact
-// list of at most kPoolCap entries or is itself that short.  Without the 64 KB
-// pool the kernel needs 72 KB of LDS and two rows share a CU.
-template <bool VEC, bool REGPOOL>
+// Agent-wide coherent accesses without a fence (written through / read past this
+// die's caches): what workgroups of one row on different dies exchange.
+__device__ __forceinline__ void store_coherent(u64* p, u64 v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ u64 load_coherent(const u64* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// `parts` workgroups per row (blockIdx.x = row * parts + part).  With parts > 1
+// each filters its share of the row against the same sampled threshold (every
+// part works it out for itself from the same sample), appends what passes to the
+// row's list in `loc` (a stretch reserved with one atomic add on row_count), and
+// the last part to arrive (row_done) selects from that list; the others leave.
+// row_count and row_done are zero on entry and zero again on exit.
+// The pooled composites are held in registers, eight per lane, from the moment
+// the pool is complete; LDS holds them only while they are being compacted.
+template <bool VEC>
 __global__ __launch_bounds__(kThreads) void select_list_kernel(
     const float* __restrict__ scores, int64_t score_stride, const int32_t* __restrict__ lens,
     const int32_t* __restrict__ budgets, const uint32_t* __restrict__ row_range, int range_parts,
     int Hq, int T, int M, int sink, int window, int write_base, int32_t* __restrict__ sparse_list,
     int64_t list_stride, int list_width, int32_t* __restrict__ sparse_len, int cap_above,
-    int counting_ok, int use_pool, const u64* __restrict__ loc, const int32_t* __restrict__ row_count) {
+    int counting_ok, int use_pool, int pool_slots, int parts, u64* __restrict__ loc,
+    int32_t* __restrict__ row_count, unsigned int* __restrict__ row_done) {
   __shared__ uint32_t hist[kBins];
   __shared__ SelectShared sh;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   u64* buf = reinterpret_cast<u64*>(lds_raw);  // winners                  [cap_above]
   u64* cand = buf + cap_above;                 // entries of the k-th bin  [kCandCap]
-  u64* pool = cand + kCandCap;                 // pooled composites        [kPoolCap] if use_pool and not REGPOOL
-  u64* tmp = pool + ((use_pool && !REGPOOL) ? kPoolCap : 0);  // counting placement [2*cap_above] if counting_ok
+  u64* pool = cand + kCandCap;                 // what passes the filter   [pool_slots]: kPoolCap for rows beyond that
+  u64* tmp = pool + pool_slots;                // counting placement       [2*cap_above] if counting_ok
 
-  const int rowi = blockIdx.x;
+  const int rowi = blockIdx.x / parts, part = blockIdx.x % parts;
   const int b = rowi / Hq;
   const int tid = threadIdx.x;
   const int lane = tid & (SOCKET_WAVE - 1);
@@ -647,8 +559,9 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
   row_shape(lens, budgets, b, T, M, sink, window, write_base, list_width, n, m, nbase);
   const float* row = scores + (int64_t)rowi * score_stride;
   int32_t* out = sparse_list + (int64_t)rowi * list_stride;
-  write_list_base(out, n, m, nbase, sink, window, write_base, list_width,
-                  sparse_len ? sparse_len + rowi : nullptr, tid, kThreads);
+  if (part == 0)
+    write_list_base(out, n, m, nbase, sink, window, write_base, list_width,
+                    sparse_len ? sparse_len + rowi : nullptr, tid, kThreads);
   if (m == 0) return;
   int32_t* heavy = out + nbase;
 
@@ -662,66 +575,43 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
       sh.kmax = 0u;
     }
     int total = -1;  // uniform; stays -1 when no pool could be formed
-    uint32_t kmin = 0xffffffffu, kmax = 0u;  // key range of what this lane pooled
+    uint32_t kmin = 0xffffffffu, kmax = 0u;  // key range of what this lane holds
     constexpr int U = kPoolCap / kThreads;
-    u64 pv[REGPOOL ? U : 1];                 // REGPOOL: entry tid + u * kThreads of the pool
-    if (n <= kPoolCap) {  // the whole row
-      if (REGPOOL) {
+    u64 pv[U];                               // entry tid + u * kThreads of the pool
+    if (n <= kPoolCap) {  // the whole row, by one workgroup
+      if (part != 0) return;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int i = tid + u * kThreads;
-          const uint32_t k = score_to_key(i < n ? row[i] : 0.f);
-          if (i < n) {
-            kmin = min(kmin, k);
-            kmax = max(kmax, k);
-          }
-          pv[REGPOOL ? u : 0] = composite(k, i);
-        }
-      } else {
-        for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
-          const uint32_t k = score_to_key(x);
+      for (int u = 0; u < U; ++u) {
+        const int i = tid + u * kThreads;
+        const uint32_t k = score_to_key(i < n ? row[i] : 0.f);
+        if (i < n) {
           kmin = min(kmin, k);
           kmax = max(kmax, k);
-          pool[i] = composite(k, i);
-        });
+        }
+        pv[u] = composite(k, i);
       }
       total = n;
-    } else if (loc) {  // what the slices found above the sampled threshold
-      // The row's list is compact; its length and its entries are requested
-      // together (entries past the length are stale and never used), so the
-      // gather costs one memory latency.
-      const u64* src = loc + (int64_t)rowi * kPoolCap;
-      const int sum = row_count[rowi];
-      u64 v[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) v[u] = src[tid + u * kThreads];
-      if (sum >= m && sum <= kPoolCap) {
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-          if (tid + u * kThreads < sum) {
-            const uint32_t k = (uint32_t)(v[u] >> 32);
-            kmin = min(kmin, k);
-            kmax = max(kmax, k);
-            if (REGPOOL) pv[REGPOOL ? u : 0] = v[u];
-            else pool[tid + u * kThreads] = v[u];
-          }
-        total = sum;
-      }
-    } else if (!REGPOOL && sampling_ok(m)) {  // one workgroup: threshold from the sample, one pass
+    } else if (sampling_ok(m)) {
+      // This part's share of the row; the last part also takes the one to three
+      // scores past the last multiple of four.
+      const int n4 = n & ~3;
+      const int chunk = (((n + parts - 1) / parts) + 3) & ~3;
+      const int begin = min(part * chunk, n4), e4 = min(begin + chunk, n4);
+      const int tail_end = (part == parts - 1) ? n : e4;
       if (VEC) {
-        // The row in batches of 16 scores per lane (four 16-byte loads, all in
-        // flight together); the first two batches are requested before the threshold is
-        // worked out, each further one two batches ahead of the one being filtered.  A wave
-        // counts what passes in its batch, reserves a stretch of the pool with one
-        // LDS atomic and writes its entries there: no barrier in the loop.
+        // In batches of 16 scores per lane (four 16-byte loads, all in flight
+        // together); the first two batches are requested before the threshold is
+        // worked out, each further one two batches ahead of the one being filtered.  A
+        // wave counts what passes in its batch, reserves a stretch of the pool with
+        // one LDS atomic and writes its entries there: no barrier in the loop.
         constexpr int kLoads = 4, kStep = kThreads * 4 * kLoads;
-        const int n4 = n & ~3;
+        static_assert(kStep == kBatch, "batch size");
         auto fetch = [&](int base, float4 (&x)[kLoads]) {
 #pragma unroll
           for (int u = 0; u < kLoads; ++u) {
-            // (past the end: the row's last four, fetched and ignored -- a load under a
-            // condition would make every wait in the loop a wait for all loads)
-            const int i0 = min(base + (u * kThreads + tid) * 4, n4 - 4);
+            // (past the end: the share's last four, fetched and ignored -- a load under
+            // a condition would make every wait in the loop a wait for all loads)
+            const int i0 = max(min(base + (u * kThreads + tid) * 4, e4 - 4), 0);
             x[u] = *reinterpret_cast<const float4*>(row + i0);
           }
         };
@@ -731,12 +621,12 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         // below -inf's is no float's key and is widened to that infinity (the pool
         // only has to hold everything at or above tau; more is allowed).
         auto filter = [&](int base, const float4 (&x)[kLoads], float tau_f) {
-          if (base >= n4) return;  // uniform
+          if (base >= e4) return;  // uniform
           uint32_t taken = 0;      // bit u * 4 + c: score c of load u passes
 #pragma unroll
           for (int u = 0; u < kLoads; ++u) {
             const float xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
-            const bool in = base + (u * kThreads + tid) * 4 < n4;
+            const bool in = base + (u * kThreads + tid) * 4 < e4;
 #pragma unroll
             for (int c = 0; c < 4; ++c) taken |= (in && !(xs[c] < tau_f)) ? (1u << (u * 4 + c)) : 0u;
           }
@@ -760,12 +650,12 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
           }
         };
         float4 b0[kLoads], b1[kLoads], b2[kLoads];
-        fetch(0, b0);
-        fetch(kStep, b1);
+        fetch(begin, b0);
+        fetch(begin + kStep, b1);
         const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
         const float tau_f = tau >= 0xff800000u ? INFINITY : tau <= 0x007fffffu ? -INFINITY
                             : __uint_as_float((tau & 0x80000000u) ? (tau & 0x7fffffffu) : ~tau);
-        for (int base = 0; base < n4; base += 3 * kStep) {
+        for (int base = begin; base < e4; base += 3 * kStep) {
           fetch(base + 2 * kStep, b2);
           filter(base, b0, tau_f);
           fetch(base + 3 * kStep, b0);
@@ -773,41 +663,72 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
           fetch(base + 4 * kStep, b1);
           filter(base + 2 * kStep, b2, tau_f);
         }
-        // the last one to three scores of a row whose length is no multiple of four
         if (wave == 0) {
-          const int i = n4 + lane;
-          const float x = i < n ? row[i] : 0.f;
-          wave_append(i < n && !(x < tau_f), composite(__float_as_uint(x), i), &sh.fill_pool, pool, kPoolCap);
-        }
-        __syncthreads();
-        // the pooled scores become keys, eight entries a lane at most
-        const int got = min(sh.fill_pool, kPoolCap);
-        for (int i = tid; i < got; i += kThreads) {
-          const u64 e = pool[i];
-          const uint32_t k = score_to_key(__uint_as_float((uint32_t)(e >> 32)));
-          kmin = min(kmin, k);
-          kmax = max(kmax, k);
-          pool[i] = ((u64)k << 32) | (e & 0xffffffffull);
+          const int i = e4 + lane;
+          const float x = i < tail_end ? row[i] : 0.f;
+          wave_append(i < tail_end && !(x < tau_f), composite(__float_as_uint(x), i), &sh.fill_pool, pool, kPoolCap);
         }
       } else {
         const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
-        for_each_in<VEC, kThreads>(row, 0, n, tid, [&](int i, float x) {
-          const uint32_t k = score_to_key(x);
-          if (k >= tau) {
-            kmin = min(kmin, k);
-            kmax = max(kmax, k);
-          }
-          wave_append(k >= tau, composite(k, i), &sh.fill_pool, pool, kPoolCap);
+        for_each_in<VEC, kThreads>(row, begin, tail_end, tid, [&](int i, float x) {
+          wave_append(score_to_key(x) >= tau, composite(__float_as_uint(x), i), &sh.fill_pool, pool, kPoolCap);
         });
       }
       __syncthreads();
-      const int got = sh.fill_pool;
-      if (got >= m && got <= kPoolCap) total = got;
+      // (an entry of the pool: the score's bits over the complemented index)
+      auto keyed = [](u64 e) {
+        return ((u64)score_to_key(__uint_as_float((uint32_t)(e >> 32))) << 32) | (e & 0xffffffffull);
+      };
+      const int got = sh.fill_pool;   // what passed here, also when it is more than the pool holds
+      if (parts == 1) {
+        if (got >= m && got <= kPoolCap) {
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            if (tid + u * kThreads < got) pv[u] = keyed(pool[tid + u * kThreads]);
+          total = got;
+        }
+      } else {
+        if (tid == 0) sh.base = atomicAdd(&row_count[rowi], got);
+        __syncthreads();
+        const int at = sh.base;
+        u64* mine = loc + (int64_t)rowi * kPoolCap;
+        if (at + got <= kPoolCap) {   // (a row whose parts pass more than the list holds is redone from scratch)
+          for (int i = tid; i < got; i += kThreads) store_coherent(mine + at + i, keyed(pool[i]));
+        }
+        // Every lane waits until its written-through stores have been acknowledged,
+        // the barrier collects the lanes, and only then is the ticket drawn: whoever
+        // draws the last one can read every part's entries.
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (tid == 0) sh.last = atomicInc(&row_done[rowi], (unsigned int)(parts - 1)) == (unsigned int)(parts - 1);
+        __syncthreads();
+        if (!sh.last) return;
+        const int sum = __hip_atomic_load(&row_count[rowi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (tid == 0) __hip_atomic_store(&row_count[rowi], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (sum >= m && sum <= kPoolCap) {
+#pragma unroll
+          for (int u = 0; u < U; ++u)
+            if (tid + u * kThreads < sum) pv[u] = load_coherent(mine + tid + u * kThreads);
+          total = sum;
+        }
+      }
+      if (total >= 0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (tid + u * kThreads < total) {
+            const uint32_t k = (uint32_t)(pv[u] >> 32);
+            kmin = min(kmin, k);
+            kmax = max(kmax, k);
+          }
+      }
+    } else if (part != 0) {
+      return;   // no threshold can be relied on: one workgroup selects from scratch
     }
     __syncthreads();
     if (total >= 0) {
-      // range of the pooled composites, from their keys (the high halves, noted
-      // as the pool was filled): any range that holds them all serves the refinement
+      // range of the pooled composites, from their keys (the high halves): any range
+      // that holds them all serves the refinement
 #pragma unroll
       for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
         kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
@@ -835,17 +756,10 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         const int shift = range_shift(lo, hi);
         for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
         __syncthreads();
-        if (REGPOOL) {
 #pragma unroll
-          for (int u = 0; u < U; ++u) {
-            const u64 v = pv[REGPOOL ? u : 0];
-            if (tid + u * kThreads < total && v >= lo && v <= hi) atomicAdd(&hist[(int)((v - lo) >> shift)], 1u);
-          }
-        } else {
-          for (int i = tid; i < total; i += kThreads) {
-            const u64 v = pool[i];
-            if (v >= lo && v <= hi) atomicAdd(&hist[(int)((v - lo) >> shift)], 1u);
-          }
+        for (int u = 0; u < U; ++u) {
+          const u64 v = pv[u];
+          if (tid + u * kThreads < total && v >= lo && v <= hi) atomicAdd(&hist[(int)((v - lo) >> shift)], 1u);
         }
         __syncthreads();
         find_bin<kThreads>(hist, need_in, 1, sh, tid);
@@ -862,26 +776,20 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
       }
       const u64 blo = sh.lo, bhi = sh.hi;
       const int need = sh.need;
-      if (REGPOOL) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const u64 v = pv[REGPOOL ? u : 0];
-          const bool have = tid + u * kThreads < total;
-          wave_append(have && v > bhi, v, &sh.fill_above, buf, cap_above);
-          wave_append(have && v >= blo && v <= bhi, v, &sh.fill_cand, cand, kCandCap);
-        }
-      } else {
-        for (int i = tid; i < total; i += kThreads) {
-          const u64 v = pool[i];
-          wave_append(v > bhi, v, &sh.fill_above, buf, cap_above);
-          wave_append(v >= blo && v <= bhi, v, &sh.fill_cand, cand, kCandCap);
-        }
+      for (int u = 0; u < U; ++u) {
+        const u64 v = pv[u];
+        const bool have = tid + u * kThreads < total;
+        wave_append(have && v > bhi, v, &sh.fill_above, buf, cap_above);
+        wave_append(have && v >= blo && v <= bhi, v, &sh.fill_cand, cand, kCandCap);
       }
       __syncthreads();
       order_and_write(buf, m - need, cand, min(sh.fill_cand, kCandCap), need, lo0, shift0, tmp, hist, sh,
                       counting_ok != 0, heavy, tid);
       return;
     }
+  } else if (part != 0) {
+    return;
   }
 
   // ================================ from scratch ======================================
@@ -1019,24 +927,29 @@ int next_pow2(int x) {
   return p;
 }
 
-// One workgroup per row does everything (threshold from the sample, one streaming
-// pass, select) in about 19 + 1.47 us per slice length of its row; with slices the
-// three launches cost about 27.5 us + 3.2 us per (rows x slices / CU).  Slices
-// therefore pay off for few, long rows only (measured on 256 CUs, top-k 2048:
-// 32 rows from 131072 scores up, 64 rows from about 200000, 128 rows never).
-bool use_slices(int rows, int T, int m_max, int* S_out) {
-  const int S = (T + kSliceLen - 1) / kSliceLen;
-  *S_out = S;
-  if (!(S >= 4 && S <= kMaxSlices && m_max > 0 && sampling_ok(m_max))) return false;
-  const float cus = (float)socket_device_limits().cu_count;
-  return (float)S * (1.467f - 3.2f * (float)rows / cus) > 8.2f;
+// Workgroups per row.  One workgroup streams its row at what one CU can pull
+// (about 35 GB/s: 3.7 us per 32768 scores); sharing a row between several costs
+// about 3 us for the exchange through memory, more when the launch then fills
+// every CU (each part works out the threshold from the same sample, and each
+// needs a CU to itself for its LDS).  Measured on 256 CUs with top-k 2048: two
+// parts never pay; 8 or 32 rows gain from 49152 / 65536 scores up (9.5 and 7.6 us
+// at 131072), 64 rows from 98304 up, 128 rows never.
+int row_parts(int rows, int T, int m_max) {
+  if (!(T > kPoolCap && m_max > 0 && sampling_ok(m_max))) return 1;
+  const int cus = socket_device_limits().cu_count;
+  int p = cus / rows;
+  p = p < kMaxParts ? p : kMaxParts;
+  p = p < T / kBatch ? p : T / kBatch;
+  if (p < 3) return 1;
+  const double saved = (double)T * (p - 1) / p;                 // scores a workgroup no longer streams
+  return saved >= 24576.0 + 49152.0 * rows * p / cus ? p : 1;
 }
 
 struct SplitLayout {
-  size_t off_loc, off_count, off_tau, total;
+  size_t off_loc, off_count, off_done, total;
 };
 
-// per row: a candidate list of kPoolCap composites, its length, the threshold
+// per row: a list of kPoolCap composites, its length, the arrivals
 SplitLayout split_layout(int rows) {
   SplitLayout l;
   size_t o = 0;
@@ -1045,9 +958,9 @@ SplitLayout split_layout(int rows) {
     o += (bytes + 255) / 256 * 256;
     return at;
   };
+  l.off_count = take((size_t)rows * sizeof(int32_t));     // the two counter arrays first: they are
+  l.off_done = take((size_t)rows * sizeof(uint32_t));     // what has to be zero on entry
   l.off_loc = take((size_t)rows * kPoolCap * sizeof(u64));
-  l.off_count = take((size_t)rows * sizeof(int32_t));
-  l.off_tau = take((size_t)rows * sizeof(uint32_t));
   l.total = o;
   return l;
 }
@@ -1056,9 +969,13 @@ SplitLayout split_layout(int rows) {
 
 extern "C" size_t socket_select_workspace_bytes(int B, int Hq, int T, int M) {
   if (B <= 0 || Hq <= 0 || T <= 0 || M < 0) return 0;
-  int S = 0;
-  if (!use_slices(B * Hq, T, M < T ? M : T, &S)) return 0;
+  if (row_parts(B * Hq, T, M < T ? M : T) < 2) return 0;
   return split_layout(B * Hq).total;
+}
+
+extern "C" size_t socket_select_workspace_zero_bytes(int B, int Hq, int T, int M) {
+  if (socket_select_workspace_bytes(B, Hq, T, M) == 0) return 0;
+  return split_layout(B * Hq).off_loc;
 }
 
 extern "C" int socket_select_list(const float* scores, int64_t score_stride, const int32_t* lens,
@@ -1086,16 +1003,13 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
 
   // extras as LDS allows: the pool (where a pooled select can apply at all), then
   // counting placement (2 * cap_above more slots)
-  // With slices the pool lives in registers (a row brings at most kPoolCap entries or
-  // is that short itself) and costs no LDS.
-  int use_pool = 0, counting_ok = 0;
-  int S = 0;
-  const bool pool_applies = T <= kPoolCap || sampling_ok(m_max);
-  const bool slices = workspace && pool_applies && use_slices(rows, T, m_max, &S);
-  if (slices) {
+  // (rows of at most kPoolCap scores are pooled whole, straight into registers)
+  int use_pool = 0, counting_ok = 0, pool_slots = 0;
+  if (T <= kPoolCap) {
     use_pool = 1;
-  } else if (pool_applies && lds + (size_t)kPoolCap * sizeof(u64) + lds_static <= lds_max) {
+  } else if (sampling_ok(m_max) && lds + (size_t)kPoolCap * sizeof(u64) + lds_static <= lds_max) {
     use_pool = 1;
+    pool_slots = kPoolCap;
     lds += (size_t)kPoolCap * sizeof(u64);
   }
   if (lds + (size_t)2 * cap_above * sizeof(u64) + lds_static <= lds_max) {
@@ -1103,43 +1017,31 @@ extern "C" int socket_select_list(const float* scores, int64_t score_stride, con
     lds += (size_t)2 * cap_above * sizeof(u64);
   }
 
-  const u64* loc = nullptr;
-  const int32_t* loc_count = nullptr;
-  if (slices) {
+  // rows shared between workgroups exchange their entries through the workspace
+  int parts = (workspace && use_pool) ? row_parts(rows, T, m_max) : 1;
+  u64* loc = nullptr;
+  int32_t* row_count = nullptr;
+  unsigned int* row_done = nullptr;
+  if (parts > 1) {
     const SplitLayout l = split_layout(rows);
     SOCKET_REQUIRE(workspace_bytes >= l.total, SOCKET_ERR_WORKSPACE);
     SOCKET_REQUIRE(socket_aligned16(workspace), SOCKET_ERR_ALIGN);
     char* ws = (char*)workspace;
-    u64* loc_w = (u64*)(ws + l.off_loc);
-    int32_t* count_w = (int32_t*)(ws + l.off_count);
-    uint32_t* tau_w = (uint32_t*)(ws + l.off_tau);
-    const dim3 sgrid(S, rows);
-    if (vec) {
-      hipLaunchKernelGGL(select_tau_kernel<true>, dim3(rows), dim3(kThreads), 0, s, scores, score_stride, lens,
-                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w, count_w);
-      hipLaunchKernelGGL(select_local_kernel<true>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride, lens,
-                         Hq, T, tau_w, loc_w, count_w);
-    } else {
-      hipLaunchKernelGGL(select_tau_kernel<false>, dim3(rows), dim3(kThreads), 0, s, scores, score_stride, lens,
-                         budgets, Hq, T, M, sink, window, write_base, list_width, tau_w, count_w);
-      hipLaunchKernelGGL(select_local_kernel<false>, sgrid, dim3(kLocThreads), 0, s, scores, score_stride, lens,
-                         Hq, T, tau_w, loc_w, count_w);
-    }
-    SOCKET_LAUNCH_CHECK();
-    loc = loc_w;
-    loc_count = count_w;
+    loc = (u64*)(ws + l.off_loc);
+    row_count = (int32_t*)(ws + l.off_count);
+    row_done = (unsigned int*)(ws + l.off_done);
   }
+  SOCKET_REQUIRE((int64_t)rows * parts <= 0x7fffffff, SOCKET_ERR_SHAPE);
 
-  auto kern = slices ? (vec ? select_list_kernel<true, true> : select_list_kernel<false, true>)
-                     : (vec ? select_list_kernel<true, false> : select_list_kernel<false, false>);
+  auto kern = vec ? select_list_kernel<true> : select_list_kernel<false>;
   if (lds > 32 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return SOCKET_ERR_LAUNCH;
-  hipLaunchKernelGGL(kern, dim3(rows), dim3(kThreads), lds, s, scores, score_stride, lens, budgets,
+  hipLaunchKernelGGL(kern, dim3(rows * parts), dim3(kThreads), lds, s, scores, score_stride, lens, budgets,
                      row_range, range_parts, Hq, T, M, sink, window, write_base, sparse_list,
-                     list_stride, list_width, sparse_len, cap_above, counting_ok, use_pool, loc,
-                     loc_count);
+                     list_stride, list_width, sparse_len, cap_above, counting_ok, use_pool, pool_slots, parts,
+                     loc, row_count, row_done);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }

@@ -33,6 +33,22 @@ def _get_soft_hash_ext():
     return _SOFT_HASH_EXT
 
 
+# Workspaces of the selection, one per (device, stream, size): the kernel wants the
+# arrival counters at its head zero on entry and leaves them zero, so a workspace is
+# zeroed once, when it is made, and serves every later call issued on that stream.
+_SELECT_WS = {}
+
+
+def _select_workspace(device: torch.device, nbytes: int, zero_bytes: int) -> torch.Tensor:
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream, nbytes)
+    ws = _SELECT_WS.get(key)
+    if ws is None:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        ws[:zero_bytes].zero_()
+        _SELECT_WS[key] = ws
+    return ws
+
+
 def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=None, budgets=None,
                 write_base: bool = True, list_width=None, row_range=None, split: bool = True):
     """Top-M + [sink | window | heavy] assembly on fp32 score rows [B,H,T]
@@ -41,7 +57,7 @@ def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=No
     (per-sequence context length and top-k budget).  `row_range`: the int32
     [B,H,parts,2] key ranges `hash_cache.score_packed(..., with_range=True)`
     returns for these scores (saves the kernel's first pass).  `split=False`
-    forces the one-workgroup-per-row kernel (the result is the same)."""
+    keeps every row to one workgroup (the result is the same)."""
     assert scores.is_cuda and scores.dtype == torch.float32 and scores.dim() == 3
     assert scores.stride(2) == 1 and scores.stride(0) == scores.shape[1] * scores.stride(1)
     B, H, T = scores.shape
@@ -62,7 +78,7 @@ def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=No
     L = lib()
     ws, ws_bytes = None, L.socket_select_workspace_bytes(B, H, T, M) if split else 0
     if ws_bytes:
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=scores.device)
+        ws = _select_workspace(scores.device, ws_bytes, L.socket_select_workspace_zero_bytes(B, H, T, M))
     check("socket_select_list", L.socket_select_list(
         ptr(scores), scores.stride(1), ptr(lens), ptr(budgets), ptr(row_range),
         0 if row_range is None else row_range.shape[2], B, H, T, M, int(sink), int(window),
