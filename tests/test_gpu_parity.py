@@ -296,6 +296,26 @@ def test_select_ragged_lengths_and_budgets(dev, T):
     _check_select(scores, 4, 128, 500, dev, lens=lens, budgets=budgets)
 
 
+def test_select_long_rows_with_an_odd_pitch(dev):
+    """Rows long and few enough to be shared between workgroups, at a row pitch
+    that rules out 16-byte loads (the scalar-load variant of the same kernel),
+    with ragged lengths and budgets."""
+    g = torch.Generator().manual_seed(23)
+    B, H, T, M = 2, 2, 100003, 700
+    scores = (torch.randn(B, H, T, generator=g) * 2).to(dev)          # pitch T: odd
+    assert scores.stride(1) % 4 != 0
+    lens = torch.tensor([T, 60001], dtype=torch.int32)
+    budgets = torch.tensor([700, 333], dtype=torch.int32)
+    sl, ln = sparse.select_list(scores, 4, 64, M, lens=lens.to(dev), budgets=budgets.to(dev))
+    sl, ln, sc = sl.cpu(), ln.cpu(), scores.cpu()
+    for b in range(B):
+        n, m = int(lens[b]), int(budgets[b])
+        base = torch.from_numpy(orc.base_indices(n, 4, 64))
+        for h in range(H):
+            want = torch.cat([base, orc.topk_lower_index_first(sc[b, h, :n], m).to(torch.int32)])
+            assert int(ln[b, h]) == want.numel() and torch.equal(sl[b, h, :want.numel()], want), (b, h)
+
+
 def test_select_base_enumeration(dev):
     """List arithmetic for every small T (sparse.py:70-95), including the
     'empty base -> [T-1]' rule."""

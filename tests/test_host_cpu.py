@@ -104,7 +104,7 @@ def test_sizes_helpers(lib):
     ns = (2308 + bs - 1) // bs
     assert lib.socket_sparse_attention_workspace_bytes(4, 32, 128, 2308) == 4 * 32 * ns * 129 * 4
     assert lib.socket_select_workspace_bytes(4, 32, 4096, 128) == 0        # short rows: one workgroup per row
-    assert lib.socket_select_workspace_bytes(1, 32, 131072, 2048) > 0      # few long rows: filtered by slices
+    assert lib.socket_select_workspace_bytes(1, 32, 131072, 2048) > 0      # few long rows: shared between workgroups
     assert lib.socket_select_workspace_bytes(4, 32, 131072, 2048) == 0     # a row per CU and more: one workgroup each
     assert lib.socket_score_range_parts(4, 32, 8, 131072, 1, 60, 10, 1024) * 8192 >= 131072
     assert lib.socket_score_range_parts_grouped(4, 32, 8, 131072, 1, 60, 10, 1024) == 16
