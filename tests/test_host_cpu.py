@@ -76,11 +76,28 @@ def test_entry_points_reject_bad_arguments_without_a_device(lib):
     assert lib.socket_hash_keys(one, nul, 1, 0, 0, 128, 0, 0, 128, one, one, nul, nul, 4, 1, 1, 8, 128, 60, 10, 8, nul) == _lib.SOCKET_ERR_SHAPE  # t0 + S > Tcap
     assert lib.socket_select_list(one, 64, nul, nul, nul, 0, 1, 1, 64, 20000, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # M too large
     assert lib.socket_select_list(one, 32, nul, nul, nul, 0, 1, 1, 64, 4, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_SHAPE  # pitch < T
+    need = lib.socket_select_workspace_bytes(1, 8, 131072, 2048)       # few long rows: a workspace is asked for
+    assert need > lib.socket_select_workspace_zero_bytes(1, 8, 131072, 2048) > 0
+    assert lib.socket_select_list(one, 131072, nul, nul, nul, 0, 1, 8, 131072, 2048, 4, 64, 1, one, 2400, 2400, nul, one, need - 1,
+                                  nul) == _lib.SOCKET_ERR_WORKSPACE
     a = [one, one, one, 1, 128, 128, 0, 0, 128, 0, 0, 128, one, 8, 8, one, 1, 1, one, one]
     assert lib.socket_attend_stage1(*a, 1, 4, 1, 48, 16, 8, 1, 256, nul) == _lib.SOCKET_ERR_UNSUPPORTED       # D = 48
     assert lib.socket_attend_stage1(*a, 1, 5, 2, 128, 16, 8, 1, 256, nul) == _lib.SOCKET_ERR_SHAPE             # Hq % Hkv
     a[5] = 100                                                                                            # q head stride not 16-byte aligned for bf16
     assert lib.socket_attend_stage1(*a, 1, 4, 1, 128, 16, 8, 1, 256, nul) == _lib.SOCKET_ERR_ALIGN
+    # the fused head of a decode step: bf16, D = 128, K = 10 only; strides in steps of 16 bytes
+    def prologue(dtype=1, D=128, K=10, qkv=one, qkv_sb=6144, Hq=32, Hkv=8, R=1024, css=128):
+        return lib.socket_decode_prologue(qkv, dtype, qkv_sb, one, 1, 64, one, 0, one, one, one, 8 * 64 * 128, 64 * 128, css, nul,
+                                          one, one, one, one, one, one, 1, 1, 1, Hq, Hkv, D, 60, K, R, 64, 0.088, 1.0, nul)
+    assert prologue(qkv=nul) == _lib.SOCKET_ERR_NULL
+    assert prologue(dtype=0) == _lib.SOCKET_ERR_UNSUPPORTED          # fp32 activations: the three separate entry points
+    assert prologue(D=64) == _lib.SOCKET_ERR_UNSUPPORTED
+    assert prologue(K=8) == _lib.SOCKET_ERR_UNSUPPORTED
+    assert prologue(R=2048) == _lib.SOCKET_ERR_UNSUPPORTED
+    assert prologue(Hq=36, Hkv=8) == _lib.SOCKET_ERR_SHAPE            # Hq % Hkv
+    assert prologue(Hq=72, Hkv=8) == _lib.SOCKET_ERR_UNSUPPORTED      # nine heads per KV head
+    assert prologue(qkv_sb=6148) == _lib.SOCKET_ERR_ALIGN
+    assert prologue(css=132) == _lib.SOCKET_ERR_ALIGN
     # workspace too small
     need = lib.socket_sparse_attention_workspace_bytes(1, 4, 128, 300)
     assert need > 0
