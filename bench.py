@@ -9,10 +9,13 @@ configuration 3 (batch 4, 32/8 heads, head dim 128, 131072-token bf16 cache,
 L=60 x P=10, top-k 2048 + 4 sink + 256 window).
 
 Prints one JSON line.  `value` is microseconds per layer per step of the sparse
-path on configuration 3, exactly --steps graph replays after --warmup, taken
-in the sustained power state of a decode loop (a settle phase of untimed
-replays comes first; the figure of a burst that starts on an idle GPU is
-reported beside it as `power_state.us_per_step_from_idle`); `roofline`
+path on configuration 3: exactly --steps steps after --warmup, recorded back to
+back into one HIP graph as the layers of a decode step are in the model's graph
+(`power_state.steps_per_graph`; the figure with one graph launch per step is
+beside it as `us_per_step_one_graph_launch_each`), taken in the sustained power
+state of a decode loop (a settle phase of untimed replays comes first; the
+figure of a burst that starts on an idle GPU is reported as
+`power_state.us_per_step_from_idle`); `roofline`
 prices the scorer (the kernel moving the most bytes) against HBM peak; `kernels`
 does the same for every kernel of the step and for the dense flash-decode
 comparator on the same GPU (each timed as a HIP-graph replay of ten launches, so
@@ -417,27 +420,55 @@ def timed_graph_steps(step_fn, steps, warmup, eager=False):
             graph, ok = None, None
     run = graph.replay if graph is not None else step_fn
 
-    def timed():
+    # The timed replays: `per` steps recorded back to back into one graph, as the
+    # layers of a decode step are (32 of them per token in the model's graph), so
+    # the figure carries the in-graph gap between steps and not the larger one
+    # between two graph launches.  `per` divides `steps`: exactly `steps` steps run.
+    per, graph_k = 1, None
+    if graph is not None:
+        per = max(d for d in range(1, min(steps, 64) + 1) if steps % d == 0)
+        if per > 1:
+            try:
+                graph_k = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph_k):
+                    for _ in range(per):
+                        out_k = step_fn()
+                graph_k.replay()
+                torch.cuda.synchronize()
+                if not torch.equal(out_k, out_eager):
+                    raise RuntimeError("replay of the multi-step graph differs from the eager step")
+            except Exception as e:  # noqa: BLE001
+                print(f"bench: multi-step graph unavailable ({e}); one graph launch per step", file=sys.stderr)
+                per, graph_k = 1, None
+        if graph_k is None:
+            per = 1
+    run_k = graph_k.replay if graph_k is not None else run
+
+    def timed(fn, calls, steps_per_call):
         for _ in range(warmup):
             run()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()
-        for _ in range(steps):
-            run()
+        for _ in range(calls):
+            fn()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps, (time.perf_counter() - t0) * 1e3
+        return e0.elapsed_time(e1) / (calls * steps_per_call), (time.perf_counter() - t0) * 1e3
 
     # once from an idle GPU (reported beside the result), then after the settle phase
     torch.cuda.synchronize()
     time.sleep(0.05)
-    after_idle_ms, _ = timed()
+    after_idle_ms, _ = timed(run_k, steps // per, per)
     settled = settle(run)
-    ms_per_step, wall_ms = timed()
-    return (ms_per_step, wall_ms, "hip graph replay" if graph is not None else "eager", ok,
-            {"settle_steps_untimed": settled, "settle_ms": SETTLE_MS, "us_per_step_from_idle": round(after_idle_ms * 1e3, 2)})
+    ms_per_step, wall_ms = timed(run_k, steps // per, per)
+    state = {"settle_steps_untimed": settled, "settle_ms": SETTLE_MS,
+             "us_per_step_from_idle": round(after_idle_ms * 1e3, 2), "steps_per_graph": per}
+    if graph_k is not None:
+        single_ms, _ = timed(run, steps, 1)
+        state["us_per_step_one_graph_launch_each"] = round(single_ms * 1e3, 2)
+    return (ms_per_step, wall_ms, ("hip graph replay" if graph is not None else "eager"), ok, state)
 
 
 def measure_workload(w, dev, steps, warmup, args, full):

@@ -23,7 +23,7 @@ from typing import Optional, Tuple
 import torch
 
 from ._lib import check, dtype_enum, lib, ptr, stream_ptr
-from .socket_kernels import fits_static_scratch, sparse_attention_fwd, sparse_attention_fwd_static
+from .socket_kernels import prefers_one_launch, sparse_attention_fwd, sparse_attention_fwd_static
 from .sparse import select_list
 
 
@@ -342,7 +342,7 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens, n_heads=q.shape[1])
     sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets)
     B, Hq, D = q.shape
-    if fits_static_scratch(B, Hq, D, sparse_list.shape[-1]):
+    if prefers_one_launch(B, Hq, D, sparse_list.shape[-1]):
         # one launch (the last split of a row merges it) on the library's own scratch array;
         # the decode step is issued on one stream, as that entry point requires
         out = sparse_attention_fwd_static(q, k_cache, v_cache, sparse_list, sparse_len,
