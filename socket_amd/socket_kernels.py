@@ -188,16 +188,16 @@ def fits_static_scratch(B: int, H: int, D: int, width: int) -> bool:
 def prefers_one_launch(B: int, H: int, D: int, width: int) -> bool:
     """Which of the two attention entry points a decode step should take: the
     one-launch variant (the last split of a row merges it) wherever it fits and
-    the launch has a workgroup per CU or more.  Below that the merge is a serial
-    tail behind a handful of splits and a second, tiny launch is the faster
-    (32 rows x 4 splits: 55.6 against 57.5 us per step on 256 CUs)."""
+    there is a row for every other CU or more.  With few rows the merge is a
+    serial tail that every row reaches at about the same time, and a second, tiny
+    launch does as well or better (on 256 CUs, steps of 32 rows: 55.6 against
+    57.5 us with lists of 1156 entries, equal with 2308; 128 rows: 162.6 against
+    165.7 us the other way)."""
     if not fits_static_scratch(B, H, D, width):
         return False
-    L = lib()
     cus = ctypes.c_int(0)
-    L.socket_device_query(ctypes.byref(cus), None)
-    block_seq = L.socket_sparse_attention_block_seq(B, H, width)
-    return B * H * ((width + block_seq - 1) // block_seq) >= cus.value
+    lib().socket_device_query(ctypes.byref(cus), None)
+    return 2 * B * H >= cus.value
 
 
 @torch.no_grad()

@@ -139,6 +139,19 @@ def test_sizes_helpers(lib):
     assert lib.socket_score_prefers_grouped(1, 5, 2, 100, 1, 60, 10, 1024) == -1
 
 
+def test_attention_entry_point_by_launch_size(lib):
+    """The decode step takes the one-launch attention where there is a row for
+    every other CU or more (256 CUs assumed without a device) and the call fits
+    the library's fixed scratch array, else the two-launch one."""
+    from socket_amd import socket_kernels as sk
+    sk.prefers_one_launch.cache_clear()
+    assert sk.prefers_one_launch(4, 32, 128, 2308)            # 128 rows
+    assert sk.prefers_one_launch(16, 28, 128, 2100)           # 448 rows
+    assert not sk.prefers_one_launch(1, 32, 128, 1156)        # 32 rows
+    assert not sk.prefers_one_launch(64, 512, 128, 4096)      # beyond the scratch array
+    sk.prefers_one_launch.cache_clear()
+
+
 def _plan(lib, B, Hq, Hkv, T, dt, L, P, grouped):
     from ctypes import byref, c_float, c_int
     tile, direct, one_head, cost = c_int(), c_int(), c_int(), c_float()
