@@ -300,8 +300,7 @@ __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
       float d = 0.f;
 #pragma unroll
       for (int i = 0; i < E; ++i) d += qf[i] * kf[i];
-#pragma unroll
-      for (int x = 1; x < LPR; x <<= 1) d += __shfl_xor(d, x, SOCKET_WAVE);
+      d = group_sum<LPR>(d);
       sc[u] = live[u] ? d * sm_scale : -INFINITY;
       nm = fmaxf(nm, sc[u]);
     }
@@ -412,8 +411,7 @@ __global__ __launch_bounds__(kAttThreads) void dense_stage1_kernel(
         float d = 0.f;
 #pragma unroll
         for (int i = 0; i < E; ++i) d += qf[g][i] * kf[i];
-#pragma unroll
-        for (int x = 1; x < LPR; x <<= 1) d += __shfl_xor(d, x, SOCKET_WAVE);
+        d = group_sum<LPR>(d);
         sc[u][g] = live[u] ? d * sm_scale : -INFINITY;
       }
     }

@@ -131,6 +131,35 @@ __device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s
   im = cc + d;
 }
 
+// Step MASK (1, 2, 4 or 8) of a butterfly sum over lanes: the value a lane adds to
+// its own.  After the steps below MASK every lane of an aligned group of MASK
+// lanes holds the same value, so any lane of the partner group serves, and the
+// quad permutes and the half-row and row mirrors of the vector ALU's data-parallel
+// primitives deliver one -- without a trip through the LDS crossbar.
+template <int MASK>
+__device__ __forceinline__ float butterfly_partner(float x) {
+  static_assert(MASK == 1 || MASK == 2 || MASK == 4 || MASK == 8, "inside a row of 16 lanes");
+  constexpr int ctrl = MASK == 1 ? 0xB1     // quad_perm [1,0,3,2]
+                     : MASK == 2 ? 0x4E     // quad_perm [2,3,0,1]
+                     : MASK == 4 ? 0x141    // row_half_mirror: lane i <- lane 7 - i of its half row
+                                 : 0x140;   // row_mirror: lane i <- lane 15 - i of its row
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), ctrl, 0xf, 0xf, false));
+}
+
+// Sum of x over each aligned group of N lanes (N a power of two up to 64), left in
+// every lane of the group; the same pairs in the same order as the butterfly
+// x += shfl_xor(x, 1), 2, 4, ... so the result is the same bit for bit.
+template <int N>
+__device__ __forceinline__ float group_sum(float x) {
+  if constexpr (N >= 2) x += butterfly_partner<1>(x);
+  if constexpr (N >= 4) x += butterfly_partner<2>(x);
+  if constexpr (N >= 8) x += butterfly_partner<4>(x);
+  if constexpr (N >= 16) x += butterfly_partner<8>(x);
+  if constexpr (N >= 32) x += __shfl_xor(x, 16, SOCKET_WAVE);
+  if constexpr (N >= 64) x += __shfl_xor(x, 32, SOCKET_WAVE);
+  return x;
+}
+
 // 16 bytes per lane from global memory straight into LDS: lane i's bytes land at
 // lds_dst + 16 * i (lds_dst is the same for the whole wave).  Written as assembly
 // so that the compiler does not serialise later LDS reads behind it; M0, which

@@ -89,6 +89,21 @@ __device__ __forceinline__ int wave_incl_scan(int v, int /*lane*/) {
   return v;
 }
 
+// Minimum and maximum over the 64 lanes, left in lane 63 (the same six steps as
+// the prefix sum; lanes a step does not reach take the identity).
+__device__ __forceinline__ void wave_minmax_to_last(uint32_t& kmin, uint32_t& kmax) {
+#define SOCKET_MINMAX_STEP(ctrl, rows)                                                                        \
+  kmin = min(kmin, (uint32_t)__builtin_amdgcn_update_dpp((int)0xffffffffu, (int)kmin, ctrl, rows, 0xf, false)); \
+  kmax = max(kmax, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)kmax, ctrl, rows, 0xf, false));
+  SOCKET_MINMAX_STEP(0x111, 0xf)   // row_shr:1
+  SOCKET_MINMAX_STEP(0x112, 0xf)   // row_shr:2
+  SOCKET_MINMAX_STEP(0x114, 0xf)   // row_shr:4
+  SOCKET_MINMAX_STEP(0x118, 0xf)   // row_shr:8
+  SOCKET_MINMAX_STEP(0x142, 0xa)   // row_bcast:15 into rows 1 and 3
+  SOCKET_MINMAX_STEP(0x143, 0xc)   // row_bcast:31 into rows 2 and 3
+#undef SOCKET_MINMAX_STEP
+}
+
 __device__ __forceinline__ u64 shfl_xor_u64(u64 v, int mask) {
   const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, SOCKET_WAVE);
   const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, SOCKET_WAVE);
@@ -183,7 +198,7 @@ __device__ __forceinline__ void wave_append(bool take, u64 value, int* cursor, u
   const int leader = __ffsll((long long)mask) - 1;
   int base = 0;
   if (lane == leader) base = atomicAdd(cursor, __popcll(mask));
-  base = __shfl(base, leader, SOCKET_WAVE);
+  base = __builtin_amdgcn_readlane(base, leader);   // (leader is wave-uniform: a scalar read, no LDS crossbar)
   if (take) {
     const int p = base + __popcll(mask & ((1ull << lane) - 1ull));
     if (p < cap) list[p] = value;
@@ -466,12 +481,8 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
       }
     }
   }
-#pragma unroll
-  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
-    kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
-    kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, SOCKET_WAVE));
-  }
-  if (lane == 0) {
+  wave_minmax_to_last(kmin, kmax);
+  if (lane == 63) {
     sh.wmin[wave] = kmin;
     sh.wmax[wave] = kmax;
   }
@@ -479,7 +490,9 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
   const int target = max(2 * m, 1024);
   const int r = (int)min((int64_t)nsample, ((int64_t)target * nsample + n - 1) / n);
   if (tid == 0) {
-    for (int w = 1; w < THREADS / SOCKET_WAVE; ++w) {
+    kmin = 0xffffffffu;
+    kmax = 0u;
+    for (int w = 0; w < THREADS / SOCKET_WAVE; ++w) {
       kmin = min(kmin, (uint32_t)sh.wmin[w]);
       kmax = max(kmax, (uint32_t)sh.wmax[w]);
     }
@@ -644,7 +657,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
           const int incl = wave_incl_scan(cnt, lane);
           int at = 0;
           if (lane == 63 && incl) at = atomicAdd(&sh.fill_pool, incl);
-          at = __shfl(at, 63, SOCKET_WAVE) + incl - cnt;
+          at = __builtin_amdgcn_readlane(at, 63) + incl - cnt;
           if (taken) {
 #pragma unroll
             for (int u = 0; u < kLoads; ++u) {
@@ -739,12 +752,8 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     if (total >= 0) {
       // range of the pooled composites, from their keys (the high halves): any range
       // that holds them all serves the refinement
-#pragma unroll
-      for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
-        kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
-        kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, SOCKET_WAVE));
-      }
-      if (lane == 0) {
+      wave_minmax_to_last(kmin, kmax);
+      if (lane == 63) {
         atomicMin(&sh.kmin, kmin);
         atomicMax(&sh.kmax, kmax);
       }
@@ -819,18 +828,16 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         kmax = max(kmax, k);
       });
     }
-#pragma unroll
-    for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
-      kmin = min(kmin, (uint32_t)__shfl_xor((int)kmin, d, SOCKET_WAVE));
-      kmax = max(kmax, (uint32_t)__shfl_xor((int)kmax, d, SOCKET_WAVE));
-    }
-    if (lane == 0) {
+    wave_minmax_to_last(kmin, kmax);
+    if (lane == 63) {
       sh.wmin[wave] = kmin;
       sh.wmax[wave] = kmax;
     }
     __syncthreads();
     if (tid == 0) {
-      for (int w = 1; w < kWaves; ++w) {
+      kmin = 0xffffffffu;
+      kmax = 0u;
+      for (int w = 0; w < kWaves; ++w) {
         kmin = min(kmin, (uint32_t)sh.wmin[w]);
         kmax = max(kmax, (uint32_t)sh.wmax[w]);
       }
