@@ -156,9 +156,8 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(
       ss += h * h;
     }
   }
-#pragma unroll
-  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) ss += __shfl_xor(ss, d, SOCKET_WAVE);
-  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  ss = wave_reduce_to_last<false>(ss);
+  if ((tid & 63) == 63) red[tid >> 6] = ss;
   __syncthreads();
   float tot = 0.f;
 #pragma unroll
@@ -260,15 +259,13 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_bf16_kernel(
       }
     }
   }
+  // (sums over the wave on the data-parallel-primitive path, left in the last lane)
 #pragma unroll
   for (int m = 0; m < M; ++m) {
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) {
-      acc[m] += __shfl_xor(acc[m], d, 64);
-      if (GATE) accg[m] += __shfl_xor(accg[m], d, 64);
-    }
+    acc[m] = wave_reduce_to_last<false>(acc[m]);
+    if (GATE) accg[m] = wave_reduce_to_last<false>(accg[m]);
   }
-  if (lane == 0) {
+  if (lane == 63) {
 #pragma unroll
     for (int m = 0; m < M; ++m) {
       float r = acc[m];

@@ -160,6 +160,28 @@ __device__ __forceinline__ float group_sum(float x) {
   return x;
 }
 
+// Sum (or maximum) of x over the 64 lanes, left in lane 63: four shifts inside
+// each row of 16 lanes, then the last lane of a row is folded into the row after
+// it and the lower half's last lane into the upper half; lanes a step does not
+// reach take the identity.
+template <bool MAX>
+__device__ __forceinline__ float wave_reduce_to_last(float x) {
+  const int ident = __float_as_int(MAX ? -INFINITY : 0.f);
+#define SOCKET_REDUCE_STEP(ctrl, rows)                                                                       \
+  {                                                                                                          \
+    const float o = __int_as_float(__builtin_amdgcn_update_dpp(ident, __float_as_int(x), ctrl, rows, 0xf, false)); \
+    x = MAX ? fmaxf(x, o) : x + o;                                                                           \
+  }
+  SOCKET_REDUCE_STEP(0x111, 0xf)   // row_shr:1
+  SOCKET_REDUCE_STEP(0x112, 0xf)   // row_shr:2
+  SOCKET_REDUCE_STEP(0x114, 0xf)   // row_shr:4
+  SOCKET_REDUCE_STEP(0x118, 0xf)   // row_shr:8
+  SOCKET_REDUCE_STEP(0x142, 0xa)   // row_bcast:15 into rows 1 and 3
+  SOCKET_REDUCE_STEP(0x143, 0xc)   // row_bcast:31 into rows 2 and 3
+#undef SOCKET_REDUCE_STEP
+  return x;
+}
+
 // 16 bytes per lane from global memory straight into LDS: lane i's bytes land at
 // lds_dst + 16 * i (lds_dst is the same for the whole wave).  Written as assembly
 // so that the compiler does not serialise later LDS reads behind it; M0, which

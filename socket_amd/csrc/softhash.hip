@@ -229,8 +229,7 @@ __device__ __forceinline__ void soft_hash_block(
 #pragma unroll 8
       for (int d = part; d < D; d += 4) s += qrow[d] * prow[d];
     }
-    s += __shfl_xor(s, 1, SOCKET_WAVE);
-    s += __shfl_xor(s, 2, SOCKET_WAVE);
+    s = group_sum<4>(s);
     if (p < G * K && part == 0) ts[p] = tanhf(s) * tanh_scale * inv_temperature;   // ts[g][k], p = g*K + k
   }
   __syncthreads();
@@ -297,15 +296,9 @@ __device__ __forceinline__ void soft_hash_block(
   // workgroup-wide reduction of one value per head; every lane gets the result
   auto reduce = [&](float (&v)[GC], bool is_max) {
 #pragma unroll
-    for (int g = 0; g < GC; ++g) {
-#pragma unroll
-      for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) {
-        const float o = __shfl_xor(v[g], d, SOCKET_WAVE);
-        v[g] = is_max ? fmaxf(v[g], o) : v[g] + o;
-      }
-    }
+    for (int g = 0; g < GC; ++g) v[g] = is_max ? wave_reduce_to_last<true>(v[g]) : wave_reduce_to_last<false>(v[g]);
     __syncthreads();  // earlier readers of `red` are done
-    if (lane == 0) {
+    if (lane == 63) {   // (the reduction leaves a wave's result in its last lane)
 #pragma unroll
       for (int g = 0; g < GC; ++g) red[wave * GC + g] = v[g];
     }
