@@ -99,11 +99,14 @@ __device__ __forceinline__ void finish_split(float (&m)[GH], float (&l)[GH], flo
   for (int d = LPR; d < SOCKET_WAVE; d <<= 1) {
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
-      const float m2 = __shfl_xor(m[g], d, SOCKET_WAVE);
-      const float l2 = __shfl_xor(l[g], d, SOCKET_WAVE);
+      auto partner = [&](float x) {
+        return d == 16 ? lane_xor16(x) : d == 32 ? lane_xor32(x) : __shfl_xor(x, d, SOCKET_WAVE);
+      };
+      const float m2 = partner(m[g]);
+      const float l2 = partner(l[g]);
       float a2[E];
 #pragma unroll
-      for (int i = 0; i < E; ++i) a2[i] = __shfl_xor(acc[g][i], d, SOCKET_WAVE);
+      for (int i = 0; i < E; ++i) a2[i] = partner(acc[g][i]);
       merge_state<E>(m[g], l[g], acc[g], m2, l2, a2);
     }
   }
@@ -678,8 +681,8 @@ __global__ __launch_bounds__(kAttThreads) void dense_mma_kernel(
       sc[i] = (key0 + i < hi) ? sc[i] : -INFINITY;
       m_blk = fmaxf(m_blk, sc[i]);
     }
-    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, SOCKET_WAVE));
-    m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, SOCKET_WAVE));
+    m_blk = fmaxf(m_blk, lane_xor16(m_blk));   // (lane swaps on the vector ALU, not the LDS crossbar)
+    m_blk = fmaxf(m_blk, lane_xor32(m_blk));
     // The maximum is kept on the raw dot products and the (positive) scale applied
     // to the difference, in base 2: the largest score of a block then gives exactly
     // exp2(0) whatever its magnitude, which scaling first and subtracting the rounded
@@ -728,8 +731,8 @@ __global__ __launch_bounds__(kAttThreads) void dense_mma_kernel(
   // before the ring is reused for the waves' records
   wait_copies<0>();
   float l = l_part;
-  l += __shfl_xor(l, 16, SOCKET_WAVE);
-  l += __shfl_xor(l, 32, SOCKET_WAVE);
+  l += lane_xor16(l);
+  l += lane_xor32(l);
   __syncthreads();
   constexpr int REC = D + 2;
   float* lds = reinterpret_cast<float*>(att_lds);

@@ -75,18 +75,6 @@ __device__ __forceinline__ uint4 load_frag8<DType_f16>(const uint16_t* p) {
   return r;
 }
 
-// v of lane x ^ 16 / x ^ 32, without the LDS crossbar: v_permlane16_swap exchanges
-// the odd 16-lane rows of its first operand with the even rows of its second,
-// v_permlane32_swap the upper half of the first with the lower half of the second.
-__device__ __forceinline__ uint32_t lane_xor16(uint32_t v, bool odd_row) {
-  const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
-  return odd_row ? r[0] : r[1];
-}
-__device__ __forceinline__ uint32_t lane_xor32(uint32_t v, bool upper_half) {
-  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
-  return upper_half ? r[0] : r[1];
-}
-
 // A cache position handed over on the device (per-sequence positions) is not
 // checked by the host: rows that would land outside [0, Tcap) are dropped.
 __device__ __forceinline__ bool in_cache(int pos, int64_t Tcap) { return (uint64_t)(int64_t)pos < (uint64_t)Tcap; }

@@ -131,6 +131,24 @@ __device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s
   im = cc + d;
 }
 
+// v of lane x ^ 16 / x ^ 32, without the LDS crossbar: v_permlane16_swap exchanges
+// the odd 16-lane rows of its first operand with the even rows of its second,
+// v_permlane32_swap the upper half of the first with the lower half of the second.
+__device__ __forceinline__ uint32_t lane_xor16(uint32_t v, bool odd_row) {
+  const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return odd_row ? r[0] : r[1];
+}
+__device__ __forceinline__ uint32_t lane_xor32(uint32_t v, bool upper_half) {
+  const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return upper_half ? r[0] : r[1];
+}
+__device__ __forceinline__ float lane_xor16(float v) {
+  return __uint_as_float(lane_xor16(__float_as_uint(v), (threadIdx.x >> 4) & 1));
+}
+__device__ __forceinline__ float lane_xor32(float v) {
+  return __uint_as_float(lane_xor32(__float_as_uint(v), (threadIdx.x >> 5) & 1));
+}
+
 // Step MASK (1, 2, 4 or 8) of a butterfly sum over lanes: the value a lane adds to
 // its own.  After the steps below MASK every lane of an aligned group of MASK
 // lanes holds the same value, so any lane of the partner group serves, and the
@@ -155,8 +173,8 @@ __device__ __forceinline__ float group_sum(float x) {
   if constexpr (N >= 4) x += butterfly_partner<2>(x);
   if constexpr (N >= 8) x += butterfly_partner<4>(x);
   if constexpr (N >= 16) x += butterfly_partner<8>(x);
-  if constexpr (N >= 32) x += __shfl_xor(x, 16, SOCKET_WAVE);
-  if constexpr (N >= 64) x += __shfl_xor(x, 32, SOCKET_WAVE);
+  if constexpr (N >= 32) x += lane_xor16(x);
+  if constexpr (N >= 64) x += lane_xor32(x);
   return x;
 }
 
