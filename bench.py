@@ -449,13 +449,19 @@ def timed_graph_steps(step_fn, steps, warmup, eager=False):
             run()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
         e0.record()
         for _ in range(calls):
             fn()
         e1.record()
+        # host clock between seeing the first event done and the second: the region is
+        # queued behind the settle phase's replays, which this must not count (and a
+        # synchronize before the region would idle the GPU the settle phase warmed)
+        e0.synchronize()
+        t0 = time.perf_counter()
+        e1.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / (calls * steps_per_call), (time.perf_counter() - t0) * 1e3
+        return e0.elapsed_time(e1) / (calls * steps_per_call), wall_ms
 
     # once from an idle GPU (reported beside the result), then after the settle phase
     torch.cuda.synchronize()
