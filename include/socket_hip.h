@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SOCKET_ABI_VERSION 2
+#define SOCKET_ABI_VERSION 3   /* 3: socket_select_list wants the head of its workspace zeroed; socket_decode_prologue */
 
 /* status codes */
 #define SOCKET_OK 0

@@ -112,7 +112,7 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.socket_abi_version() != 2:
+        if handle.socket_abi_version() != 3:
             raise RuntimeError("libsocket_hip.so ABI version mismatch; rebuild it")
         _lib = handle
     return _lib

@@ -40,7 +40,7 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_status_strings_and_version(lib):
-    assert lib.socket_abi_version() == 2
+    assert lib.socket_abi_version() == 3
     seen = set()
     for st in range(0, -7, -1):
         s = lib.socket_status_string(st).decode()
