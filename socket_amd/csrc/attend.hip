@@ -148,9 +148,8 @@ __device__ __forceinline__ void merge_splits(const float* mo, const float* ml, i
 
   float m = -INFINITY;
   for (int s = tid; s < nblk; s += kMergeThreads) m = fmaxf(m, COHERENT ? load_coherent(ml + s) : ml[s]);
-#pragma unroll
-  for (int d = SOCKET_WAVE / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, SOCKET_WAVE));
-  if (lane == 0) red[wave] = m;
+  m = wave_reduce_to_last<true>(m);
+  if (lane == 63) red[wave] = m;
   __syncthreads();
   m = red[0];
 #pragma unroll
@@ -584,12 +583,7 @@ __global__ __launch_bounds__(kAttThreads) void dense_mma_kernel(
   if (flat) {
     if (wave == 0) {
       const int n = lane < B ? (max(0, min(lens[lane], T)) + rows_per_split - 1) / rows_per_split : 0;
-      int incl = n;
-#pragma unroll
-      for (int d = 1; d < SOCKET_WAVE; d <<= 1) {
-        const int up = __shfl_up(incl, d, SOCKET_WAVE);
-        if (lane >= d) incl += up;
-      }
+      const int incl = wave_incl_scan(n);
       if (t >= incl - n && t < incl) {
         item[0] = lane;
         item[1] = t - (incl - n);

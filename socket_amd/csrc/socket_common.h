@@ -178,6 +178,20 @@ __device__ __forceinline__ float group_sum(float x) {
   return x;
 }
 
+// Inclusive prefix sum over the 64 lanes on the data-parallel-primitive path of the
+// vector ALU: four shifts inside each row of 16 lanes, then the last lane of row 0
+// (and 2) is added to the row after it and the last lane of the lower half to the
+// upper half.  (Six dependent LDS-crossbar shuffles took ~0.25 us per scan.)
+__device__ __forceinline__ int wave_incl_scan(int v, int /*lane*/ = 0) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Sum (or maximum) of x over the 64 lanes, left in lane 63: four shifts inside
 // each row of 16 lanes, then the last lane of a row is folded into the row after
 // it and the lower half's last lane into the upper half; lanes a step does not

@@ -75,20 +75,6 @@ __device__ __forceinline__ int32_t composite_index(u64 c) {
   return (int32_t)(0xffffffffu - (uint32_t)(c & 0xffffffffull));
 }
 
-// Inclusive prefix sum over the 64 lanes on the data-parallel-primitive path of the
-// vector ALU: four shifts inside each row of 16 lanes, then the last lane of row 0
-// (and 2) is added to the row after it and the last lane of the lower half to the
-// upper half.  (Six dependent LDS-crossbar shuffles took ~0.25 us per scan.)
-__device__ __forceinline__ int wave_incl_scan(int v, int /*lane*/) {
-  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
-  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
-  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
-  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
-  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 into rows 1 and 3
-  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 into rows 2 and 3
-  return v;
-}
-
 // Minimum and maximum over the 64 lanes, left in lane 63 (the same six steps as
 // the prefix sum; lanes a step does not reach take the identity).
 __device__ __forceinline__ void wave_minmax_to_last(uint32_t& kmin, uint32_t& kmax) {
