@@ -66,6 +66,7 @@ struct SelectShared {
   uint32_t kmin, kmax;  // key range of the pool
   int base;             // where this workgroup's entries go in the row's shared list
   int last;             // this workgroup is the last of its row to arrive
+  int crowded;          // a bin above the k-th holds more than kMaxBinForCounting entries
 };
 
 __device__ __forceinline__ u64 composite(uint32_t key, int idx) {
@@ -99,9 +100,13 @@ __device__ __forceinline__ u64 shfl_xor_u64(u64 v, int mask) {
 // All THREADS lanes.  Ranks the bins from the top (descending != 0) or from the
 // bottom, kBins / THREADS per lane, and publishes in `sh` the bin where the
 // running count first reaches `need`, the count ranked before it and its own.
-template <int THREADS>
-__device__ __forceinline__ void find_bin(const uint32_t* hist, int need, int descending,
-                                         SelectShared& sh, int tid) {
+// With OFFSETS every bin's counter is replaced by `entries ranked before the bin |
+// its own count << 16` (each lane rewrites the bins it read, nobody else's), and
+// sh.crowded is raised (never cleared here) when a bin ranked wholly before the
+// found one holds more than kMaxBinForCounting entries.
+template <int THREADS, bool OFFSETS = false>
+__device__ __forceinline__ void find_bin(uint32_t* hist, int need, int descending, SelectShared& sh,
+                                         int tid) {
   constexpr int PER = kBins / THREADS;
   const int lane = tid & 63, wave = tid >> 6;
   int c[PER], mine = 0;
@@ -127,6 +132,11 @@ __device__ __forceinline__ void find_bin(const uint32_t* hist, int need, int des
       sh.found_bin = descending ? (kBins - 1 - r) : r;
       sh.found_before = run;
       sh.found_count = c[i];
+    }
+    if constexpr (OFFSETS) {
+      const int r = tid * PER + i;
+      hist[descending ? (kBins - 1 - r) : r] = (uint32_t)run | ((uint32_t)c[i] << 16);
+      if (c[i] > kMaxBinForCounting && run + c[i] < need) sh.crowded = 1;
     }
     run += c[i];
   }
@@ -336,7 +346,7 @@ __device__ __forceinline__ int range_shift(u64 lo, u64 hi) {
 __device__ __forceinline__ void order_and_write(u64* buf, int n_above, u64* cand, int ncand, int need,
                                                 u64 lo0, int shift0, u64* tmp, uint32_t* hist,
                                                 SelectShared& sh, bool counting_ok, int32_t* out,
-                                                int tid) {
+                                                int tid, bool placed = false) {
   const int lane = tid & 63, wave = tid >> 6;
   // ---- the k-th bin: rank its entries, the best `need` follow the winners ----------
   if (ncand <= kMaxBinForCounting || need == ncand) {
@@ -356,6 +366,18 @@ __device__ __forceinline__ void order_and_write(u64* buf, int n_above, u64* cand
   if (n_above == 0) return;
 
   // ---- winners above the bin ----------------------------------------------------------
+  if (placed) {
+    // `buf` holds them grouped by level-0 bin already, hist[bin] = offset | population << 16
+    for (int p = tid; p < n_above; p += kThreads) {
+      const u64 v = buf[p];
+      const uint32_t h = hist[(int)((v - lo0) >> shift0)];
+      const int s0 = (int)(h & 0xffffu), c = (int)(h >> 16);
+      int r = 0;
+      for (int q = s0; q < s0 + c; ++q) r += buf[q] > v;
+      out[s0 + r] = composite_index(v);
+    }
+    return;
+  }
   if (counting_ok) {
     for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
     __syncthreads();
@@ -749,13 +771,62 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         sh.hi = ((u64)sh.kmax << 32) | 0xffffffffull;
         sh.need = m;
         sh.done = 0;
+        sh.crowded = 0;
       }
       __syncthreads();
       const u64 lo0 = sh.lo;
       const int shift0 = range_shift(sh.lo, sh.hi);
       // refinement on the composites; they are distinct, so it ends with a bin of
-      // at most kCandCap entries (ties need no special case here)
-      for (int iter = 0; iter < 8; ++iter) {
+      // at most kCandCap entries (ties need no special case here).
+      // The first pass covers every entry, and every entry keeps the slot that its
+      // bin's counter hands out.  When that pass already isolates the k-th bin (the
+      // usual case) the bins' counters, turned into offsets by the same scan that
+      // finds the bin, and those slots place every winner next to the others of its
+      // bin and the k-th bin's entries in their list with no further counting.
+      {
+        uint32_t slot2[U / 2];   // 16 bits per entry
+#pragma unroll
+        for (int u = 0; u < U / 2; ++u) slot2[u] = 0;
+        for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          if (tid + u * kThreads < total) {
+            const uint32_t sl = atomicAdd(&hist[(int)((pv[u] - lo0) >> shift0)], 1u);
+            slot2[u >> 1] |= sl << (16 * (u & 1));
+          }
+        }
+        __syncthreads();
+        find_bin<kThreads, true>(hist, m, 1, sh, tid);
+        if (tid == 0) {
+          const u64 hi = sh.hi;
+          const u64 blo = lo0 + ((u64)sh.found_bin << shift0);
+          const u64 bspan = (shift0 == 0) ? 0ull : ((1ull << shift0) - 1ull);
+          sh.lo = blo;
+          sh.hi = (hi - blo < bspan) ? hi : blo + bspan;
+          sh.need = m - sh.found_before;
+          sh.done = (sh.found_count <= kCandCap || shift0 == 0) ? 1 : 0;
+        }
+        __syncthreads();
+        if (sh.done && !sh.crowded) {
+          const int fb = sh.found_bin, need = sh.need, ncand = min(sh.found_count, kCandCap);
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            if (tid + u * kThreads < total) {
+              const u64 v = pv[u];
+              const int bin = (int)((v - lo0) >> shift0);
+              const int sl = (int)((slot2[u >> 1] >> (16 * (u & 1))) & 0xffffu);
+              if (bin > fb) buf[(int)(hist[bin] & 0xffffu) + sl] = v;
+              else if (bin == fb && sl < kCandCap) cand[sl] = v;
+            }
+          }
+          __syncthreads();
+          order_and_write(buf, m - need, cand, ncand, need, lo0, shift0, tmp, hist, sh, counting_ok != 0, heavy,
+                          tid, true);
+          return;
+        }
+      }
+      for (int iter = 1; iter < 8 && !sh.done; ++iter) {
         const u64 lo = sh.lo, hi = sh.hi;
         const int need_in = sh.need;
         const int shift = range_shift(lo, hi);
