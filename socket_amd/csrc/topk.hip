@@ -604,6 +604,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
       sh.fill_pool = 0;
       sh.kmin = 0xffffffffu;
       sh.kmax = 0u;
+      sh.crowded = 0;
     }
     int total = -1;  // uniform; stays -1 when no pool could be formed
     uint32_t kmin = 0xffffffffu, kmax = 0u;  // key range of what this lane holds
@@ -622,6 +623,8 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         pv[u] = composite(k, i);
       }
       total = n;
+      for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;   // for the first refinement pass
+      __syncthreads();
     } else if (sampling_ok(m)) {
       // This part's share of the row; the last part also takes the one to three
       // scores past the last multiple of four.
@@ -684,6 +687,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         fetch(begin, b0);
         fetch(begin + kStep, b1);
         const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
+        for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;   // for the first refinement pass
         const float tau_f = tau >= 0xff800000u ? INFINITY : tau <= 0x007fffffu ? -INFINITY
                             : __uint_as_float((tau & 0x80000000u) ? (tau & 0x7fffffffu) : ~tau);
         for (int base = begin; base < e4; base += 3 * kStep) {
@@ -701,6 +705,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         }
       } else {
         const uint32_t tau = sample_threshold<kThreads, VEC>(row, n, m, hist, sh, tid);
+        for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;   // for the first refinement pass
         for_each_in<VEC, kThreads>(row, begin, tail_end, tid, [&](int i, float x) {
           wave_append(score_to_key(x) >= tau, composite(__float_as_uint(x), i), &sh.fill_pool, pool, kPoolCap);
         });
@@ -756,7 +761,6 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
     } else if (part != 0) {
       return;   // no threshold can be relied on: one workgroup selects from scratch
     }
-    __syncthreads();
     if (total >= 0) {
       // range of the pooled composites, from their keys (the high halves): any range
       // that holds them all serves the refinement
@@ -766,16 +770,8 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         atomicMax(&sh.kmax, kmax);
       }
       __syncthreads();
-      if (tid == 0) {
-        sh.lo = (u64)sh.kmin << 32;
-        sh.hi = ((u64)sh.kmax << 32) | 0xffffffffull;
-        sh.need = m;
-        sh.done = 0;
-        sh.crowded = 0;
-      }
-      __syncthreads();
-      const u64 lo0 = sh.lo;
-      const int shift0 = range_shift(sh.lo, sh.hi);
+      const u64 lo0 = (u64)sh.kmin << 32, hi0 = ((u64)sh.kmax << 32) | 0xffffffffull;
+      const int shift0 = range_shift(lo0, hi0);
       // refinement on the composites; they are distinct, so it ends with a bin of
       // at most kCandCap entries (ties need no special case here).
       // The first pass covers every entry, and every entry keeps the slot that its
@@ -786,9 +782,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
       {
         uint32_t slot2[U / 2];   // 16 bits per entry
 #pragma unroll
-        for (int u = 0; u < U / 2; ++u) slot2[u] = 0;
-        for (int i = tid; i < kBins; i += kThreads) hist[i] = 0;
-        __syncthreads();
+        for (int u = 0; u < U / 2; ++u) slot2[u] = 0;   // (hist is zero: cleared ahead of the pool)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           if (tid + u * kThreads < total) {
@@ -799,7 +793,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         __syncthreads();
         find_bin<kThreads, true>(hist, m, 1, sh, tid);
         if (tid == 0) {
-          const u64 hi = sh.hi;
+          const u64 hi = hi0;
           const u64 blo = lo0 + ((u64)sh.found_bin << shift0);
           const u64 bspan = (shift0 == 0) ? 0ull : ((1ull << shift0) - 1ull);
           sh.lo = blo;
