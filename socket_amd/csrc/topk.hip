@@ -52,6 +52,11 @@ constexpr int kMaxParts = 16;          // workgroups that share one row at most
 
 typedef unsigned long long u64;
 
+template <bool B>
+struct BoolTag {
+  static constexpr bool value = B;
+};
+
 struct SelectShared {
   u64 lo, hi;           // current key / composite range (inclusive)
   int need;             // winners still to take from inside [lo, hi]
@@ -447,7 +452,8 @@ __host__ __device__ __forceinline__ bool sampling_ok(int m) {
 // places, 4096 scores in all (16384 for rows beyond 262144) -- whose r-th largest
 // key is located with the same histogram refinement as everywhere else; tau is
 // the lower edge of its bin.  Every workgroup that calls this for a row gets the
-// same tau.  Needs n > kPoolCap.  Ends with a barrier.
+// same tau.  Needs n > kPoolCap; clears hist itself (nobody may be using it).  When
+// it returns every lane has passed the barrier that follows the last read of hist.
 template <int THREADS, bool VEC>
 __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, int m, uint32_t* hist,
                                                      SelectShared& sh, int tid) {
@@ -457,6 +463,7 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
   const int nchunk = nsample / 64;
   const int nq = nsample / 4 / THREADS;  // 1 or 4 (1024 lanes), 4 or 16 (256 lanes)
   uint32_t key[kMaxQ * 4];
+  for (int i = tid; i < kBins; i += THREADS) hist[i] = 0;   // (no one uses hist before this call)
 #pragma unroll
   for (int j = 0; j < kMaxQ; ++j) {
     if (j < nq) {
@@ -494,29 +501,26 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
     sh.wmin[wave] = kmin;
     sh.wmax[wave] = kmax;
   }
-  __syncthreads();
+  __syncthreads();   // (also: hist is zero everywhere)
+  // every wave reduces the waves' extremes for itself
+  kmin = (uint32_t)sh.wmin[lane & (THREADS / SOCKET_WAVE - 1)];
+  kmax = (uint32_t)sh.wmax[lane & (THREADS / SOCKET_WAVE - 1)];
+  wave_minmax_to_last(kmin, kmax);
+  const uint32_t smin = (uint32_t)__builtin_amdgcn_readlane((int)kmin, 63);
+  const uint32_t smax = max(smin, (uint32_t)__builtin_amdgcn_readlane((int)kmax, 63));
   const int target = max(2 * m, 1024);
   const int r = (int)min((int64_t)nsample, ((int64_t)target * nsample + n - 1) / n);
-  if (tid == 0) {
-    kmin = 0xffffffffu;
-    kmax = 0u;
-    for (int w = 0; w < THREADS / SOCKET_WAVE; ++w) {
-      kmin = min(kmin, (uint32_t)sh.wmin[w]);
-      kmax = max(kmax, (uint32_t)sh.wmax[w]);
-    }
-    sh.lo = kmin;
-    sh.hi = max(kmin, kmax);
-    sh.need = r;
-    sh.done = 0;
-  }
-  __syncthreads();
   const int fine = max(4, r / 8);  // a bin this small pins tau well enough
   for (int iter = 0; iter < 4; ++iter) {
-    const uint32_t lo = (uint32_t)sh.lo, hi = (uint32_t)sh.hi;
-    const int need_in = sh.need;
+    // the first pass takes its range from the sample's extremes, the later ones from
+    // what the pass before published
+    const uint32_t lo = iter ? (uint32_t)sh.lo : smin, hi = iter ? (uint32_t)sh.hi : smax;
+    const int need_in = iter ? sh.need : r;
     const int shift = range_shift(lo, hi);
-    for (int i = tid; i < kBins; i += THREADS) hist[i] = 0;
-    __syncthreads();
+    if (iter) {
+      for (int i = tid; i < kBins; i += THREADS) hist[i] = 0;
+      __syncthreads();
+    }
 #pragma unroll
     for (int j = 0; j < kMaxQ; ++j) {
       if (j < nq) {
@@ -540,9 +544,7 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
     __syncthreads();
     if (sh.done) break;
   }
-  const uint32_t tau = (uint32_t)sh.lo;
-  __syncthreads();
-  return tau;
+  return (uint32_t)sh.lo;
 }
 
 // ---------------------------------------------------------------------------
@@ -649,39 +651,56 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
             x[u] = *reinterpret_cast<const float4*>(row + i0);
           }
         };
-        // What passes in one batch of one lane, as a bit per score.  The test is made
-        // on the floats (one compare per score; keys only for the pool): x passes
-        // when it is not below the float whose key is tau.  A tau above +inf's key or
-        // below -inf's is no float's key and is widened to that infinity (the pool
-        // only has to hold everything at or above tau; more is allowed).
-        auto filter = [&](int base, const float4 (&x)[kLoads], float tau_f) {
-          if (base >= e4) return;  // uniform
-          uint32_t taken = 0;      // bit u * 4 + c: score c of load u passes
+        // One batch of one wave.  Each of a lane's 16 scores is tested on the float (one
+        // compare per score; keys only for the pool): x passes when it is not below the
+        // float whose key is tau.  A tau above +inf's key or below -inf's is no float's
+        // key and is widened to that infinity (the pool only has to hold everything at
+        // or above tau; more is allowed).  A compare leaves a wave-wide mask in scalar
+        // registers; the 16 masks' population is the stretch of the pool that one LDS
+        // atomic reserves for the wave, and an entry's place in it is the count of its
+        // mask's bits below its lane, on top of a scalar running base -- no per-lane
+        // bookkeeping, no cross-lane traffic.  A batch that would run past the pool is
+        // counted but not written (the row is then redone from scratch anyway).
+        auto filter_batch = [&](auto full, int base, const float4 (&x)[kLoads], float tau_f) {
+          constexpr bool FULL = decltype(full)::value;   // every lane's 16 scores are inside the share
+          int total = 0;
+          u64 mask[kLoads * 4];   // (scalar registers)
 #pragma unroll
           for (int u = 0; u < kLoads; ++u) {
             const float xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
-            const bool in = base + (u * kThreads + tid) * 4 < e4;
+            const bool in = FULL || base + (u * kThreads + tid) * 4 < e4;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) taken |= (in && !(xs[c] < tau_f)) ? (1u << (u * 4 + c)) : 0u;
-          }
-          const int cnt = __popc(taken);
-          const int incl = wave_incl_scan(cnt, lane);
-          int at = 0;
-          if (lane == 63 && incl) at = atomicAdd(&sh.fill_pool, incl);
-          at = __builtin_amdgcn_readlane(at, 63) + incl - cnt;
-          if (taken) {
-#pragma unroll
-            for (int u = 0; u < kLoads; ++u) {
-              const float xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
-#pragma unroll
-              for (int c = 0; c < 4; ++c) {
-                if (taken & (1u << (u * 4 + c))) {   // (the score as it is: keys are made afterwards)
-                  if (at < kPoolCap) pool[at] = composite(__float_as_uint(xs[c]), base + (u * kThreads + tid) * 4 + c);
-                  ++at;
-                }
-              }
+            for (int c = 0; c < 4; ++c) {
+              mask[u * 4 + c] = __builtin_amdgcn_ballot_w64(in && !(xs[c] < tau_f));
+              total += __popcll(mask[u * 4 + c]);
             }
           }
+          if (total == 0) return;  // uniform
+          int at = 0;
+          if (lane == 0) at = atomicAdd(&sh.fill_pool, total);
+          at = __builtin_amdgcn_readfirstlane(at);
+          if (at + total > kPoolCap) return;  // uniform
+          const uint32_t cidx = 0xffffffffu - (uint32_t)(base + tid * 4);
+#pragma unroll
+          for (int u = 0; u < kLoads; ++u) {
+            const float xs[4] = {x[u].x, x[u].y, x[u].z, x[u].w};
+            const bool in = FULL || base + (u * kThreads + tid) * 4 < e4;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              const bool pass = in && !(xs[c] < tau_f);
+              const u64 mk = mask[u * 4 + c];
+              const int slot = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mk >> 32),
+                                                               __builtin_amdgcn_mbcnt_lo((uint32_t)mk, (uint32_t)at));
+              if (pass)
+                pool[slot] = ((u64)__float_as_uint(xs[c]) << 32) | (u64)(cidx - (uint32_t)(u * kThreads * 4 + c));
+              at += __popcll(mk);
+            }
+          }
+        };
+        auto filter = [&](int base, const float4 (&x)[kLoads], float tau_f) {
+          if (base >= e4) return;  // uniform
+          if (base + kStep <= e4) filter_batch(BoolTag<true>{}, base, x, tau_f);
+          else filter_batch(BoolTag<false>{}, base, x, tau_f);
         };
         float4 b0[kLoads], b1[kLoads], b2[kLoads];
         fetch(begin, b0);
