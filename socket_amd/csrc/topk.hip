@@ -109,9 +109,14 @@ __device__ __forceinline__ u64 shfl_xor_u64(u64 v, int mask) {
 // its own count << 16` (each lane rewrites the bins it read, nobody else's), and
 // sh.crowded is raised (never cleared here) when a bin ranked wholly before the
 // found one holds more than kMaxBinForCounting entries.
-template <int THREADS, bool OFFSETS = false>
+// `on_found(bin, ranked before it, its count)` runs in the one lane that finds the
+// bin, before the closing barrier: what it writes to `sh` every lane sees afterwards.
+struct NoFoundAction {
+  __device__ void operator()(int, int, int) const {}
+};
+template <int THREADS, bool OFFSETS = false, class F = NoFoundAction>
 __device__ __forceinline__ void find_bin(uint32_t* hist, int need, int descending, SelectShared& sh,
-                                         int tid) {
+                                         int tid, F&& on_found = F()) {
   constexpr int PER = kBins / THREADS;
   const int lane = tid & 63, wave = tid >> 6;
   int c[PER], mine = 0;
@@ -137,6 +142,7 @@ __device__ __forceinline__ void find_bin(uint32_t* hist, int need, int descendin
       sh.found_bin = descending ? (kBins - 1 - r) : r;
       sh.found_before = run;
       sh.found_count = c[i];
+      on_found(descending ? (kBins - 1 - r) : r, run, c[i]);
     }
     if constexpr (OFFSETS) {
       const int r = tid * PER + i;
@@ -532,16 +538,14 @@ __device__ __forceinline__ uint32_t sample_threshold(const float* row, int n, in
       }
     }
     __syncthreads();
-    find_bin<THREADS>(hist, need_in, 1, sh, tid);
-    if (tid == 0) {
-      const uint32_t blo = lo + ((uint32_t)sh.found_bin << shift);
+    find_bin<THREADS>(hist, need_in, 1, sh, tid, [&](int bin, int before, int count) {
+      const uint32_t blo = lo + ((uint32_t)bin << shift);
       const uint32_t bspan = (shift == 0) ? 0u : ((1u << shift) - 1u);
       sh.lo = blo;
       sh.hi = (hi - blo < bspan) ? hi : blo + bspan;
-      sh.need = need_in - sh.found_before;
-      sh.done = (sh.found_count <= fine || shift == 0) ? 1 : 0;
-    }
-    __syncthreads();
+      sh.need = need_in - before;
+      sh.done = (count <= fine || shift == 0) ? 1 : 0;
+    });
     if (sh.done) break;
   }
   return (uint32_t)sh.lo;
@@ -810,17 +814,14 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
           }
         }
         __syncthreads();
-        find_bin<kThreads, true>(hist, m, 1, sh, tid);
-        if (tid == 0) {
-          const u64 hi = hi0;
-          const u64 blo = lo0 + ((u64)sh.found_bin << shift0);
+        find_bin<kThreads, true>(hist, m, 1, sh, tid, [&](int bin, int before, int count) {
+          const u64 blo = lo0 + ((u64)bin << shift0);
           const u64 bspan = (shift0 == 0) ? 0ull : ((1ull << shift0) - 1ull);
           sh.lo = blo;
-          sh.hi = (hi - blo < bspan) ? hi : blo + bspan;
-          sh.need = m - sh.found_before;
-          sh.done = (sh.found_count <= kCandCap || shift0 == 0) ? 1 : 0;
-        }
-        __syncthreads();
+          sh.hi = (hi0 - blo < bspan) ? hi0 : blo + bspan;
+          sh.need = m - before;
+          sh.done = (count <= kCandCap || shift0 == 0) ? 1 : 0;
+        });
         if (sh.done && !sh.crowded) {
           const int fb = sh.found_bin, need = sh.need, ncand = min(sh.found_count, kCandCap);
 #pragma unroll
