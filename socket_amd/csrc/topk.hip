@@ -34,7 +34,11 @@
 // histogram bins already order them coarsely and a bin seldom holds more than a
 // few, so each winner goes to (#winners in higher bins) + (#bin-mates beating
 // it); crowded bins fall back to an in-LDS bitonic sort whose short exchange
-// distances stay in registers and wave shuffles.
+// distances stay in registers and wave shuffles.  In the pooled path the first
+// refinement pass is that level-0 histogram: every entry keeps the slot its
+// bin's counter handed it, the scan that finds the m-th bin turns the counters
+// into offsets, and when that one pass isolates the bin (the usual case) the
+// winners are grouped by bin with no second count.
 #include "socket_common.h"
 
 
