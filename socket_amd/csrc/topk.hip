@@ -699,8 +699,14 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
               const u64 mk = mask[u * 4 + c];
               const int slot = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mk >> 32),
                                                                __builtin_amdgcn_mbcnt_lo((uint32_t)mk, (uint32_t)at));
-              if (pass)
-                pool[slot] = ((u64)__float_as_uint(xs[c]) << 32) | (u64)(cidx - (uint32_t)(u * kThreads * 4 + c));
+              if (pass) {
+                // the two halves of the entry from wherever they are, in one write
+                // (a 64-bit store would first copy them into a register pair)
+                const uint32_t addr = (uint32_t)(uintptr_t)(pool + slot);
+                asm volatile("ds_write2_b32 %0, %1, %2 offset1:1"
+                             :: "v"(addr), "v"(cidx - (uint32_t)(u * kThreads * 4 + c)), "v"(__float_as_uint(xs[c]))
+                             : "memory");
+              }
               at += __popcll(mk);
             }
           }
@@ -725,6 +731,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
           fetch(base + 4 * kStep, b1);
           filter(base + 2 * kStep, b2, tau_f);
         }
+        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the pool writes above are not the compiler's to wait for
         if (wave == 0) {
           const int i = e4 + lane;
           const float x = i < tail_end ? row[i] : 0.f;
