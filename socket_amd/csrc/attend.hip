@@ -645,8 +645,8 @@ __global__ __launch_bounds__(kAttThreads) void dense_mma_kernel(
       const int r = 4 * i + quarter;
       const int key = min(key0 + r, hi - 1);
       const int piece = prow ^ r;
-      lds_dma16(kbase + (int64_t)key * k_ss + piece * 8, dst + i * 1024);
-      lds_dma16(vbase + (int64_t)key * v_ss + piece * 8, dst + kMmaTileBytes + i * 1024);
+      lds_dma16_stream(kbase + (int64_t)key * k_ss + piece * 8, dst + i * 1024);
+      lds_dma16_stream(vbase + (int64_t)key * v_ss + piece * 8, dst + kMmaTileBytes + i * 1024);
     }
   };
 

@@ -394,8 +394,8 @@ __global__ __launch_bounds__(kHashThreads) __attribute__((amdgpu_waves_per_eu(2,
       const int row = 4 * p + quarter;
       const int srow = min(s0 + row, S - 1);  // rows past the end re-read the last one; never stored
       const int chunk = prow ^ (row & 15);
-      lds_dma16(kbase + (int64_t)srow * k_ss + chunk * 8, dst + p * 1024);
-      if (with_values) lds_dma16(vbase + (int64_t)srow * v_ss + chunk * 8, dst + kStreamTileBytes + p * 1024);
+      lds_dma16_stream(kbase + (int64_t)srow * k_ss + chunk * 8, dst + p * 1024);
+      if (with_values) lds_dma16_stream(vbase + (int64_t)srow * v_ss + chunk * 8, dst + kStreamTileBytes + p * 1024);
     }
   };
 

@@ -232,6 +232,22 @@ __device__ __forceinline__ void lds_dma16(const void* src_lane, void* lds_dst) {
       : "v"(src_lane), "s"(base)
       : "memory");
 }
+// The same copy with the streaming hint: data that is read once and should not
+// displace what the caches hold.
+__device__ __forceinline__ void lds_dma16_stream(const void* src_lane, void* lds_dst) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_dst);
+  uint32_t saved;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %1, off nt\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved)
+      : "v"(src_lane), "s"(base)
+      : "memory");
+}
 
 // s_waitcnt vmcnt(n) only (n <= 15 here; larger requests wait for 15)
 __device__ __forceinline__ void wait_vmcnt(int n) {

@@ -656,7 +656,9 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
             // (past the end: the share's last four, fetched and ignored -- a load under
             // a condition would make every wait in the loop a wait for all loads)
             const int i0 = max(min(base + (u * kThreads + tid) * 4, e4 - 4), 0);
-            x[u] = *reinterpret_cast<const float4*>(row + i0);
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(row + i0));
+            x[u] = make_float4(v.x, v.y, v.z, v.w);
           }
         };
         // One batch of one wave.  Each of a lane's 16 scores is tested on the float (one
