@@ -36,7 +36,9 @@ __device__ __forceinline__ float entry_to_f32(uint16_t x) { return f16_bits_to_f
 // wait in `out` between slices (each thread re-reads what it wrote itself), which
 // costs 8 bytes per token and slice against the 2 L + 9 of the stream and keeps
 // the order of the fp32 adds.
-template <typename QT, int THREADS, bool VEC, bool INLDS>
+// STREAM: the codes are loaded with the streaming hint (a code array too large to
+// stay in the memory-side cache from one call to the next; VEC only).
+template <typename QT, int THREADS, bool VEC, bool INLDS, bool STREAM>
 __global__ __launch_bounds__(THREADS) void collision_i16_kernel(
     const QT* __restrict__ q_probs, const int16_t* __restrict__ key_buckets,
     const uint8_t* __restrict__ allowed, const QT* __restrict__ v_hist, float* __restrict__ out,
@@ -51,7 +53,12 @@ __global__ __launch_bounds__(THREADS) void collision_i16_kernel(
   // the eight codes of a thread's tokens for table l, as loaded (two per word; -1 where no token is)
   auto codes_of = [&](int l, int t0) -> uint4 {
     const int16_t* row = kb + (int64_t)l * T + t0;
-    if (VEC) return *reinterpret_cast<const uint4*>(row);
+    if (VEC && !STREAM) return *reinterpret_cast<const uint4*>(row);
+    if (VEC) {
+      typedef uint32_t u32x4_stream __attribute__((ext_vector_type(4)));
+      const u32x4_stream v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_stream*>(row));
+      return make_uint4(v.x, v.y, v.z, v.w);
+    }
     uint32_t u[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -201,9 +208,11 @@ int launch_collision_i16(const QT* q_probs, const int16_t* key_buckets, const ui
   chunks = chunks < 1 ? 1 : chunks > 8 ? 8 : chunks;
   if (chunks > tiles) chunks = tiles;
   dim3 grid((tiles + chunks - 1) / chunks, B * H);
-#define SOCKET_COLLIDE(TH, V, LD)                                                                       \
+  // (measured: 2 GB of codes gain 10 % from the hint, 135 MB that the cache still holds from the last call lose 7 %)
+  const bool stream_codes = (int64_t)B * H * L * T * (int64_t)sizeof(int16_t) > (192ll << 20);
+#define SOCKET_COLLIDE(TH, V, LD, ST)                                                                     \
   do {                                                                                                \
-    auto kern = collision_i16_kernel<QT, TH, V, LD>;                                                     \
+    auto kern = collision_i16_kernel<QT, TH, V, LD, ST>;                                                 \
     if (lds > 64 * 1024) {                                                                            \
       static std::atomic<size_t> granted{0};                                                          \
       if (granted.load(std::memory_order_acquire) < lds) {                                            \
@@ -217,8 +226,9 @@ int launch_collision_i16(const QT* q_probs, const int16_t* key_buckets, const ui
   } while (0)
 #define SOCKET_COLLIDE_V(TH, LD)         \
   do {                                   \
-    if (vec) SOCKET_COLLIDE(TH, true, LD); \
-    else SOCKET_COLLIDE(TH, false, LD);  \
+    if (vec && stream_codes) SOCKET_COLLIDE(TH, true, LD, true); \
+    else if (vec) SOCKET_COLLIDE(TH, true, LD, false); \
+    else SOCKET_COLLIDE(TH, false, LD, false);  \
   } while (0)
   if (ct > 0) {
     if (small) SOCKET_COLLIDE_V(256, true);
