@@ -292,6 +292,14 @@ __device__ __forceinline__ void score_tile(
     tsafe[j] = live[j] ? tbase[j] : tile * TW;
   }
 
+  // The value norms of the lane's tokens are requested now and used in the epilogue:
+  // asked for there, every tile would end on one exposed memory latency with nothing
+  // else on the CU to cover it.
+  const uint16_t* vn_pair = v_norm + (int64_t)pair * Tcap;
+  uint2 vn_raw[KT4];
+#pragma unroll
+  for (int j = 0; j < KT4; ++j) vn_raw[j] = *reinterpret_cast<const uint2*>(vn_pair + tsafe[j]);
+
   float acc[KT4][4][GP];
 #pragma unroll
   for (int j = 0; j < KT4; ++j)
@@ -645,7 +653,6 @@ __device__ __forceinline__ void score_tile(
 
   // epilogue: multiply by the value norm, mask, store one float4 per head; on
   // request also the tile's range of score keys per head, for the select kernel
-  const uint16_t* vn_pair = v_norm + (int64_t)pair * Tcap;
   uint32_t kmin[GP], kmax[GP];
 #pragma unroll
   for (int g = 0; g < GP; ++g) {
@@ -655,7 +662,7 @@ __device__ __forceinline__ void score_tile(
 #pragma unroll
   for (int j = 0; j < KT4; ++j) {
     if (!live[j]) continue;
-    const uint2 vraw = *reinterpret_cast<const uint2*>(vn_pair + tbase[j]);
+    const uint2 vraw = vn_raw[j];
     float vn[4];
     vn[0] = f16_bits_to_f32((uint16_t)(vraw.x & 0xffffu));
     vn[1] = f16_bits_to_f32((uint16_t)(vraw.x >> 16));
