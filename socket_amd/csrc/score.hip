@@ -356,6 +356,9 @@ __device__ __forceinline__ void score_tile(
     constexpr bool kFlat = GP > 1 && std::is_same<TT, TabBF16>::value;
     constexpr int kPrefetch = kFlat ? (DMA ? (KT4 == 1 ? 8 : 4) : (KT4 == 2 && THREADS == 1024 ? 2 : 3)) : DMA ? 4 : 3;
     uint4 ring[kPrefetch][KT4];
+    // (the first slice's copies go out ahead of the code words, so that the wait below
+    // can leave all but the first word in flight)
+    if (DMA && !table_resident) dma_slice(0, 0);
 #pragma unroll
     for (int d = 0; d < kPrefetch; ++d)
 #pragma unroll
@@ -428,8 +431,9 @@ __device__ __forceinline__ void score_tile(
     const bool staged = nbuf == 2;
     if (DMA) {
       if (!table_resident) {
-        dma_slice(0, 0);
-        wait_vmcnt(0);    // (the code prefetches above are waited for too; once per workgroup)
+        // loads retire in order: with the words 1 .. kPrefetch-1 still outstanding, slice
+        // 0 and word 0 have landed
+        wait_vmcnt((kPrefetch - 1) * KT4);
         __syncthreads();  // slice 0 is in place
       }
     } else if (staged) {
