@@ -46,7 +46,6 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
-BOX_CPU_SHARE = 16              # host cores a one-GPU job is given on the benchmark box
 
 # HBM bytes per launch of the scorer from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `bench.py --only score_grouped` (profiles/score_packed_c3_hbm_counters.txt
@@ -211,11 +210,17 @@ def cpu_baseline(w, inp_cpu, codes_cpu, vnorm_cpu, seconds_budget=20.0):
     heads (2*G query heads), full context; scaled to the whole layer."""
     from oracle import socket_oracle as orc
 
-    # every core this job may use: the GPU box gives a one-GPU job 16 of the host's cores
-    # (its os.cpu_count() reports the whole host); both figures are in the record
+    # every core this job may use: the cores the process is allowed on, capped by the
+    # thread budget the environment sets for it (OMP_NUM_THREADS; a shared host reports all
+    # its cores to every job); the threads actually used and the host's count are both recorded
     host_cores = os.cpu_count() or 1
-    cores = min(host_cores, BOX_CPU_SHARE)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else host_cores
+    try:
+        cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+    except ValueError:
+        pass
     torch.set_num_threads(cores)
+    cores = torch.get_num_threads()
     G = w.Hq // w.Hkv
     nkv = min(2, w.Hkv)
     T = int(inp_cpu["len0"])

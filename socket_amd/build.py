@@ -82,23 +82,5 @@ def build(verbose: bool = False, extra_flags=(), only_changed: bool = False) -> 
     return LIB_PATH
 
 
-def build_measurement_lib(path: str) -> str:
-    """A second library at `path` whose scorer takes its launch shape from the
-    SOCKET_SCORE_FORCE environment variable ("tile,direct,one_head"): what
-    socket_amd.score_plan_fit sweeps.  The product library never reads it.
-    Reuses the product build's objects for every other source."""
-    hipcc = _hipcc()
-    objdir = os.path.join(HERE, "build")
-    build(only_changed=True)
-    forced = os.path.join(objdir, "score_forced_shape.o")
-    _run([hipcc, *FLAGS, "-DSOCKET_SCORE_PLAN_OVERRIDE", "-c", os.path.join(CSRC, "score.hip"), "-o", forced])
-    objs = [forced] + [os.path.join(objdir, src.replace(".hip", ".o")) for src in SOURCES if src != "score.hip"]
-    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", path])
-    return path
-
-
 if __name__ == "__main__":
-    if "--measurement-lib" in sys.argv:
-        print(build_measurement_lib(sys.argv[sys.argv.index("--measurement-lib") + 1]))
-    else:
-        print(build(verbose="-v" in sys.argv, only_changed="--changed" in sys.argv))
+    print(build(verbose="-v" in sys.argv, only_changed="--changed" in sys.argv))

@@ -21,10 +21,6 @@
 // (The reference's own operand layout, int16 codes per query head, is served by
 // collide.hip.)
 #include <type_traits>
-#ifdef SOCKET_SCORE_PLAN_OVERRIDE
-#include <cstdio>
-#include <cstdlib>
-#endif
 
 #include "socket_common.h"
 
@@ -992,12 +988,6 @@ template <class TT>
 int dispatch_g(const ScoreArgs& a) {
   const int G = a.Hq / a.Hkv;
   ScorePlan plan = score_plan(a.B, a.Hkv, G, a.T, a.grouped, sizeof(typename TT::elem), a.L, a.P, a.R);
-#ifdef SOCKET_SCORE_PLAN_OVERRIDE
-  if (const char* f = getenv("SOCKET_SCORE_FORCE")) {  // "tile,dma,solo" (measurement builds only)
-    int t = 0, d = 0, so = 0;
-    if (sscanf(f, "%d,%d,%d", &t, &d, &so) == 3) plan = {t, d != 0, so != 0, 0.f};
-  }
-#endif
   if (G == 1 || plan.solo) return dispatch_tile<1, TT>(a, plan);
   if (G == 2) return dispatch_tile<2, TT>(a, plan);
   return dispatch_tile<4, TT>(a, plan);

@@ -52,6 +52,8 @@ def warmup_sparse_decode(model: Transformer, device: torch.device, *, T: int = 4
     for _ in range(2):
         hash_cache.sparse_decode_step(q, q_probs, k, v, codes, v_norm, T, P, int(cfg.sink_size),
                                       int(cfg.window_size), int(attn.heavy_const))
+    # the library's fixed scratch array is looked up here, outside any capture
+    hash_cache.prepare_one_launch_attention(device)
     torch.cuda.synchronize()
 
 
@@ -114,6 +116,7 @@ class DecodeGraph:
             for _ in range(2):
                 self._step()
         torch.cuda.current_stream().wait_stream(side)
+        hash_cache.prepare_one_launch_attention(self.tok.device)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):

@@ -324,17 +324,60 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
     return out[:, :, :T]
 
 
+# Devices whose copy of the library's fixed scratch array has had its address looked up
+# (socket_static_scratch_init), which has to happen outside any stream capture.
+_STATIC_READY = set()
+
+
+def prepare_one_launch_attention(device=None) -> None:
+    """Look up the library's fixed scratch array on `device` (default: the current
+    one).  Call it outside stream capture -- `generate.warmup_sparse_decode` and any
+    eager `sparse_decode_step` do -- before a step is recorded into a graph."""
+    idx = torch.cuda.current_device() if device is None or torch.device(device).index is None \
+        else torch.device(device).index
+    if idx in _STATIC_READY or torch.cuda.is_current_stream_capturing():
+        return
+    with torch.cuda.device(idx):
+        check("socket_static_scratch_init", lib().socket_static_scratch_init())
+    _STATIC_READY.add(idx)
+
+
+def _use_one_launch(q: torch.Tensor, width: int, one_launch: Optional[bool]) -> bool:
+    B, Hq, D = q.shape
+    if one_launch is False or not prefers_one_launch(B, Hq, D, width):
+        return False
+    idx = q.device.index if q.device.index is not None else torch.cuda.current_device()
+    capturing = torch.cuda.is_current_stream_capturing()
+    if not capturing:
+        prepare_one_launch_attention(q.device)
+    if one_launch is True:
+        return idx in _STATIC_READY
+    # default: only inside a graph capture, whose replays the caller issues one after another
+    return capturing and idx in _STATIC_READY
+
+
 @torch.no_grad()
 def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Tensor,
                        v_cache: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
                        sink: int, window: int, M: int, lens: Optional[torch.Tensor] = None,
                        budgets: Optional[torch.Tensor] = None,
-                       return_details: bool = False):
+                       return_details: bool = False, one_launch: Optional[bool] = None):
     """One decode step of sparse attention for one layer: score every cached key,
     select top-M + sink + window, attend over the selected rows.
 
     q [B,Hq,D]; q_probs [B,Hq,L,R]; T = number of cached tokens to consider (an
     upper bound when `lens` gives per-sequence lengths).  Returns out [B,Hq,D].
+
+    `one_launch`: the attention has a one-launch form whose split partials and
+    arrival counters live in ONE array per GPU inside the library
+    (`socket_sparse_attention_static`): two such calls that overlap on a GPU -- two
+    streams, two threads, an eager step beside a graph replay -- corrupt each other
+    silently.  The default (None) therefore takes it only while the step is being
+    recorded into a HIP graph, where it also saves the allocation, and the eager
+    step takes the re-entrant two-launch form with a workspace per call (same
+    output, bit for bit).  Replays of graphs that hold this step must not overlap
+    on one GPU.  True forces the one-launch form (the caller answers for the
+    serialisation), False forbids it.
     """
     # (no per-tile key ranges from the scorer: the selection draws its threshold from a
     # sample of the row and only a row whose sample misleads it falls back to a pass
@@ -342,9 +385,7 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens, n_heads=q.shape[1])
     sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets)
     B, Hq, D = q.shape
-    if prefers_one_launch(B, Hq, D, sparse_list.shape[-1]):
-        # one launch (the last split of a row merges it) on the library's own scratch array;
-        # the decode step is issued on one stream, as that entry point requires
+    if _use_one_launch(q, sparse_list.shape[-1], one_launch):
         out = sparse_attention_fwd_static(q, k_cache, v_cache, sparse_list, sparse_len,
                                           torch.empty((B, Hq, D), dtype=q.dtype, device=q.device))
     else:
@@ -352,6 +393,40 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     if return_details:
         return out, scores, sparse_list, sparse_len
     return out
+
+
+@functools.lru_cache(maxsize=1024)
+def step_cost_estimate(B: int, Hq: int, Hkv: int, D: int, T: int, L: int, P: int, R: int, M: int,
+                       sink: int, window: int, table_bf16: bool = True) -> Tuple[float, float]:
+    """(sparse_us, dense_us): rough device time of one layer's decode attention
+    over T cached tokens, for choosing between the two.  The scorer's figure is the
+    library's own launch-shape estimate (`socket_score_plan_query`); the selection,
+    the two attentions and the launches are priced from what they read at the rates
+    measured for them on a 256-CU MI355X (a row's selection: ~11 us of threshold
+    and placement plus 3.7 us per 32768 scores a workgroup streams, 3 us more when
+    a row is shared; gathers at 5.2 TB/s; the dense stream at 6.4 TB/s; ~4 us a
+    launch).  Good to some 20 %: it places the crossover, it is not a timing."""
+    import ctypes
+    cus = ctypes.c_int(0)
+    lib().socket_device_query(ctypes.byref(cus), None)
+    cu = max(1, cus.value)
+    cost = ctypes.c_float(0.0)
+    check("socket_score_plan_query", lib().socket_score_plan_query(
+        B, Hq, Hkv, T, dtype_enum(torch.bfloat16 if table_bf16 else torch.float32), L, P, R, 1,
+        None, None, None, ctypes.byref(cost)))
+    rows = B * Hq
+    parts = 1
+    ws = lib().socket_select_workspace_bytes(B, Hq, T, M)
+    if ws:
+        parts = max(1, min(16, cu // rows, T // 16384))
+    rounds = -(-rows * parts // cu)
+    select = rounds * (11.0 + 3.7 * (T / parts) / 32768.0 + (3.0 if parts > 1 else 0.0))
+    listed = min(T, sink + window + M)
+    esize = 2 if D * 2 <= 256 else 4     # (16-bit caches are what the decode path serves; an upper bound otherwise)
+    attend = rows * listed * (2 * D * esize + 4) / 5.2e6 + (0.0 if 2 * rows >= cu else 5.0)
+    dense = B * Hkv * T * 2 * D * esize / 6.4e6 + 5.0
+    launch = 4.0
+    return float(cost.value + select + attend + 3 * launch), float(dense + launch)
 
 
 class SocketHashCache:

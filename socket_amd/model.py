@@ -61,6 +61,11 @@ class ModelArgs:
     heavy_const: int = 3600
     sink_size: int = 120
     window_size: int = 120
+    # Not in the reference: with True a sparse decode step takes the dense kernel while
+    # the cache is short enough for `hash_cache.step_cost_estimate` to price dense
+    # attention below score + select + attend (exact attention, and faster there);
+    # False keeps `decode_type="sparse"` sparse at every length, as the reference does.
+    dense_below_crossover: bool = False
 
     def __post_init__(self):
         if self.n_local_heads == -1:
@@ -100,9 +105,11 @@ class KVCache(nn.Module):
 
     Constructor as GPT-FAST/model.py:162-171 with two keyword additions (`K`,
     the bits per table, which fixes the packing; `device`).  `update` keeps the
-    reference's signature and bounds error (model.py:187-229); positions must be
-    one ascending run (they always are: arange(T) for prefill, [pos] for a decode
-    step)."""
+    reference's signature and bounds error (model.py:187-229) and takes any index
+    tensor; one ascending run (arange(T) for prefill, [pos] for a decode step: all
+    the reference's own call path produces) is written in one piece, anything else
+    as the runs it consists of.  The cached length `lens` follows the last write
+    (largest position + 1) where the reference keeps a running maximum."""
 
     def __init__(self, max_batch_size: int, max_seq_length: int, n_heads: int, head_dim: int, L: int, R: int,
                  dtype=torch.bfloat16, K: int = 10, device=None):
@@ -170,9 +177,36 @@ class KVCache(nn.Module):
             # does not expose the rows a longer sequence left behind
             self.lens.copy_(torch.where(ok, pos_b + 1, self.lens))
             return self.k_cache, self.v_cache
-        if pos0 is None:
-            pos0 = int(input_pos[0])
-        self._bounds(pos0, S)
+        if pos0 is not None:
+            # the caller vouches for one ascending run that starts at pos0 (prefill: arange)
+            self._bounds(pos0, S)
+            self._write_run(pos0, k_val, v_val, v_norm, k_hard, hash_keys)
+            self.lens.fill_(pos0 + S)
+            return self.k_cache, self.v_cache
+        # Any index tensor, as the reference's advanced-index write takes (model.py:208-226):
+        # the positions come to the host once (the reference reads their extremes back too) and
+        # are written as the maximal ascending runs they consist of, in order, so that a
+        # position listed twice keeps its last row.
+        pos = [int(p) for p in input_pos.tolist()]
+        lo, hi = min(pos), max(pos)
+        if lo < 0:
+            self._bounds(lo, 1)
+        self._bounds(hi, 1)
+        start = 0
+        for i in range(1, S + 1):
+            if i == S or pos[i] != pos[i - 1] + 1:
+                sl = slice(start, i)
+                self._write_run(pos[start], k_val[:, sl], v_val[:, sl],
+                                None if v_norm is None else v_norm[:, sl],
+                                None if k_hard is None else k_hard[:, sl], hash_keys)
+                start = i
+        self.lens.fill_(hi + 1)
+        return self.k_cache, self.v_cache
+
+    def _write_run(self, pos0: int, k_val: Tensor, v_val: Tensor, v_norm: Optional[Tensor],
+                   k_hard: Optional[Tensor], hash_keys: bool) -> None:
+        """Rows [pos0, pos0 + S) of every buffer from k_val / v_val [B,S,H,D]."""
+        S = k_val.shape[1]
         self.k_cache[:, :, pos0:pos0 + S].copy_(k_val.permute(0, 2, 1, 3))
         self.v_cache[:, :, pos0:pos0 + S].copy_(v_val.permute(0, 2, 1, 3))
         if hash_keys:
@@ -182,8 +216,6 @@ class KVCache(nn.Module):
                 self.v_norm[:, :, pos0:pos0 + S].copy_(v_norm.permute(0, 2, 1))
             if k_hard is not None:
                 hash_cache.pack_codes_into(k_hard.permute(0, 2, 3, 1), self.codes, self.K, t0=pos0)
-        self.lens.fill_(pos0 + S)
-        return self.k_cache, self.v_cache
 
 
 # The places where the attention hook enters the HIP library.  They are
@@ -195,7 +227,22 @@ def _hash_rows(cache: KVCache, k_bshd: Tensor, v_bshd: Tensor, t0: int = 0, pos_
                               t0=t0, pos_b=pos_b, layout="bshd")
 
 
+def _sparse_is_slower(cfg: "ModelArgs", cache: KVCache, n_head: int) -> bool:
+    """config.dense_below_crossover: True when a dense step over this cache is priced
+    below the sparse one (decided from the cache's capacity, on the host)."""
+    if not getattr(cfg, "dense_below_crossover", False) or not cache.k_cache.is_cuda:
+        return False
+    B, Hkv, T, D = cache.k_cache.shape
+    sparse_us, dense_us = hash_cache.step_cost_estimate(
+        B, n_head, Hkv, D, T, cache.L, cache.K, cache.R, int(cfg.heavy_const), int(cfg.sink_size),
+        int(cfg.window_size), cache.k_cache.dtype == torch.bfloat16)
+    return dense_us < sparse_us
+
+
 def _sparse_step(q_bhd: Tensor, q_probs: Tensor, cache: KVCache, T: int, sink: int, window: int, M: int) -> Tensor:
+    """One layer's score -> select -> attend.  Issued on the current stream; under graph
+    capture the attention is the one-launch form on the library's per-GPU scratch array
+    (`hash_cache.sparse_decode_step`): replays of such graphs must not overlap on a GPU."""
     return hash_cache.sparse_decode_step(q_bhd, q_probs, cache.k_cache, cache.v_cache, cache.codes, cache.v_norm,
                                          T, cache.K, sink, window, M, lens=cache.lens)
 
@@ -445,7 +492,7 @@ class Attention(nn.Module):
             return self.wo(y.reshape(bsz, seqlen, self.dim))
 
         q_bhd = q[:, 0]                                                       # [B,H,D]
-        if sparse:
+        if sparse and not _sparse_is_slower(self.config, cache, self.n_head):
             T = cache.k_cache.size(2)       # upper bound; the kernels stop at cache.lens
             cfg = self.config
             # on the device the table is written in the layout the scorer prefers (same values);
@@ -464,7 +511,15 @@ class Attention(nn.Module):
         bsz = x.shape[0]
         cache = self.kv_cache
         qkv = decode_ops.linear_rows(x, self.wqkv.weight)
-        if sparse:
+        if sparse and _sparse_is_slower(self.config, cache, self.n_head):
+            # below the crossover: the dense kernel, with the new key still hashed so that the
+            # cache's hash state stays complete
+            q_bhd, k_new, v_new = decode_ops.rope_append(qkv, step.freqs_table, input_pos, cache.k_cache,
+                                                         cache.v_cache, cache.lens, self.n_head,
+                                                         self.n_local_heads, return_new=True)
+            _hash_rows(cache, k_new, v_new, pos_b=step.pos_b)
+            out_bhd = _dense_step(q_bhd, cache)
+        elif sparse:
             cfg = self.config
             fused = _decode_prologue(qkv, step.freqs_table, input_pos, cache, self.planes, self.protos_T,
                                      self.n_head, self.n_local_heads)

@@ -12,6 +12,8 @@ use `socket_amd.hash_cache`.
 """
 from __future__ import annotations
 
+import collections
+
 import torch
 
 from ._lib import SOCKET_TOPK_MAX_M, check, lib, ptr, stream_ptr
@@ -33,20 +35,57 @@ def _get_soft_hash_ext():
     return _SOFT_HASH_EXT
 
 
-# Workspaces of the selection, one per (device, stream, size): the kernel wants the
-# arrival counters at its head zero on entry and leaves them zero, so a workspace is
-# zeroed once, when it is made, and serves every later call issued on that stream.
-_SELECT_WS = {}
+# Workspaces of the selection.  The kernel wants the arrival counters at a workspace's
+# head zero on entry and leaves them zero, so a workspace is zeroed once, when it is made,
+# and serves every later call that cannot overlap with another user of it:
+#   * eager calls: one per (device, stream, size) -- calls on one stream are ordered;
+#   * calls recorded into a HIP graph: one per (device, size), made and zeroed OUTSIDE the
+#     capture by the eager call of the same shape that precedes any capture (a buffer made
+#     during a capture would live in that graph's private pool, be zeroed only by a
+#     recorded node, and outlive the graph in this table).  Replays of graphs that hold a
+#     decode step must not overlap on one GPU (hash_cache.sparse_decode_step), which is
+#     what lets them share it.
+# The table is bounded: the least recently used entries are dropped beyond _SELECT_WS_MAX.
+_SELECT_WS = collections.OrderedDict()
+_SELECT_WS_MAX = 32
+
+
+def _new_workspace(device: torch.device, nbytes: int, zero_bytes: int) -> torch.Tensor:
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    ws[:zero_bytes].zero_()
+    return ws
 
 
 def _select_workspace(device: torch.device, nbytes: int, zero_bytes: int) -> torch.Tensor:
+    capturing = torch.cuda.is_current_stream_capturing()
+    graph_key = (device.index, None, nbytes)
+    if capturing:
+        ws = _SELECT_WS.get(graph_key)
+        if ws is None:
+            # no eager call of this shape came first: a buffer of this capture's own, zeroed by a
+            # recorded node on every replay, and not kept here
+            return _new_workspace(device, nbytes, zero_bytes)
+        _SELECT_WS.move_to_end(graph_key)
+        return ws[0]
     key = (device.index, torch.cuda.current_stream(device).cuda_stream, nbytes)
-    ws = _SELECT_WS.get(key)
-    if ws is None:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    for k in (key, graph_key):
+        if k not in _SELECT_WS:
+            _SELECT_WS[k] = (_new_workspace(device, nbytes, zero_bytes), zero_bytes)
+        _SELECT_WS.move_to_end(k)
+    while len(_SELECT_WS) > _SELECT_WS_MAX:
+        _SELECT_WS.popitem(last=False)
+    return _SELECT_WS[key][0]
+
+
+def reset_select_workspaces() -> None:
+    """Zero the arrival counters of every cached workspace again.  A selection that
+    was aborted mid-launch (a device error) can leave them counting; `select_list`
+    calls this when the library reports a failure, and a caller who tore down a
+    stream with work in flight should too."""
+    if torch.cuda.is_current_stream_capturing():
+        return
+    for ws, zero_bytes in _SELECT_WS.values():
         ws[:zero_bytes].zero_()
-        _SELECT_WS[key] = ws
-    return ws
 
 
 def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=None, budgets=None,
@@ -79,11 +118,16 @@ def select_list(scores: torch.Tensor, sink: int, window: int, M: int, *, lens=No
     ws, ws_bytes = None, L.socket_select_workspace_bytes(B, H, T, M) if split else 0
     if ws_bytes:
         ws = _select_workspace(scores.device, ws_bytes, L.socket_select_workspace_zero_bytes(B, H, T, M))
-    check("socket_select_list", L.socket_select_list(
-        ptr(scores), scores.stride(1), ptr(lens), ptr(budgets), ptr(row_range),
-        0 if row_range is None else row_range.shape[2], B, H, T, M, int(sink), int(window),
-        1 if write_base else 0, ptr(sparse_list), list_width, list_width, ptr(sparse_len),
-        ptr(ws), ws_bytes, stream_ptr(scores.device)))
+    try:
+        check("socket_select_list", L.socket_select_list(
+            ptr(scores), scores.stride(1), ptr(lens), ptr(budgets), ptr(row_range),
+            0 if row_range is None else row_range.shape[2], B, H, T, M, int(sink), int(window),
+            1 if write_base else 0, ptr(sparse_list), list_width, list_width, ptr(sparse_len),
+            ptr(ws), ws_bytes, stream_ptr(scores.device)))
+    except RuntimeError:
+        if ws is not None:
+            reset_select_workspaces()
+        raise
     return sparse_list, sparse_len
 
 

@@ -735,6 +735,58 @@ def test_soft_hash_matches_oracle(dev, dtype, B, Hq, Hkv, D, L, K, R, temp, cube
         assert torch.equal(have32.argmax(-1)[clear], hard[clear])
 
 
+def _bf16_ulps(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance in bf16 units in the last place between two non-negative bf16 tensors."""
+    return (a.view(torch.int16).int() - b.view(torch.int16).int()).abs()
+
+
+@pytest.mark.parametrize("name,Hq,Hkv,L,temp,cube,plane_scale,proto_scale", [
+    ("gpt-fast", 32, 8, 60, 1.0, False, 0.3, 3.0),    # GPT-FAST/model.py:392-401: random prototypes, no temperature
+    ("hf", 28, 4, 48, 0.3, True, 1.0, 1.0),           # modeling_llama.py:618-638: hypercube corners, logits / 0.3
+])
+def test_bf16_soft_hash_against_the_reference_dtype_chain(dev, name, Hq, Hkv, L, temp, cube, plane_scale, proto_scale):
+    """The reference runs its two einsums, the tanh, the division and the softmax in the
+    model dtype, rounding to bf16 after each (the oracle's soft_hash does the same when
+    it is handed bf16 tensors); the kernel computes in fp32 and rounds once.  Stated
+    bound: every entry within 8 bf16 units in the last place of the reference-dtype
+    chain (measured: at most 4, 0.04-31 % of the entries differ at all, depending on how
+    peaked the tables are), every row still summing to 1 within bf16 rounding -- and the
+    difference does not move the selection: at a 32768-token context with top-1024 the
+    lists built from the two tables share at least 98 % of their entries in every row."""
+    g = torch.Generator().manual_seed(77 + L)
+    B, D, K, T, M = 1, 128, 10, 32768, 1024
+    R, G = 1 << K, Hq // Hkv
+    q = torch.randn(B, Hq, D, generator=g).to(torch.bfloat16)
+    planes = (torch.randn(L, K, D, generator=g) * plane_scale).to(torch.bfloat16)
+    protos = (orc.hypercube_protos_T(K) if cube else torch.randn(K, R, generator=g) * proto_scale).to(torch.bfloat16)
+    chain = orc.soft_hash(q, planes, protos, temperature=temp)                        # bf16 at every step
+    assert chain.dtype == torch.bfloat16
+    have = hash_cache.soft_hash(q.to(dev), planes.to(dev), protos.to(dev), temp, Hkv, out_dtype=torch.bfloat16)
+    ulps = _bf16_ulps(have.cpu(), chain)
+    frac = float((ulps > 0).float().mean())
+    print(f"soft hash {name}: {100 * frac:.2f} % of entries differ from the bf16 chain, max {int(ulps.max())} ulps")
+    assert int(ulps.max()) <= 8
+    assert float((have.float().sum(-1) - 1).abs().max()) <= 4e-3
+    # the selection from either table
+    keys = torch.randn(B, T, Hkv, D, generator=g).to(torch.bfloat16)
+    vals = torch.randn(B, T, Hkv, D, generator=g).to(torch.bfloat16)
+    cache = hash_cache.SocketHashCache(B, T, Hkv, D, L, K, dtype=torch.bfloat16, device=dev)
+    cache.set_planes(planes.float())
+    cache.append(0, keys.to(dev), vals.to(dev))
+    lists = []
+    for table in (have, chain.to(dev)):
+        scores = hash_cache.score_packed(table, cache.codes, cache.v_norm, T, K)
+        sl, _ = sparse.select_list(scores, 0, 0, M, write_base=False)
+        lists.append(sl.cpu())
+    worst = 1.0
+    for h in range(Hq):
+        a, b = set(lists[0][0, h].tolist()), set(lists[1][0, h].tolist())
+        assert len(a) == M and len(b) == M
+        worst = min(worst, len(a & b) / M)
+    print(f"soft hash {name}: smallest top-{M} overlap over {Hq} rows {worst:.4f}")
+    assert worst >= 0.98
+
+
 @pytest.mark.parametrize("B,Hq,Hkv,L,P,T,dtype", [
     (2, 8, 2, 20, 10, 5000, torch.bfloat16),     # G=4
     (1, 14, 2, 12, 10, 3000, torch.bfloat16),    # G=7: two parts of width 4

@@ -247,31 +247,25 @@ def test_score_plan_on_the_benchmark_shapes():
     assert _shape_cost(lib, 1, 32, 8, 8192, 1, 60, 10, 1, 2048, 1, 1)[0] != 0       # one head per workgroup on a grouped table
 
 
-def test_score_plan_fit_recovers_the_model_from_its_own_prices(tmp_path):
-    """The refit tool on measurements that ARE the model (every forced shape timed at
-    the library's own estimate): the fitted constants must choose as the library does."""
-    import json
-    from socket_amd import score_plan_fit
-    from socket_amd._lib import lib as load
-    lib = load()
-    rows = []
-    for (L, P, G, dt) in ((60, 10, 4, "bfloat16"), (32, 8, 4, "float32"), (48, 10, 7, "bfloat16"), (60, 10, 1, "bfloat16")):
-        for (B, Hkv, T) in ((1, 8, 32768), (4, 8, 131072), (16, 4, 65536)):
-            for tile in score_plan_fit.TILES:
-                for dma, solo in score_plan_fit.VARIANTS:
-                    for layout in ("grouped", "ref"):
-                        if (dma and not solo and layout != "grouped") or (solo and layout != "ref"):
-                            continue
-                        rc, _, _, cost = _shape_cost(lib, B, Hkv * G, Hkv, T, 1 if dt == "bfloat16" else 0, L, P,
-                                                     int(layout == "grouped"), tile, dma, int(solo and G > 1))
-                        rows.append(dict(L=L, P=P, G=G, dt=dt, B=B, Hkv=Hkv, T=T, tile=tile, dma=dma, solo=solo,
-                                         layout=layout, us=cost if rc == 0 else None))
-    path = tmp_path / "sweep.jsonl"
-    path.write_text("\n".join(json.dumps(r) for r in rows) + "\n")
-    shape_mean, shape_max, layout_mean, layout_max = score_plan_fit.fit(str(path))
-    assert shape_mean <= 1.0 + 1e-6 and shape_max <= 1.0 + 1e-6          # the library's constants on its own prices
-    # the grouped layout is preferred unless the other is more than 1.3 times cheaper: that margin bounds the regret
-    assert 1.0 <= layout_mean <= layout_max <= 1.3 + 1e-6
+def test_step_cost_estimate_places_the_crossover():
+    """The estimate behind ModelArgs.dense_below_crossover: sparse is priced below dense
+    at 4 x 131072 and at 1 x 131072 tokens, above it at 1 x 32768 (as measured on the
+    device), and neither price falls as the context grows."""
+    from socket_amd import hash_cache as hc
+    geo = dict(Hq=32, Hkv=8, D=128, L=60, P=10, R=1024, sink=4, window=256)
+    at = lambda B, T, M: hc.step_cost_estimate(B, geo["Hq"], geo["Hkv"], geo["D"], T, geo["L"], geo["P"], geo["R"],
+                                               M, geo["sink"], geo["window"])
+    s, d = at(4, 131072, 2048)
+    assert s < d and 1.6 < d / s < 3.0
+    s, d = at(1, 131072, 2048)
+    assert s < d
+    s, d = at(1, 32768, 1024)
+    assert d < s
+    prev = (0.0, 0.0)
+    for T in (8192, 16384, 32768, 65536, 131072, 262144):
+        cur = at(1, T, 1024)
+        assert cur[1] >= prev[1] and cur[0] > 0
+        prev = cur
 
 
 def test_python_api_keeps_reference_signatures():

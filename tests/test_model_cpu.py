@@ -125,6 +125,36 @@ def test_kv_cache_update_bookkeeping(monkeypatch):
         c.update(torch.arange(4), k, v)
 
 
+def test_kv_cache_update_takes_any_position_tensor(monkeypatch):
+    """GPT-FAST/model.py:208-226 writes with an advanced index, so any position
+    tensor is legal there: scattered positions, a descending order, two runs.  Every
+    buffer must end up as that indexed write leaves it (codes and norms as a cache
+    that received the same rows in one ascending piece holds them)."""
+    oracle_backend.install(monkeypatch, M)
+    planes = oracle_backend.planes_to_words(torch.randn(6, 4, 128, generator=torch.Generator().manual_seed(40)))
+    g = torch.Generator().manual_seed(41)
+    pos = torch.tensor([9, 10, 11, 3, 20, 19, 2])
+    k = torch.randn(2, 7, 1, 128, generator=g); v = torch.randn(2, 7, 1, 128, generator=g)
+    c = M.KVCache(2, 30, 1, 128, L=6, R=16, dtype=torch.float32, K=4)
+    c.planes_words = planes
+    c.update(pos, k, v, hash_keys=True)
+    want_k = torch.zeros_like(c.k_cache); want_v = torch.zeros_like(c.v_cache)
+    want_k[:, :, pos] = k.permute(0, 2, 1, 3); want_v[:, :, pos] = v.permute(0, 2, 1, 3)
+    assert torch.equal(c.k_cache, want_k) and torch.equal(c.v_cache, want_v)
+    assert c.lens.tolist() == [21, 21]
+    # the same rows given to a second cache in ascending order, one piece per position
+    d = M.KVCache(2, 30, 1, 128, L=6, R=16, dtype=torch.float32, K=4)
+    d.planes_words = planes
+    for i in torch.argsort(pos).tolist():
+        d.update(pos[i:i + 1], k[:, i:i + 1], v[:, i:i + 1], hash_keys=True, pos0=int(pos[i]))
+    assert torch.equal(c.codes, d.codes) and torch.equal(c.v_norm, d.v_norm)
+    e = M.KVCache(2, 30, 1, 128, L=6, R=16, dtype=torch.float32, K=4)
+    with pytest.raises(RuntimeError, match="out-of-bounds"):
+        e.update(torch.tensor([4, 32, 5]), k[:, :3], v[:, :3])
+    with pytest.raises(RuntimeError, match="out-of-bounds"):
+        e.update(torch.tensor([4, -1]), k[:, :2], v[:, :2])
+
+
 def test_sparse_decode_with_an_all_covering_window_reproduces_dense_tokens(monkeypatch):
     """With no sink, no heavy budget and a window longer than the context the
     list is every cached row exactly once (sparse.py:70-84), so greedy decoding

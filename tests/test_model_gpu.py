@@ -9,6 +9,7 @@ import torch
 
 from oracle import socket_oracle as orc
 from socket_amd import generate as gen
+from socket_amd import hash_cache
 from socket_amd import model as M
 from tests import oracle_backend
 
@@ -91,6 +92,38 @@ def test_a_cache_reused_for_a_shorter_prompt_forgets_the_longer_one(dev, sparse)
     assert torch.equal(have, want)
 
 
+def test_dense_below_crossover_takes_the_dense_kernel_and_keeps_the_hash_state(dev):
+    """ModelArgs.dense_below_crossover on a short cache (where dense attention is priced
+    below score + select + attend): the sparse hook's logits are the dense hook's, plain
+    and fused step alike, and the cache's codes are those a sparse run writes."""
+    g = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, 331, (2, 150), generator=g).to(dev)
+    plain = toy_model(dev, torch.bfloat16)
+    plain.setup_caches(2, 160)
+    want_sparse_codes = None
+    _run_steps(plain, ids, 140)
+    want_sparse_codes = plain.layers[1].attention.kv_cache.codes.clone()
+    _reset(plain)
+    want = _run_steps(plain, ids, 140, sparse=False)
+    model = toy_model(dev, torch.bfloat16, dense_below_crossover=True)
+    model.setup_caches(2, 160)
+    c = model.layers[0].attention.kv_cache
+    s_us, d_us = hash_cache.step_cost_estimate(2, 4, 2, 128, c.k_cache.shape[2], 20, 10, 1024, 48, 4, 16)
+    assert d_us < s_us
+    have = _run_steps(model, ids, 140)
+    assert torch.equal(have, want)
+    assert torch.equal(model.layers[1].attention.kv_cache.codes, want_sparse_codes)
+    # the fused single-token step (what the decode graph records)
+    step = gen.DecodeGraph(model, 2, "sparse", dev)
+    ref = gen.DecodeGraph(plain, 2, "dense", dev)
+    for dg in (step, ref):
+        dg.tok.copy_(ids[:, 149:150].to(torch.int))
+        dg.pos.fill_(149)
+    a, _ = step._step()
+    b, _ = ref._step()
+    assert torch.equal(a, b)
+
+
 def test_eager_decode_step_at_a_position_outside_the_cache_writes_nothing(dev):
     """The unfused single-token path with a device-side position past the cache:
     no row is written and the length stays (the fused path and the hashing kernel
@@ -105,6 +138,36 @@ def test_eager_decode_step_at_a_position_outside_the_cache_writes_nothing(dev):
     c.update(torch.tensor([64], device=dev), k, k, hash_keys=True)
     assert c.lens.tolist() == [6, 6]
     assert torch.equal(c.k_cache, snap[0]) and torch.equal(c.codes, snap[1]) and torch.equal(c.v_norm, snap[2])
+
+
+def test_kv_cache_update_scatters_rows_codes_and_norms(dev):
+    """Positions in any order with the reference's calling convention (precomputed
+    v_norm and k_hard, GPT-FAST/model.py:222-226) and with the fused hashing: every
+    buffer as the reference's advanced-index write leaves it."""
+    g = torch.Generator().manual_seed(24)
+    pos = torch.tensor([9, 10, 11, 3, 40, 39, 2], device=dev)
+    k = torch.randn(2, 7, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    v = torch.randn(2, 7, 2, 128, generator=g).to(torch.bfloat16).to(dev)
+    kh = torch.randint(0, 1024, (2, 7, 2, 20), generator=g).to(torch.int16).to(dev)
+    vn = torch.rand(2, 7, 2, generator=g).to(torch.float16).to(dev)
+    c = M.KVCache(2, 64, 2, 128, L=20, R=1024, dtype=torch.bfloat16, K=10, device=dev)
+    c.update(pos, k, v, v_norm=vn, k_hard=kh)
+    want_k = torch.zeros_like(c.k_cache)
+    want_k[:, :, pos] = k.permute(0, 2, 1, 3)
+    assert torch.equal(c.k_cache, want_k) and c.lens.tolist() == [41, 41]
+    assert torch.equal(c.k_hard(64)[:, :, pos], kh.permute(0, 2, 1, 3))
+    assert torch.equal(c.v_norm[:, :, pos], vn.permute(0, 2, 1))
+    untouched = torch.ones(64, dtype=torch.bool, device=dev)
+    untouched[pos] = False
+    assert not c.k_hard(64)[:, :, untouched].any() and not c.v_norm[:, :, untouched].any()
+    # fused hashing: the same as one position at a time
+    a = M.KVCache(2, 64, 2, 128, L=20, R=1024, dtype=torch.bfloat16, K=10, device=dev)
+    b = M.KVCache(2, 64, 2, 128, L=20, R=1024, dtype=torch.bfloat16, K=10, device=dev)
+    a.planes_words = b.planes_words = hash_cache_planes(dev)
+    a.update(pos, k, v, hash_keys=True)
+    for i in range(7):
+        b.update(pos[i:i + 1], k[:, i:i + 1], v[:, i:i + 1], hash_keys=True)
+    assert torch.equal(a.codes, b.codes) and torch.equal(a.v_norm, b.v_norm) and torch.equal(a.v_cache, b.v_cache)
 
 
 def hash_cache_planes(dev):
