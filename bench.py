@@ -608,10 +608,15 @@ def decode_tok_s(dev, prompt_len, new_tokens, n_layer=None, kinds=("sparse", "de
            "prompt_len": prompt_len, "new_tokens": new_tokens, "batch": 1,
            "budget": f"top-k {cfg.heavy_const} + sink {cfg.sink_size} + window {cfg.window_size}"}
     for kind in kinds:
-        _, st = gen.generate(model, prompt, new_tokens, decode_type=kind, use_graph=True)
+        # check_graph: before the timed tokens the recorded step is replayed three times from one
+        # state and compared with the eager step (logits and chosen token); the figures travel
+        # with the tok/s so that a fast run whose graph went wrong cannot pass unnoticed
+        _, st = gen.generate(model, prompt, new_tokens, decode_type=kind, use_graph=True, check_graph=True)
+        chk = st.get("graph_check") or {}
         rec[kind] = {"decode_tok_s": round(st["decode_only_tokens"] / st["decode_time_s"], 2),
                      "ms_per_token": round(1e3 * st["decode_time_s"] / st["decode_only_tokens"], 3),
-                     "prefill_s": round(st["prefill_time_s"], 2), "graph": st["graph"]}
+                     "prefill_s": round(st["prefill_time_s"], 2), "graph": st["graph"],
+                     "same_token": chk.get("same_token"), "max_abs_logit_diff": chk.get("max_abs_logit_diff")}
     if "sparse" in rec and "dense" in rec:
         rec["sparse_vs_dense"] = round(rec["sparse"]["decode_tok_s"] / rec["dense"]["decode_tok_s"], 3)
     del model
