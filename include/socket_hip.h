@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SOCKET_ABI_VERSION 3   /* 3: socket_select_list wants the head of its workspace zeroed; socket_decode_prologue */
+#define SOCKET_ABI_VERSION 4   /* 4: the packed scorers take a flags word */
 
 /* status codes */
 #define SOCKET_OK 0
@@ -106,6 +106,8 @@ int socket_pack_codes(const int16_t* in, int64_t in_stride_b, int64_t in_stride_
  * K2  soft-collision scorer
  * ---------------------------------------------------------------------- */
 
+#define SOCKET_SCORE_SKIP_MASKED 1   /* flags bit of the packed scorers, see below */
+
 /* Native scorer on the packed cache.  For every b, kv head, token t < T and
  * each of the G query heads h of that kv head:
  *   scores[b,h,t] = t < len(b) ? (sum_{l<L} q_probs[b,h,l,code_l(b,kv,t)]) * v_norm[b,kv,t] : -inf
@@ -120,6 +122,10 @@ int socket_pack_codes(const int16_t* in, int64_t in_stride_b, int64_t in_stride_
  * Requires Tcap % 4 == 0, score_stride % 4 == 0, 16-byte aligned pointers,
  * R a power of two >= 8, 2^P <= R, G <= 8, and the tables of one packed word
  * (32/P tables x R entries x G values) must fit in LDS.
+ * flags: 0, or SOCKET_SCORE_SKIP_MASKED -- scores[b,h,t] for t >= len(b) may be left
+ * unwritten (a caller that reads rows only up to len(b), as socket_select_list does
+ * with the same lens, saves the write: 73 MB of -inf on a ragged batch of 16 x 28
+ * rows of 98304).  Positions below len(b) are not affected.
  *
  * row_range (optional, may be NULL): uint32 [B*Hq, range_parts, 2]; for every row
  * and token tile the minimum and maximum order-preserving key of the tile's
@@ -138,7 +144,7 @@ int socket_score_packed(const void* q_probs, int q_dtype, const uint32_t* codes,
                         const uint16_t* v_norm, const int32_t* lens, float* scores,
                         uint32_t* row_range, int range_parts,
                         int B, int Hq, int Hkv, int L, int P, int R, int T, int64_t Tcap,
-                        int64_t score_stride, void* stream);
+                        int64_t score_stride, int flags, void* stream);
 
 /* Grouped table layout.  The scorer gathers from an LDS image of the table in which
  * the query heads that share a KV head are interleaved: [table][bucket][head].
@@ -179,7 +185,7 @@ int socket_score_packed_grouped(const void* q_table, int q_dtype, const uint32_t
                                 const uint16_t* v_norm, const int32_t* lens, float* scores,
                                 uint32_t* row_range, int range_parts,
                                 int B, int Hq, int Hkv, int L, int P, int R, int T, int64_t Tcap,
-                                int64_t score_stride, void* stream);
+                                int64_t score_stride, int flags, void* stream);
 
 /* The reference extension's entry point on its own layout:
  * q_probs f32 [B,H,1,L,R], key_buckets i16 [B,H,L,T], allowed bool [B,H,1,T],

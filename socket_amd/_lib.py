@@ -43,7 +43,7 @@ SIGNATURES = {
     "socket_unpack_codes": (_I, [_P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _P]),
     "socket_pack_codes": (_I, [_P, _L, _L, _L, _L, _P, _I, _I, _I, _I, _I, _I, _L, _P]),
     "socket_score_range_parts": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
-    "socket_score_packed": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
+    "socket_score_packed": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _I, _P]),
     "socket_soft_hash_collision": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "socket_soft_hash_score_f16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "socket_score_plan_query": (_I, [_I, _I, _I, _I, _I, _I, _I, _I, _I, POINTER(c_int), POINTER(c_int),
@@ -54,7 +54,7 @@ SIGNATURES = {
     "socket_score_prefers_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "socket_score_range_parts_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "socket_group_q_probs": (_I, [_P, _I, _P, _I, _I, _I, _I, _I, _P]),
-    "socket_score_packed_grouped": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _P]),
+    "socket_score_packed_grouped": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _I, _P]),
     "socket_soft_hash_grouped": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),
     "socket_soft_hash": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),
     "socket_select_workspace_bytes": (_Z, [_I, _I, _I, _I]),
@@ -112,7 +112,7 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        if handle.socket_abi_version() != 3:
+        if handle.socket_abi_version() != 4:
             raise RuntimeError("libsocket_hip.so ABI version mismatch; rebuild it")
         _lib = handle
     return _lib

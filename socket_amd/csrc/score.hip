@@ -765,6 +765,295 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same scoring as one persistent launch dealt from the cached lengths.
+//
+// Tokens are counted in units of 512 (what one wave scores in a tile: two groups of
+// 256, four tokens per lane each).  The units of all (sequence, kv head, head part)
+// rows, each row as long as its sequence's cached length, are laid end to end and
+// cut into gridDim.x equal stretches; a workgroup walks its stretch as tiles of up
+// to 16 units of one row (a tile ends where the row or the stretch ends; the waves
+// past its end skip the lookups and only join the copies and barriers).  Across a
+// tile boundary nothing drains: the last LDS slice of a tile is gathered from while
+// the first slice of the next tile's table is being copied, the code ring fetches
+// the next tile's first words where it would run past the current tile's last, and
+// the sums of the finished tile are stored after the next tile's first slice has
+// been waited for -- so the stores are the oldest memory operations by the time
+// the following slice is waited on, and never hold a wait up.  Every wave runs the
+// same instruction stream whether it has tokens in a tile or not (the ring's loads
+// are unconditional, clamped to the tile's first token), which keeps the exact
+// s_waitcnt counts of the slice copies valid for all of them.
+// Workgroup n of N takes stretch (n % 8) * N / 8 + n / 8: consecutive stretches --
+// the tiles of one row, and the two head parts of a wide group, which walk the same
+// codes at the same time -- sit on one XCD and share its L2.
+// Needs: grouped table, entries of 4 or 8 heads x bf16 or fp32, every packed word
+// full (L a multiple of 32/P), a word count that is a multiple of the ring depth,
+// at most 64 sequences.
+// ---------------------------------------------------------------------------
+constexpr int kFlatUnit = 512;
+constexpr int kFlatTileUnits = 16;
+constexpr int kFlatPrefetch = 4;
+
+template <int GP, class TT, int PT>
+__global__ __launch_bounds__(1024) void score_flat_kernel(
+    const typename TT::elem* __restrict__ q_table, const uint32_t* __restrict__ codes,
+    const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens, float* __restrict__ scores,
+    int B, int Hq, int Hkv, int G, int L, int R, int T, int64_t Tcap, int64_t score_stride, int NW,
+    int chunk_words, int hsplit, uint32_t bf16_one, int fill_masked) {
+  typedef typename TT::elem TE;
+  constexpr int THREADS = 1024, KT4 = 2, kPrefetch = kFlatPrefetch;
+  constexpr int CPW = 32 / PT, EB = GP * (int)sizeof(TE);
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const Bf16Select sel = make_bf16_select(bf16_one);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int VS = Hkv * hsplit;                      // rows of the flattened space per sequence
+  const int chunk_elems = chunk_words * CPW * R * GP;
+  const int offl = wave * kFlatUnit + lane * 4;      // the lane's first token in a tile (group 1: + 256)
+
+  // ---- this workgroup's stretch of the flattened unit space -----------------------------
+  int len_l = 0;                                     // lane l: cached length of sequence l
+  if (lane < B) len_l = lens ? max(0, min(lens[lane], T)) : T;
+  const int u_l = (len_l + kFlatUnit - 1) / kFlatUnit;
+  const int incl = wave_incl_scan(u_l);
+  const int64_t total = (int64_t)__builtin_amdgcn_readlane(incl, 63) * VS;
+  int wg = blockIdx.x;
+  const int nwg = gridDim.x;
+  if ((nwg & 7) == 0) wg = (wg & 7) * (nwg >> 3) + (wg >> 3);
+  const int64_t p0 = total * wg / nwg, p1 = total * (wg + 1) / nwg;
+  int wk_b = 0, wk_vp = 0, wk_pos = 0, wk_left = (int)(p1 - p0);
+  if (wk_left > 0) {
+    // sequence whose rows hold unit p0: the first whose inclusive prefix passes it
+    wk_b = __popcll(__builtin_amdgcn_ballot_w64((int64_t)incl * VS <= p0));
+    const int ub = __builtin_amdgcn_readlane(u_l, wk_b);
+    const int64_t before = (int64_t)(__builtin_amdgcn_readlane(incl, wk_b) - ub) * VS;
+    const int rem = (int)(p0 - before);
+    wk_vp = rem / ub;
+    wk_pos = rem % ub;
+  }
+  struct Tile {   // tokens [start, end) of row (b, vp); end <= the sequence's length; start == end: none
+    int b, vp, start, end;
+  };
+  auto next_tile = [&]() __attribute__((always_inline)) {
+    Tile t{0, 0, 0, 0};
+    if (wk_left <= 0) return t;
+    const int ub = __builtin_amdgcn_readlane(u_l, wk_b);
+    const int n = min(min(kFlatTileUnits, ub - wk_pos), wk_left);
+    t.b = wk_b;
+    t.vp = wk_vp;
+    t.start = wk_pos * kFlatUnit;
+    t.end = min((wk_pos + n) * kFlatUnit, __builtin_amdgcn_readlane(len_l, wk_b));
+    wk_pos += n;
+    wk_left -= n;
+    if (wk_pos >= ub) {
+      wk_pos = 0;
+      if (++wk_vp == VS) {
+        wk_vp = 0;
+        do ++wk_b;
+        while (wk_b < B && __builtin_amdgcn_readlane(u_l, wk_b) == 0);
+      }
+    }
+    return t;
+  };
+  auto codes_of = [&](const Tile& t) __attribute__((always_inline)) { return codes + (int64_t)(t.b * Hkv + t.vp / hsplit) * NW * Tcap; };
+  auto table_of = [&](const Tile& t) __attribute__((always_inline)) { return q_table + (int64_t)(t.b * VS + t.vp) * L * R * GP; };
+
+  float acc[KT4][4][GP];
+  uint4 ring[kPrefetch][KT4];
+  uint2 vn_raw[KT4];
+  auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < KT4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < GP; ++g) acc[j][i][g] = 0.f;
+  };
+  // a wave's share of the table slice that starts at table l0 -> LDS buffer `b`
+  auto dma_slice = [&](const TE* table, int l0, int b) __attribute__((always_inline)) {
+    const int nt = min(chunk_words * CPW, L - l0);
+    const int bytes = nt * R * GP * (int)sizeof(TE);
+    const char* src = reinterpret_cast<const char*>(table + (int64_t)l0 * R * GP);
+    unsigned char* dst = lds_raw + (size_t)b * chunk_elems * sizeof(TE);
+    for (int o = wave * 1024; o < bytes; o += (THREADS / SOCKET_WAVE) * 1024)
+      if (o + lane * 16 < bytes) lds_dma16(src + o + lane * 16, dst + o);
+  };
+  // the lane's token of group j in a tile, or the tile's first token where it has none
+  auto token_of = [&](int start, int end, int j) __attribute__((always_inline)) {
+    const int t = start + offl + j * 256;
+    return t < end ? t : start;
+  };
+  auto load_norms = [&](const Tile& t) __attribute__((always_inline)) {
+    const uint16_t* vn = v_norm + (int64_t)(t.b * Hkv + t.vp / hsplit) * Tcap;
+#pragma unroll
+    for (int j = 0; j < KT4; ++j) vn_raw[j] = *reinterpret_cast<const uint2*>(vn + token_of(t.start, t.end, j));
+  };
+  // sums of a finished tile -> scores
+  auto flush = [&](const Tile& t) __attribute__((always_inline)) {
+    const int part = t.vp % hsplit, kvh = t.vp / hsplit;
+    const int geff = min(GP, G - part * GP);
+    const int len = __builtin_amdgcn_readlane(len_l, t.b);
+    float* row0 = scores + (int64_t)(t.b * Hq + kvh * G + part * GP) * score_stride;
+#pragma unroll
+    for (int j = 0; j < KT4; ++j) {
+      const int tok = t.start + offl + j * 256;
+      if (tok >= t.end) continue;
+      const uint2 vraw = vn_raw[j];
+      float vn[4];
+      vn[0] = f16_bits_to_f32((uint16_t)(vraw.x & 0xffffu));
+      vn[1] = f16_bits_to_f32((uint16_t)(vraw.x >> 16));
+      vn[2] = f16_bits_to_f32((uint16_t)(vraw.y & 0xffffu));
+      vn[3] = f16_bits_to_f32((uint16_t)(vraw.y >> 16));
+#pragma unroll
+      for (int g = 0; g < GP; ++g) {
+        if (g >= geff) break;
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = tok + i < len ? acc[j][i][g] * vn[i] : -INFINITY;
+        float* dst = row0 + (int64_t)g * score_stride + tok;
+        if (tok + 4 <= T) {
+          store_stream16(dst, o[0], o[1], o[2], o[3]);
+        } else {
+          for (int i = 0; i < 4 && tok + i < T; ++i) dst[i] = o[i];
+        }
+      }
+    }
+  };
+
+  Tile cur = next_tile();
+  if (cur.end > cur.start) {
+    Tile nxt = next_tile();
+    bool more = nxt.end > nxt.start;
+    Tile prev = cur;
+    // what the ring fetches: the tile being scored and the one after it (itself when it is the last)
+    const uint32_t* cur_codes = codes_of(cur);
+    const uint32_t* nxt_codes = more ? codes_of(nxt) : cur_codes;
+    const TE* cur_table = table_of(cur);
+    int buf = 0, w0 = 0, wend = min(chunk_words, NW);
+    bool act = cur.start + wave * kFlatUnit < cur.end;
+
+    // the slice after the one that has just become current
+    auto issue_next_slice = [&]() __attribute__((always_inline)) {
+      if (wend < NW) dma_slice(cur_table, wend * CPW, buf ^ 1);
+      else if (more) dma_slice(table_of(nxt), 0, buf ^ 1);
+    };
+    // One word of the tile: the lookups of the wave's two token groups from the slice in
+    // LDS (batches of four, the reads of batch k+1 issued before batch k is added up), then
+    // the ring slot takes the word kPrefetch ahead -- of this tile or of the next.
+    auto lookups = [&](const TE* tw, auto slot) __attribute__((always_inline)) {
+      constexpr int d = decltype(slot)::value;
+      constexpr int NB = KT4 * CPW;
+      RawEntry<EB> ent[2][4];
+      auto issue = [&](int bi, RawEntry<EB>(&dst)[4]) {
+        const int j = bi / CPW, jj = bi % CPW;
+        const uint32_t wv[4] = {ring[d][j].x, ring[d][j].y, ring[d][j].z, ring[d][j].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t code = __builtin_amdgcn_ubfe(wv[i], jj * PT, PT);
+          dst[i] = load_entry<EB>(tw + (size_t)jj * R * GP + (size_t)code * GP);
+        }
+      };
+      issue(0, ent[0]);
+#pragma unroll
+      for (int bi = 0; bi < NB; ++bi) {
+        if (bi + 1 < NB) issue(bi + 1, ent[(bi + 1) & 1]);
+        const int j = bi / CPW;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) accumulate<GP>(acc[j][i], ent[bi & 1][i], (const TT*)nullptr, sel);
+      }
+    };
+    auto refill = [&](int w, auto slot) __attribute__((always_inline)) {
+      constexpr int d = decltype(slot)::value;
+      const int wn = w + kPrefetch;
+      const bool over = wn >= NW;
+      const uint32_t* base = over ? nxt_codes + (int64_t)(wn - NW) * Tcap : cur_codes + (int64_t)wn * Tcap;
+      const int st = over ? nxt.start : cur.start, en = over ? nxt.end : cur.end;
+#pragma unroll
+      for (int j = 0; j < KT4; ++j) ring[d][j] = load_stream16(base + token_of(st, en, j));
+    };
+    // `first`: word 0 of a tile that follows another one of this workgroup
+    auto word = [&](int w, auto slot, auto first) __attribute__((always_inline)) {
+      if (decltype(first)::value || w == wend) {
+        // The copies of the slice that starts here were issued at the top of the one
+        // that ends; since then this wave has issued one code load per word and token
+        // group.  Memory operations retire in order, so allowing that many to be
+        // outstanding, less one word's worth as a margin, means the copies have landed.
+        wait_vmcnt(max(0, ((decltype(first)::value ? NW : wend) - w0 - 1) * KT4));
+        __syncthreads();
+        buf ^= 1;
+        w0 = w;
+        wend = min(w + chunk_words, NW);
+        issue_next_slice();
+        if constexpr (decltype(first)::value) {
+          flush(prev);
+          zero_acc();
+          load_norms(cur);
+        }
+      }
+      const TE* tw = reinterpret_cast<const TE*>(lds_raw) + (size_t)buf * chunk_elems + (size_t)(w - w0) * CPW * R * GP;
+      if (act) lookups(tw, slot);
+      refill(w, slot);
+      // keep the words apart: left alone, the scheduler hoists the gathers of later
+      // words over the adds of earlier ones until the registers run out
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto rounds_from = [&](int wb) __attribute__((always_inline)) {
+      for (; wb < NW; wb += kPrefetch)
+        static_for<kPrefetch>([&](auto s) __attribute__((always_inline)) { word(wb + decltype(s)::value, s, std::false_type{}); });
+    };
+
+    // ---- first tile: nothing is in flight yet ------------------------------------------------
+    zero_acc();
+    load_norms(cur);
+    dma_slice(cur_table, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);   // the copies are issued before the code words: the wait below counts on it
+#pragma unroll
+    for (int d = 0; d < kPrefetch; ++d)
+#pragma unroll
+      for (int j = 0; j < KT4; ++j)
+        ring[d][j] = load_stream16(cur_codes + (int64_t)d * Tcap + token_of(cur.start, cur.end, j));
+    __builtin_amdgcn_sched_barrier(0);
+    wait_vmcnt((kPrefetch - 1) * KT4);   // all but the first word may still be in flight
+    __syncthreads();                     // slice 0 is in place
+    issue_next_slice();
+    rounds_from(0);
+    // ---- the tiles after it --------------------------------------------------------------------
+    while (more) {
+      prev = cur;
+      cur = nxt;
+      nxt = next_tile();
+      more = nxt.end > nxt.start;
+      cur_codes = nxt_codes;
+      nxt_codes = more ? codes_of(nxt) : cur_codes;
+      cur_table = table_of(cur);
+      act = cur.start + wave * kFlatUnit < cur.end;
+      static_for<kPrefetch>([&](auto s) __attribute__((always_inline)) {
+        if constexpr (decltype(s)::value == 0) word(0, s, std::true_type{});
+        else word(decltype(s)::value, s, std::false_type{});
+      });
+      rounds_from(kPrefetch);
+    }
+    flush(cur);
+  }
+
+  // ---- positions past a sequence's cached length ------------------------------------------------
+  if (fill_masked) {
+    for (int row = blockIdx.x; row < B * Hq; row += gridDim.x) {
+      const int len = __builtin_amdgcn_readlane(len_l, row / Hq);
+      float* dst = scores + (int64_t)row * score_stride;
+      // the scored tiles wrote -inf up to the next multiple of four past the length
+      const int from = (len + 3) & ~3;
+      for (int t = from + tid * 4; t < T; t += THREADS * 4) {
+        if (t + 4 <= T) {
+          store_stream16(dst + t, -INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        } else {
+          for (int i = t; i < T; ++i) dst[i] = -INFINITY;
+        }
+      }
+    }
+  }
+}
+
 // LDS past the table buffers in every launch: scratch of the key-range reduction
 constexpr size_t kScoreScratchBytes = 1024;
 
@@ -780,6 +1069,7 @@ struct ScoreArgs {
   int range_parts;
   hipStream_t stream;
   int grouped;  // table layout: 0 = [B,Hq,L,R], 1 = [B*Hkv*parts, L, R, group width]
+  int flags;    // SOCKET_SCORE_*
 };
 
 // How a workgroup's table passes through LDS: buffers, packed words per slice.
@@ -970,6 +1260,62 @@ ScorePlan score_plan(int B, int Hkv, int G, int T, int grouped, size_t table_ele
   return best;
 }
 
+// Packed words per LDS slice of the persistent kernel (two buffers, no register staging).
+int flat_chunk_words(size_t bytes_per_word, int NW, size_t lds_budget) {
+  int cw = 0;
+  while (cw < NW && 2 * bytes_per_word * (cw + 1) <= lds_budget) ++cw;
+  return cw;
+}
+
+// Whether the persistent kernel serves this call: the operands it is written for, and
+// at least one 8192-token tile for every CU (below that the launches that shrink the
+// tile to fill the chip do better).
+bool flat_serves(const ScoreArgs& a, size_t elem_bytes) {
+  const SocketDeviceLimits& lim = socket_device_limits();
+  const int G = a.Hq / a.Hkv;
+  if (!a.grouped || a.row_range || G < 2 || a.B > 64 || (a.P != 8 && a.P != 10)) return false;
+  const int cpw = 32 / a.P, NW = (a.L + cpw - 1) / cpw;
+  if (a.L % cpw != 0 || NW % kFlatPrefetch != 0) return false;
+  const int width = G == 2 ? 2 : 4, hsplit = (G + width - 1) / width;
+  const size_t bytes_per_word = (size_t)cpw * a.R * width * elem_bytes;
+  if (flat_chunk_words(bytes_per_word, NW, (size_t)lim.max_lds_per_block - kScoreScratchBytes) < 1) return false;
+  const int64_t tiles = (int64_t)a.B * a.Hkv * hsplit * ((a.T + 8191) / 8192);
+  return tiles >= lim.cu_count;
+}
+
+template <int GP, class TT, int PT>
+int launch_score_flat(const ScoreArgs& a) {
+  typedef typename TT::elem TE;
+  const SocketDeviceLimits& lim = socket_device_limits();
+  const int G = a.Hq / a.Hkv;
+  constexpr int cpw = 32 / PT;
+  const int NW = a.L / cpw;
+  const size_t bytes_per_word = (size_t)cpw * a.R * GP * sizeof(TE);
+  const int chunk_words = flat_chunk_words(bytes_per_word, NW, (size_t)lim.max_lds_per_block - kScoreScratchBytes);
+  const size_t lds_bytes = 2 * bytes_per_word * chunk_words;
+  auto kern = score_flat_kernel<GP, TT, PT>;
+  if (lds_bytes > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (int)lds_bytes) != hipSuccess)
+    return SOCKET_ERR_LAUNCH;
+  const int hsplit = (G + GP - 1) / GP;
+  // one workgroup per CU (each needs the CU's LDS to itself)
+  hipLaunchKernelGGL(kern, dim3(lim.cu_count), dim3(1024), lds_bytes, a.stream, (const TE*)a.q_probs, a.codes,
+                     a.v_norm, a.lens, a.scores, a.B, a.Hq, a.Hkv, G, a.L, a.R, a.T, a.Tcap, a.score_stride, NW,
+                     chunk_words, hsplit, 0x3f80u, (a.flags & SOCKET_SCORE_SKIP_MASKED) ? 0 : 1);
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}
+
+template <int GP, class TT>
+int dispatch_flat(const ScoreArgs& a) {
+  if constexpr (GP == 1) {
+    return SOCKET_ERR_UNSUPPORTED;
+  } else {
+    return a.P == 10 ? launch_score_flat<GP, TT, 10>(a) : launch_score_flat<GP, TT, 8>(a);
+  }
+}
+
 template <int GP, class TT>
 int dispatch_tile(const ScoreArgs& a, const ScorePlan& plan) {
   if (plan.dma) {
@@ -988,6 +1334,7 @@ template <class TT>
 int dispatch_g(const ScoreArgs& a) {
   const int G = a.Hq / a.Hkv;
   ScorePlan plan = score_plan(a.B, a.Hkv, G, a.T, a.grouped, sizeof(typename TT::elem), a.L, a.P, a.R);
+  if (flat_serves(a, sizeof(typename TT::elem))) return G == 2 ? dispatch_flat<2, TT>(a) : dispatch_flat<4, TT>(a);
   if (G == 1 || plan.solo) return dispatch_tile<1, TT>(a, plan);
   if (G == 2) return dispatch_tile<2, TT>(a, plan);
   return dispatch_tile<4, TT>(a, plan);
@@ -1052,7 +1399,7 @@ namespace {
 int score_entry(const void* q_probs, int q_dtype, const uint32_t* codes, const uint16_t* v_norm,
                 const int32_t* lens, float* scores, uint32_t* row_range, int range_parts, int B, int Hq,
                 int Hkv, int L, int P, int R, int T, int64_t Tcap, int64_t score_stride, void* stream,
-                int grouped) {
+                int grouped, int flags) {
   SOCKET_REQUIRE(q_probs && codes && v_norm && scores, SOCKET_ERR_NULL);
   SOCKET_REQUIRE(q_dtype == SOCKET_F32 || q_dtype == SOCKET_BF16, SOCKET_ERR_UNSUPPORTED);
   SOCKET_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && L > 0 && T > 0, SOCKET_ERR_SHAPE);
@@ -1067,7 +1414,7 @@ int score_entry(const void* q_probs, int q_dtype, const uint32_t* codes, const u
                  SOCKET_ERR_ALIGN);
   SOCKET_REQUIRE(Hq / Hkv <= 8, SOCKET_ERR_UNSUPPORTED);
   const ScoreArgs a{q_probs, codes, v_norm, lens, scores, B, Hq, Hkv, L, P, R, T, Tcap, score_stride,
-                    row_range, range_parts, (hipStream_t)stream, grouped};
+                    row_range, range_parts, (hipStream_t)stream, grouped, flags};
   return q_dtype == SOCKET_F32 ? dispatch_g<TabF32>(a) : dispatch_g<TabBF16>(a);
 }
 
@@ -1095,18 +1442,18 @@ extern "C" int socket_score_packed(const void* q_probs, int q_dtype, const uint3
                                    const uint16_t* v_norm, const int32_t* lens, float* scores,
                                    uint32_t* row_range, int range_parts,
                                    int B, int Hq, int Hkv, int L, int P, int R, int T,
-                                   int64_t Tcap, int64_t score_stride, void* stream) {
+                                   int64_t Tcap, int64_t score_stride, int flags, void* stream) {
   return score_entry(q_probs, q_dtype, codes, v_norm, lens, scores, row_range, range_parts, B, Hq, Hkv, L, P,
-                     R, T, Tcap, score_stride, stream, 0);
+                     R, T, Tcap, score_stride, stream, 0, flags);
 }
 
 extern "C" int socket_score_packed_grouped(const void* q_table, int q_dtype, const uint32_t* codes,
                                            const uint16_t* v_norm, const int32_t* lens, float* scores,
                                            uint32_t* row_range, int range_parts,
                                            int B, int Hq, int Hkv, int L, int P, int R, int T,
-                                           int64_t Tcap, int64_t score_stride, void* stream) {
+                                           int64_t Tcap, int64_t score_stride, int flags, void* stream) {
   return score_entry(q_table, q_dtype, codes, v_norm, lens, scores, row_range, range_parts, B, Hq, Hkv, L, P,
-                     R, T, Tcap, score_stride, stream, 1);
+                     R, T, Tcap, score_stride, stream, 1, flags);
 }
 
 extern "C" int socket_group_shape(int Hq, int Hkv, int* parts, int* width) {

@@ -277,14 +277,16 @@ def decode_prologue(qkv: torch.Tensor, freqs_cis: torch.Tensor, input_pos: torch
 @torch.no_grad()
 def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
                  lens: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                 with_range: bool = False, n_heads: Optional[int] = None):
+                 with_range: bool = False, n_heads: Optional[int] = None, skip_masked: bool = False):
     """Soft-collision scores [B,Hq,T] fp32 (row pitch padded to a multiple of 4)
     from q_probs [B,Hq,L,R] and the packed cache.  q_probs may be float32 or
     bfloat16; a bfloat16 table is read as is (the reference widens it with
     `.float()`, GPT-FAST/kernels/sparse.py:42, which changes no value) and halves
     the LDS bytes per gather.  float16 is widened to float32 first.
     with_range=True also returns the per-tile key ranges of every row (int32
-    [B,Hq,parts,2]) for `select_list(..., row_range=...)`."""
+    [B,Hq,parts,2]) for `select_list(..., row_range=...)`.
+    skip_masked=True: positions at or past `lens[b]` may be left unwritten instead of
+    set to -inf (for a consumer that reads rows only up to `lens[b]`)."""
     assert q_probs.is_cuda and q_probs.dim() in (4, 5)
     if q_probs.dtype not in (torch.float32, torch.bfloat16):
         q_probs = q_probs.float()
@@ -318,7 +320,8 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
     entry = lib().socket_score_packed_grouped if grouped else lib().socket_score_packed
     check("socket_score_packed", entry(
         ptr(q_probs), dtype_enum(q_probs.dtype), ptr(codes), ptr(v_norm), ptr(lens), ptr(out),
-        ptr(rng), parts, B, Hq, Hkv, L, int(P), R, int(T), Tcap, pitch, stream_ptr(q_probs.device)))
+        ptr(rng), parts, B, Hq, Hkv, L, int(P), R, int(T), Tcap, pitch, 1 if skip_masked else 0,
+        stream_ptr(q_probs.device)))
     if with_range:
         return out[:, :, :T], rng
     return out[:, :, :T]
@@ -382,7 +385,10 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     # (no per-tile key ranges from the scorer: the selection draws its threshold from a
     # sample of the row and only a row whose sample misleads it falls back to a pass
     # that would use them; tracking them costs the scorer more than that pass saves)
-    scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens, n_heads=q.shape[1])
+    # (positions past a sequence's length are written only when the caller gets the scores back:
+    # the selection reads a row up to the same `lens`)
+    scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens, n_heads=q.shape[1],
+                          skip_masked=not return_details)
     sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets)
     B, Hq, D = q.shape
     if _use_one_launch(q, sparse_list.shape[-1], one_launch):

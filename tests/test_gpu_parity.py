@@ -899,6 +899,83 @@ def test_decode_step_end_to_end(dev, name, T):
     # (a sanity check of the whole chain, not a parity bar)
     assert out.dtype == w.dtype
 
+# ---------------------------------------------------------------- persistent scorer
+def _definition_scores(qp, codes, vn, lens, T, G):
+    """Sequential fp32 sum over tables of gathered entries, times the value norm, -inf
+    past the length (soft_hash_collision.cu:45-53), with torch on the device."""
+    B, Hq, L, _ = qp.shape
+    want = torch.zeros(B, Hq, T, dtype=torch.float32, device=qp.device)
+    ce, qf = codes.long().repeat_interleave(G, dim=1), qp.float()
+    for l in range(L):
+        want += torch.gather(qf[:, :, l], 2, ce[:, :, l])
+    want *= vn[..., :T].float().repeat_interleave(G, dim=1)
+    if lens is not None:
+        want = want.masked_fill(torch.arange(T, device=qp.device)[None, None, :] >= lens[:, None, None], float("-inf"))
+    return want
+
+
+@pytest.mark.parametrize("B,Hkv,G,L,P,T,dt,lens_kind", [
+    (16, 4, 7, 48, 10, 16400, torch.bfloat16, "ragged"),   # two head parts per kv head, odd context
+    (16, 4, 7, 48, 10, 16400, torch.float32, "ragged"),
+    (4, 8, 4, 60, 10, 66000, torch.bfloat16, "ragged"),
+    (4, 8, 4, 60, 10, 66000, torch.float32, "edges"),
+    (8, 8, 2, 32, 8, 33000, torch.bfloat16, "edges"),      # P = 8, two heads per entry
+    (64, 2, 3, 12, 10, 17000, torch.bfloat16, "ragged"),   # the most sequences one wave ranks, a padded head group
+    (4, 8, 4, 60, 10, 65536, torch.bfloat16, "none"),      # no lengths: every row full
+    (2, 16, 4, 60, 10, 70001, torch.float32, "full"),
+])
+def test_persistent_scorer_on_ragged_batches(dev, B, Hkv, G, L, P, T, dt, lens_kind):
+    """Calls large enough for the one-workgroup-per-CU launch that is dealt from the
+    cached lengths (a tile for every CU and more, grouped table, full packed words):
+    sequences of length 0, 1, around the 512-token unit and the 8192-token tile, equal
+    to the context, or absent; with and without the -inf fill past the lengths.
+    Scores equal the definition (bit for bit with an fp32 table)."""
+    R, Hq = 1 << P, Hkv * G
+    g = torch.Generator(device=dev).manual_seed(B * 131 + T)
+    qp = (torch.rand(B, Hq, L, R, generator=g, device=dev) *
+          torch.exp(-8 * torch.rand(B, Hq, L, R, generator=g, device=dev))).to(dt)
+    codes = torch.randint(0, R, (B, Hkv, L, T), generator=g, device=dev, dtype=torch.int32).to(torch.int16)
+    Tcap = (T + 64 + 7) // 8 * 8
+    packed = torch.zeros(B, Hkv, orc.words_per_key(L, P), Tcap, dtype=torch.int32, device=dev)
+    hash_cache.pack_codes_into(codes, packed, P, t0=0)
+    vn = torch.zeros(B, Hkv, Tcap, dtype=torch.float16, device=dev)
+    vn[..., :T] = (torch.rand(B, Hkv, T, generator=g, device=dev) * 6).to(torch.float16)
+    if lens_kind == "none":
+        lens = None
+    elif lens_kind == "full":
+        lens = torch.full((B,), T, dtype=torch.int32, device=dev)
+    elif lens_kind == "edges":
+        pool = [0, 1, 3, 4, 511, 512, 513, 8191, 8192, 8193, 8704, T - 1, T, T // 2 + 2, 12345, 1025]
+        lens = torch.tensor([pool[i % len(pool)] for i in range(B)], dtype=torch.int32, device=dev).clamp_(max=T)
+    else:
+        lens = torch.randint(0, T + 1, (B,), generator=g, device=dev, dtype=torch.int32)
+        lens[0] = T
+        if B > 2:
+            lens[1] = 0
+    table = hash_cache.group_q_probs(qp, Hkv)
+    want = _definition_scores(qp, codes, vn, lens, T, G)
+    tol = 0.0 if dt == torch.float32 else 2e-6
+    got = hash_cache.score_packed(table, packed, vn, T, P, lens=lens, n_heads=Hq)
+    assert torch.equal(torch.isinf(got), torch.isinf(want))
+    rel = ((got - want).abs() / want.abs().clamp_min(1e-30)).nan_to_num(0).max().item()
+    assert rel <= tol, f"max rel diff {rel}"
+    # the reference layout goes through the tiled launches: same values
+    ref_layout = hash_cache.score_packed(qp, packed, vn, T, P, lens=lens)
+    rel = ((got - ref_layout).abs() / ref_layout.abs().clamp_min(1e-30)).nan_to_num(0).max().item()
+    assert rel <= tol
+    # without the fill: rows equal up to their lengths, nothing written past the length's float4
+    pitch = (T + 3) // 4 * 4
+    out = torch.full((B, Hq, pitch), 123.0, dtype=torch.float32, device=dev)
+    got2 = hash_cache.score_packed(table, packed, vn, T, P, lens=lens, n_heads=Hq, out=out, skip_masked=True)
+    for b in range(B):
+        n = T if lens is None else int(lens[b])
+        assert torch.equal(got2[b, :, :n], got[b, :, :n])
+        assert (out[b, :, (n + 3) // 4 * 4:T] == 123.0).all()
+    # twice in a row into the same buffer: no state is carried between launches
+    again = hash_cache.score_packed(table, packed, vn, T, P, lens=lens, n_heads=Hq)
+    assert torch.equal(again, got)
+
+
 # ---------------------------------------------------------------- randomized shapes
 @pytest.mark.parametrize("seed", [11, 12, 13])
 def test_random_shapes_score_and_select(dev, seed):

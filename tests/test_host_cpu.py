@@ -40,7 +40,7 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_status_strings_and_version(lib):
-    assert lib.socket_abi_version() == 3
+    assert lib.socket_abi_version() == 4
     seen = set()
     for st in range(0, -7, -1):
         s = lib.socket_status_string(st).decode()
@@ -62,16 +62,16 @@ def test_entry_points_reject_bad_arguments_without_a_device(lib):
     nul = ctypes.c_void_p(0)
     one = ctypes.c_void_p(16)          # non-NULL, 16-byte aligned, never dereferenced: validation fails first
     # NULL pointers
-    assert lib.socket_score_packed(nul, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_NULL
+    assert lib.socket_score_packed(nul, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 64, 64, 0, nul) == _lib.SOCKET_ERR_NULL
     assert lib.socket_select_list(nul, 64, nul, nul, nul, 0, 1, 1, 64, 4, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_NULL
     assert lib.socket_hash_keys(nul, nul, 1, 0, 0, 128, 0, 0, 128, one, one, nul, nul, 0, 1, 1, 1, 128, 60, 10, 8, nul) == _lib.SOCKET_ERR_NULL
     # shapes
-    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 5, 2, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_SHAPE    # Hq % Hkv
-    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 512, 64, 64, 64, nul) == _lib.SOCKET_ERR_SHAPE     # R < 2^P
-    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 65, 64, 68, nul) == _lib.SOCKET_ERR_SHAPE    # T > Tcap
-    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 66, 64, nul) == _lib.SOCKET_ERR_ALIGN    # Tcap % 4
-    assert lib.socket_score_packed(one, 2, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # fp16 table
-    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 16, 1, 8, 10, 1024, 64, 64, 64, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # G = 16
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 5, 2, 8, 10, 1024, 64, 64, 64, 0, nul) == _lib.SOCKET_ERR_SHAPE    # Hq % Hkv
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 512, 64, 64, 64, 0, nul) == _lib.SOCKET_ERR_SHAPE     # R < 2^P
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 65, 64, 68, 0, nul) == _lib.SOCKET_ERR_SHAPE    # T > Tcap
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 66, 64, 0, nul) == _lib.SOCKET_ERR_ALIGN    # Tcap % 4
+    assert lib.socket_score_packed(one, 2, one, one, nul, one, nul, 0, 1, 4, 1, 8, 10, 1024, 64, 64, 64, 0, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # fp16 table
+    assert lib.socket_score_packed(one, 0, one, one, nul, one, nul, 0, 1, 16, 1, 8, 10, 1024, 64, 64, 64, 0, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # G = 16
     assert lib.socket_hash_keys(one, nul, 1, 0, 0, 64, 0, 0, 64, one, one, nul, nul, 0, 1, 1, 1, 64, 60, 10, 8, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # D != 128
     assert lib.socket_hash_keys(one, nul, 1, 0, 0, 128, 0, 0, 128, one, one, nul, nul, 4, 1, 1, 8, 128, 60, 10, 8, nul) == _lib.SOCKET_ERR_SHAPE  # t0 + S > Tcap
     assert lib.socket_select_list(one, 64, nul, nul, nul, 0, 1, 1, 64, 20000, 0, 0, 1, one, 8, 8, nul, nul, 0, nul) == _lib.SOCKET_ERR_UNSUPPORTED  # M too large
