@@ -76,6 +76,7 @@ def algorithmic_bytes(w, lens=None, budgets=None):
         "score": w.Hkv * tok * (wc + 2 + 4 * G),
         "score_f32": w.Hkv * tok * (wc + 2 + 4 * G),
         "score_f32_table": w.Hkv * tok * (wc + 2 + 4 * G),
+        "score_f32_table_grouped": w.Hkv * tok * (wc + 2 + 4 * G),
         "score_reference_layout": w.Hkv * tok * (wc + 2 + 4 * G),
         "select": sel,
         "attend": w.Hq * kt * (4 * w.D + 4) + w.B * w.Hq * 4 * w.D,
@@ -303,12 +304,13 @@ class Step:
         self.abytes = algorithmic_bytes(w, None if self.lens is None else self.lens.cpu(),
                                         None if self.budgets is None else self.budgets.cpu())
         pitch = (T + 3) // 4 * 4
-        self.scores_buf = torch.empty((B, Hq, pitch), dtype=torch.float32, device=dev)
+        self.scores_buf = torch.full((B, Hq, pitch), float("-inf"), dtype=torch.float32, device=dev)
         self.new_pos = None if self.lens is None else (self.lens - w.new_keys).to(torch.int32)
         # the soft-hash table in the dtype the model produces it in: the reference's
         # soft_hash runs in the model dtype (GPT-FAST/model.py:392-401), bf16 here
         self.q_table = inp.q_probs.to(torch.bfloat16) if w.dtype == torch.bfloat16 else inp.q_probs
         self.q_table_f32 = self.q_table.float()
+        self.q_table_f32_grouped = None
         # ... and in the layout the fused soft-hash kernel writes it in (heads of a KV head
         # interleaved per bucket: the scorer's LDS image); same values
         self.q_table_grouped = hash_cache.group_q_probs(self.q_table, Hkv)
@@ -337,8 +339,15 @@ class Step:
                                     out=self.scores_buf)
 
     def k_score_grouped(self):
+        # (as the step calls it: positions past a sequence's length are not written)
         return self.hc.score_packed(self.q_table_grouped, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
-                                    out=self.scores_buf, n_heads=self.w.Hq)
+                                    out=self.scores_buf, n_heads=self.w.Hq, skip_masked=True)
+
+    def k_score_f32_grouped(self):
+        if self.q_table_f32_grouped is None:
+            self.q_table_f32_grouped = self.hc.group_q_probs(self.q_table_f32, self.w.Hkv)
+        return self.hc.score_packed(self.q_table_f32_grouped, self.codes, self.v_norm, self.w.T, self.w.P,
+                                    lens=self.lens, out=self.scores_buf, n_heads=self.w.Hq, skip_masked=True)
 
     def k_score_f32(self):
         return self.hc.score_packed(self.q_table_f32, self.codes, self.v_norm, self.w.T, self.w.P, lens=self.lens,
@@ -505,6 +514,7 @@ def measure_workload(w, dev, steps, warmup, args, full):
     if full:
         per["score_reference_layout"] = time_graph(st.k_score_ref, iters)
         per["score_f32_table"] = time_graph(st.k_score_f32, iters)
+        per["score_f32_table_grouped"] = time_graph(st.k_score_f32_grouped, iters)
     ab = st.abytes
     kernels = {k: {"us": round(v, 2), "algorithmic_MB": round(ab[k] / 1e6, 2), "gbs": round(ab[k] / v / 1e3, 1),
                    "hbm_frac": round(ab[k] / v / 1e3 / HBM_PEAK_GBS, 4)} for k, v in per.items()}

@@ -179,6 +179,14 @@ int socket_score_shape_cost(int B, int Hq, int Hkv, int T, int q_dtype, int L, i
 int socket_group_shape(int Hq, int Hkv, int* parts, int* width);
 int socket_score_prefers_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);
 int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);
+/* socket_score_persistent_serves: 1 if socket_score_packed_grouped would serve a call
+ * of this shape (without row_range) with its persistent launch -- one workgroup per
+ * CU, the token range of every (sequence, kv head, head part) dealt out by the cached
+ * lengths, no drain between tiles -- 0 if with the tiled launches, -1 for an invalid
+ * shape.  A caller that holds the table as [B,Hq,L,R] can use it to decide whether
+ * converting it with socket_group_q_probs first pays (socket_score_packed itself
+ * never takes the persistent launch: its table slices need an interleaving pass). */
+int socket_score_persistent_serves(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R);
 int socket_group_q_probs(const void* q_probs, int q_dtype, void* q_table, int B, int Hq, int Hkv,
                          int L, int R, void* stream);
 int socket_score_packed_grouped(const void* q_table, int q_dtype, const uint32_t* codes,

@@ -53,6 +53,7 @@ SIGNATURES = {
     "socket_group_shape": (_I, [_I, _I, POINTER(c_int), POINTER(c_int)]),
     "socket_score_prefers_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "socket_score_range_parts_grouped": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
+    "socket_score_persistent_serves": (_I, [_I, _I, _I, _I, _I, _I, _I, _I]),
     "socket_group_q_probs": (_I, [_P, _I, _P, _I, _I, _I, _I, _I, _P]),
     "socket_score_packed_grouped": (_I, [_P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _I, _P]),
     "socket_soft_hash_grouped": (_I, [_P, _I, _L, _L, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, c_float, c_float, _P]),

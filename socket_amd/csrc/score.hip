@@ -504,8 +504,9 @@ __device__ __forceinline__ void score_tile(
           // one that ends; since then this wave has issued one code load per word
           // and token group.  Loads retire in order, so allowing that many to be
           // outstanding, less one word's worth as a margin, means the copies have
-          // landed.
-          if (DMA) wait_vmcnt(max(0, (wend - w0 - 1) * KT4));
+          // landed (a slice of one word: no margin, its loads are pinned by the
+          // scheduling barrier that closes the word).
+          if (DMA) wait_vmcnt(max(wend - w0 - 1, 1) * KT4);
           else stage_store(w * cpw, buf ^ 1);  // the slice fetched into registers while the last one was read
           __syncthreads();
           if (nbuf == 2) buf ^= 1;
@@ -976,9 +977,11 @@ __global__ __launch_bounds__(1024) void score_flat_kernel(
       if (decltype(first)::value || w == wend) {
         // The copies of the slice that starts here were issued at the top of the one
         // that ends; since then this wave has issued one code load per word and token
-        // group.  Memory operations retire in order, so allowing that many to be
-        // outstanding, less one word's worth as a margin, means the copies have landed.
-        wait_vmcnt(max(0, ((decltype(first)::value ? NW : wend) - w0 - 1) * KT4));
+        // group (each word's, pinned before the scheduling barrier that closes it).
+        // Memory operations retire in order, so allowing that many to be outstanding --
+        // less one word's worth as a margin where the slice had more than one word --
+        // means the copies have landed.
+        wait_vmcnt(max(wend - w0 - 1, 1) * KT4);
         __syncthreads();
         buf ^= 1;
         w0 = w;
@@ -1388,6 +1391,14 @@ extern "C" int socket_score_shape_cost(int B, int Hq, int Hkv, int T, int q_dtyp
   if (cost < 0.f) return SOCKET_ERR_UNSUPPORTED;
   if (cost_us) *cost_us = cost;
   return SOCKET_OK;
+}
+
+extern "C" int socket_score_persistent_serves(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {
+  if (range_parts_of(B, Hq, Hkv, T, q_dtype, L, P, R, 1) == 0) return -1;
+  ScoreArgs a{};
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.L = L; a.P = P; a.R = R; a.T = T;
+  a.grouped = 1;
+  return flat_serves(a, q_dtype == SOCKET_F32 ? 4 : 2) ? 1 : 0;
 }
 
 extern "C" int socket_score_range_parts_grouped(int B, int Hq, int Hkv, int T, int q_dtype, int L, int P, int R) {

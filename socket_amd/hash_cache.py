@@ -149,6 +149,11 @@ def _prefers_grouped(B: int, Hq: int, Hkv: int, T: int, dtype_code: int, L: int,
     return bool(r)
 
 
+@functools.lru_cache(maxsize=4096)
+def _persistent_serves(B: int, Hq: int, Hkv: int, T: int, dtype_code: int, L: int, P: int, R: int) -> bool:
+    return lib().socket_score_persistent_serves(B, Hq, Hkv, T, dtype_code, L, P, R) == 1
+
+
 def prefers_grouped(q_bhd: torch.Tensor, planes: torch.Tensor, protos_T: torch.Tensor, n_kv_heads: int,
                     context_len: int, out_dtype: Optional[torch.dtype] = None) -> bool:
     """Which table layout `soft_hash` should write for a scorer call over
@@ -302,6 +307,12 @@ def score_packed(q_probs: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tenso
         L, R = q_probs.shape[2], q_probs.shape[3]
     else:
         B, Hq, L, R = q_probs.shape
+        if not with_range and Hq % Hkv == 0 and _persistent_serves(B, Hq, Hkv, int(T), dtype_enum(q_probs.dtype),
+                                                                   L, int(P), R):
+            # a call large enough for the persistent launch, which wants the grouped table:
+            # one pass over the table (a few percent of the scorer's bytes) buys it
+            q_probs = group_q_probs(q_probs, Hkv)
+            grouped = True
     assert codes.dtype == torch.int32 and codes.is_contiguous() and codes.shape[0] == B
     assert v_norm.dtype == torch.float16 and v_norm.is_contiguous() and tuple(v_norm.shape) == (B, Hkv, Tcap)
     assert NW == words_per_key(L, P), "codes were packed for a different (L, P)"

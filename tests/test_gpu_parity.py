@@ -959,8 +959,10 @@ def test_persistent_scorer_on_ragged_batches(dev, B, Hkv, G, L, P, T, dt, lens_k
     assert torch.equal(torch.isinf(got), torch.isinf(want))
     rel = ((got - want).abs() / want.abs().clamp_min(1e-30)).nan_to_num(0).max().item()
     assert rel <= tol, f"max rel diff {rel}"
-    # the reference layout goes through the tiled launches: same values
-    ref_layout = hash_cache.score_packed(qp, packed, vn, T, P, lens=lens)
+    # the tiled launches (asking for the key ranges keeps a call on them): same values
+    ref_layout, _ = hash_cache.score_packed(qp, packed, vn, T, P, lens=lens, with_range=True)
+    # a [B,Hq,L,R] table of this size is regrouped on the way in and served the same way
+    assert torch.equal(hash_cache.score_packed(qp, packed, vn, T, P, lens=lens), got)
     rel = ((got - ref_layout).abs() / ref_layout.abs().clamp_min(1e-30)).nan_to_num(0).max().item()
     assert rel <= tol
     # without the fill: rows equal up to their lengths, nothing written past the length's float4
