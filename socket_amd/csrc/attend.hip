@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kAttThreads) void sparse_stage1_kernel(
     // this split's result.  No fence: see store_coherent.
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    if (tid == 0) last = atomicInc(&fin.arrive[b * Hq + h], (unsigned int)(nblk - 1)) == (unsigned int)(nblk - 1);
+    if (tid == 0) last = draw_ticket(&fin.arrive[b * Hq + h], (unsigned int)(nblk - 1)) == (unsigned int)(nblk - 1);
     __syncthreads();
     if (!last) return;
     merge_splits<D, true>(mid_o + ((int64_t)b * Hq + h) * nsplit * D, mid_lse + ((int64_t)b * Hq + h) * nsplit,

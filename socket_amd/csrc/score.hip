@@ -354,7 +354,12 @@ __device__ __forceinline__ void score_tile(
     uint4 ring[kPrefetch][KT4];
     // (the first slice's copies go out ahead of the code words, so that the wait below
     // can leave all but the first word in flight)
-    if (DMA && !table_resident) dma_slice(0, 0);
+    if (DMA && !table_resident) {
+      dma_slice(0, 0);
+      // the copies are issued before the code words below: the start-up wait counts on that
+      // order, and nothing else in the source ties the two together
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int d = 0; d < kPrefetch; ++d)
 #pragma unroll
@@ -1456,21 +1461,42 @@ int score_entry(const void* q_probs, int q_dtype, const uint32_t* codes, const u
 }
 
 // [B,Hq,L,R] -> [B*Hkv*parts, L, R, width]: element (pair, part, l, r, g) is head
-// kvh*G + part*width + g of the pair, zero where that is past the group.
-template <typename TE>
+// kvh*G + part*width + g of the pair, zero where that is past the group.  A thread
+// makes one entry (the `width` heads of one bucket): reads coalesced along the
+// bucket axis of each head's row, one 4- to 16-byte store.
+template <typename TE, int WIDTH>
 __global__ __launch_bounds__(256) void group_q_probs_kernel(const TE* __restrict__ in, TE* __restrict__ out,
-                                                            int Hq, int Hkv, int G, int parts, int width,
-                                                            int64_t LR, int64_t total) {
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
-    const int g = (int)(i % width);
-    const int64_t lr = (i / width) % LR;
-    const int64_t blk = i / ((int64_t)width * LR);
-    const int part = (int)(blk % parts);
-    const int64_t pair = blk / parts;
-    const int hg = part * width + g;
-    const int b = (int)(pair / Hkv), kvh = (int)(pair % Hkv);
-    out[i] = hg < G ? in[((int64_t)b * Hq + kvh * G + hg) * LR + lr] : (TE)0;
+                                                            int Hq, int Hkv, int G, int parts, int64_t LR) {
+  const int blk = blockIdx.y;                 // (pair, part)
+  const int part = blk % parts, pair = blk / parts;
+  const int b = pair / Hkv, kvh = pair % Hkv;
+  const TE* src = in + ((int64_t)b * Hq + kvh * G + part * WIDTH) * LR;
+  TE* dst = out + (int64_t)blk * LR * WIDTH;
+  const int live = min(WIDTH, G - part * WIDTH);
+  for (int64_t lr = (int64_t)blockIdx.x * 256 + threadIdx.x; lr < LR; lr += (int64_t)gridDim.x * 256) {
+    TE e[WIDTH];
+#pragma unroll
+    for (int g = 0; g < WIDTH; ++g) e[g] = g < live ? src[(int64_t)g * LR + lr] : (TE)0;
+    typedef TE Entry __attribute__((ext_vector_type(WIDTH)));
+    Entry v;
+#pragma unroll
+    for (int g = 0; g < WIDTH; ++g) v[g] = e[g];
+    *reinterpret_cast<Entry*>(dst + lr * WIDTH) = v;
   }
+}
+
+template <typename TE>
+void launch_group_q_probs(const void* in, void* out, int B, int Hq, int Hkv, int parts, int width, int64_t LR,
+                          hipStream_t s) {
+  const int bx = (int)((LR + 255) / 256 < 64 ? (LR + 255) / 256 : 64);
+  const dim3 grid(bx, B * Hkv * parts);
+  const int G = Hq / Hkv;
+  if (width == 1)
+    hipLaunchKernelGGL((group_q_probs_kernel<TE, 1>), grid, dim3(256), 0, s, (const TE*)in, (TE*)out, Hq, Hkv, G, parts, LR);
+  else if (width == 2)
+    hipLaunchKernelGGL((group_q_probs_kernel<TE, 2>), grid, dim3(256), 0, s, (const TE*)in, (TE*)out, Hq, Hkv, G, parts, LR);
+  else
+    hipLaunchKernelGGL((group_q_probs_kernel<TE, 4>), grid, dim3(256), 0, s, (const TE*)in, (TE*)out, Hq, Hkv, G, parts, LR);
 }
 
 }  // namespace
@@ -1512,15 +1538,11 @@ extern "C" int socket_group_q_probs(const void* q_probs, int q_dtype, void* q_ta
   const int st = socket_group_shape(Hq, Hkv, &parts, &width);
   if (st != SOCKET_OK) return st;
   const int64_t LR = (int64_t)L * R;
-  const int64_t total = (int64_t)B * Hkv * parts * LR * width;
-  const int blocks = (int)((total + 255) / 256 < 65535 * 16 ? (total + 255) / 256 : 65535 * 16);
+  SOCKET_REQUIRE((int64_t)B * Hkv * parts <= 65535, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(socket_aligned16(q_table), SOCKET_ERR_ALIGN);
   hipStream_t s = (hipStream_t)stream;
-  if (q_dtype == SOCKET_F32)
-    hipLaunchKernelGGL(group_q_probs_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)q_probs,
-                       (float*)q_table, Hq, Hkv, Hq / Hkv, parts, width, LR, total);
-  else
-    hipLaunchKernelGGL(group_q_probs_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, (const uint16_t*)q_probs,
-                       (uint16_t*)q_table, Hq, Hkv, Hq / Hkv, parts, width, LR, total);
+  if (q_dtype == SOCKET_F32) launch_group_q_probs<float>(q_probs, q_table, B, Hq, Hkv, parts, width, LR, s);
+  else launch_group_q_probs<uint16_t>(q_probs, q_table, B, Hq, Hkv, parts, width, LR, s);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }

@@ -214,6 +214,36 @@ __device__ __forceinline__ float wave_reduce_to_last(float x) {
   return x;
 }
 
+// The ticket of a last-arriver hand-over between workgroups of one launch (the splits
+// of an attention row, the parts of a selection row): a wrapping increment of the row's
+// counter; whoever draws ticket `wrap` is last and finds the counter back at zero.
+// The data it hands over is published without a fence, on what gfx950 guarantees for
+// the instructions used, not on the HIP memory model (under which relaxed stores, a
+// relaxed RMW and relaxed loads are a data race):
+//   * the partial results are written with agent-scope atomic stores, which the
+//     compiler emits as write-through stores (sc1): they bypass nothing but are
+//     forwarded to the memory side of the die-local L2, and vmcnt counts them down only
+//     when that write has been acknowledged;
+//   * every lane executes s_waitcnt vmcnt(0) and the workgroup barrier before lane 0
+//     draws the ticket, so all of the workgroup's stores are acknowledged before its
+//     increment is issued; the increment is an agent-scope atomic, performed at the
+//     same memory-side point, so increments are ordered after the stores of the
+//     workgroups that issued them;
+//   * the last arriver reads with agent-scope atomic loads (sc1: they miss the local L2
+//     and are served from the memory side), after its own increment has returned.
+// A device-scope release fence in that place is correct by the model and costs a
+// write-back of the whole L2 (the scorer's 67 MB of scores at 4 x 131072 tokens: the
+// step took 315 us with it against 150).  -DSOCKET_STRICT_ATOMICS builds the ticket as an
+// acquire-release agent-scope RMW instead, for comparing results and timings; the
+// product build does not define it.
+__device__ __forceinline__ unsigned int draw_ticket(unsigned int* counter, unsigned int wrap) {
+#ifdef SOCKET_STRICT_ATOMICS
+  return __builtin_amdgcn_atomic_inc32(counter, wrap, __ATOMIC_ACQ_REL, "agent");
+#else
+  return atomicInc(counter, wrap);
+#endif
+}
+
 // 16 bytes per lane from global memory straight into LDS: lane i's bytes land at
 // lds_dst + 16 * i (lds_dst is the same for the whole wave).  Written as assembly
 // so that the compiler does not serialise later LDS reads behind it; M0, which

@@ -772,7 +772,7 @@ __global__ __launch_bounds__(kThreads) void select_list_kernel(
         // draws the last one can read every part's entries.
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        if (tid == 0) sh.last = atomicInc(&row_done[rowi], (unsigned int)(parts - 1)) == (unsigned int)(parts - 1);
+        if (tid == 0) sh.last = draw_ticket(&row_done[rowi], (unsigned int)(parts - 1)) == (unsigned int)(parts - 1);
         __syncthreads();
         if (!sh.last) return;
         const int sum = __hip_atomic_load(&row_count[rowi], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -54,6 +54,42 @@ def test_static_scratch_variant_equals_the_workspace_variant(dev):
     assert torch.equal(again, got)
 
 
+def test_one_launch_merge_over_many_rows_and_split_counts(dev):
+    """The hand-over between the splits of a row (written-through partials, a ticket per
+    row, the last arriver merges) under load: hundreds of rows whose lengths give every
+    number of running splits from 1 to the launch's maximum, calls of different shapes
+    issued back to back on one stream with no synchronisation in between, three rounds.
+    Every output must equal the two-launch result bit for bit; the first mismatch stops
+    the test and names its call."""
+    lib = _lib.lib()
+    shapes = [(8, 32, 8, 5000, 4096), (2, 32, 8, 3000, 1156), (16, 28, 4, 4000, 2100), (32, 32, 8, 900, 600),
+              (1, 32, 8, 7000, 2308)]
+    cases = []
+    for i, (B, Hq, Hkv, T, width) in enumerate(shapes):
+        g = torch.Generator().manual_seed(500 + i)
+        q = torch.randn(B, Hq, 128, generator=g).to(torch.bfloat16).to(dev)
+        k = torch.randn(B, Hkv, T, 128, generator=g).to(torch.bfloat16).to(dev)
+        v = torch.randn(B, Hkv, T, 128, generator=g).to(torch.bfloat16).to(dev)
+        sl = torch.randint(0, T, (B, Hq, width), generator=g, dtype=torch.int32).to(dev)
+        bs = lib.socket_sparse_attention_block_seq(B, Hq, width)
+        nsplit = (width + bs - 1) // bs
+        # row r runs 1 + r % nsplit splits: every count occurs, neighbours differ
+        rows = torch.arange(B * Hq)
+        ln = ((rows % nsplit) * bs + 1 + (rows * 7) % bs).clamp(max=width).to(torch.int32).view(B, Hq).to(dev)
+        want = socket_kernels.sparse_attention_fwd(q, k, v, sl, ln)
+        cases.append((q, k, v, sl, ln, want, torch.empty_like(want), nsplit))
+    assert max(c[-1] for c in cases) >= 8
+    torch.cuda.synchronize()
+    for rnd in range(3):
+        for c in cases:
+            socket_kernels.sparse_attention_fwd_static(c[0], c[1], c[2], c[3], c[4], c[6])
+        torch.cuda.synchronize()
+        for i, c in enumerate(cases):
+            assert torch.equal(c[6], c[5]), f"round {rnd}, call {i} {shapes[i]}: " \
+                                            f"{int((c[6] != c[5]).any(-1).sum())} rows differ"
+            c[6].fill_(float("nan"))
+
+
 def test_static_scratch_variant_refuses_what_does_not_fit(dev):
     lib = _lib.lib()
     B, Hq, Hkv, T, width = 64, 512, 8, 64, 4096
