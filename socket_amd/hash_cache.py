@@ -414,7 +414,7 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
 
 @functools.lru_cache(maxsize=1024)
 def step_cost_estimate(B: int, Hq: int, Hkv: int, D: int, T: int, L: int, P: int, R: int, M: int,
-                       sink: int, window: int, table_bf16: bool = True) -> Tuple[float, float]:
+                       sink: int, window: int, table_bf16: bool = True, cache_bytes: int = 2) -> Tuple[float, float]:
     """(sparse_us, dense_us): rough device time of one layer's decode attention
     over T cached tokens, for choosing between the two.  The scorer's figure is the
     library's own launch-shape estimate (`socket_score_plan_query`); the selection,
@@ -439,7 +439,7 @@ def step_cost_estimate(B: int, Hq: int, Hkv: int, D: int, T: int, L: int, P: int
     rounds = -(-rows * parts // cu)
     select = rounds * (11.0 + 3.7 * (T / parts) / 32768.0 + (3.0 if parts > 1 else 0.0))
     listed = min(T, sink + window + M)
-    esize = 2 if D * 2 <= 256 else 4     # (16-bit caches are what the decode path serves; an upper bound otherwise)
+    esize = int(cache_bytes)             # bytes per K/V element
     attend = rows * listed * (2 * D * esize + 4) / 5.2e6 + (0.0 if 2 * rows >= cu else 5.0)
     dense = B * Hkv * T * 2 * D * esize / 6.4e6 + 5.0
     launch = 4.0

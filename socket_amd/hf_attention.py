@@ -39,6 +39,7 @@ import torch.nn as nn
 from torch.nn import functional as F
 
 from . import hash_cache
+from .socket_kernels import dense_decode_fwd
 
 
 def rotate_half(x):
@@ -242,6 +243,12 @@ class SocketLlamaAttention(nn.Module):
         M = max(0, min(self._effective_size(M_cfg, T_k), T_k))
         protos_T = self.get_protos_T(self._protos_cache, P, device, k.dtype)
         q_bhd = q[:, :, 0]
+        if _dense_is_cheaper(self.config, q_bhd, k, L, P, R, T_k, sink, window, M):
+            # config.dense_below_crossover (not in the reference): exact attention over a context
+            # short enough for the dense kernel to be priced below score + select + attend
+            out_bhd = _dense_step(q_bhd, k, v, T_k)
+            out = self.o_proj(out_bhd.reshape(B, 1, -1))
+            return out, None, {"bucket_sparse": False, "mode": "dense_below_crossover", "T_k": int(T_k)}
         q_probs = _soft_hash(q_bhd, st["planes"], protos_T, Hkv, T_k)
         out_bhd = _sparse_step(q_bhd, q_probs, k, v, st, T_k, sink, window, M)
         out = self.o_proj(out_bhd.reshape(B, 1, -1))
@@ -262,6 +269,20 @@ def _hash_rows(st: dict, k_new, v_new, t0: int) -> None:
 def _soft_hash(q_bhd, planes, protos_T, n_kv_heads: int, context_len: int):
     grouped = hash_cache.prefers_grouped(q_bhd, planes, protos_T, n_kv_heads, context_len)
     return hash_cache.soft_hash(q_bhd, planes, protos_T, 0.3, n_kv_heads, grouped=grouped)
+
+
+def _dense_is_cheaper(config, q_bhd, k, L: int, P: int, R: int, T_k: int, sink: int, window: int, M: int) -> bool:
+    if not getattr(config, "dense_below_crossover", False) or not q_bhd.is_cuda:
+        return False
+    B, Hq, D = q_bhd.shape
+    sparse_us, dense_us = hash_cache.step_cost_estimate(B, Hq, k.shape[1], D, int(T_k), L, P, R, int(M), int(sink),
+                                                        int(window), q_bhd.dtype == torch.bfloat16, k.element_size())
+    return dense_us < sparse_us
+
+
+def _dense_step(q_bhd, k, v, T_k: int):
+    lengths = torch.full((q_bhd.shape[0],), int(T_k), dtype=torch.int32, device=q_bhd.device)
+    return dense_decode_fwd(q_bhd, k, v, lengths)
 
 
 def _sparse_step(q_bhd, q_probs, k, v, st: dict, T_k: int, sink: int, window: int, M: int):

@@ -235,7 +235,7 @@ def _sparse_is_slower(cfg: "ModelArgs", cache: KVCache, n_head: int) -> bool:
     B, Hkv, T, D = cache.k_cache.shape
     sparse_us, dense_us = hash_cache.step_cost_estimate(
         B, n_head, Hkv, D, T, cache.L, cache.K, cache.R, int(cfg.heavy_const), int(cfg.sink_size),
-        int(cfg.window_size), cache.k_cache.dtype == torch.bfloat16)
+        int(cfg.window_size), cache.k_cache.dtype == torch.bfloat16, cache.k_cache.element_size())
     return dense_us < sparse_us
 
 

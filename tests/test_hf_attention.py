@@ -197,6 +197,26 @@ def test_decode_branch_on_device_matches_oracle(dev, dtype, tol):
 
 
 @pytest.mark.gpu
+@torch.no_grad()
+def test_dense_below_crossover_in_the_hf_hook(dev):
+    """config.dense_below_crossover on a short context: the decode branch reports the
+    dense mode, its output is causal attention over the cache (the prefill branch's own
+    arithmetic on the same tokens), and the bucket state still receives every key."""
+    cfg = make_config(heavy_size=0.2, bucket_L=20)
+    cfg.dense_below_crossover = True
+    m = make_module(cfg, seed=3, dtype=torch.float32, device=dev)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(2, 130, 512, generator=g).to(dev)
+    cache = hf.SimpleKVCache(1, 2, 2, 128, 160, torch.float32, dev)
+    have, infos = _drive(m, x, 120, cache)
+    assert infos[-1] == {"bucket_sparse": False, "mode": "dense_below_crossover", "T_k": 130}
+    assert cache.bucket_states[0]["cached"] == 130
+    full = hf.SimpleKVCache(1, 2, 2, 128, 160, torch.float32, dev)
+    want, _ = _drive(m, x, 130, full)                      # one causal pass over all 130 tokens
+    assert float((have[:, 120:] - want[:, 120:]).abs().max()) <= 2e-3 * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.gpu
 def test_device_helpers_use_reference_layouts(dev):
     m = make_module(make_config(), device=dev)
     planes = m.get_hyper_planes(m._planes_cache, 128, 12, 8, dev, torch.float32, m._rng(dev))
