@@ -47,15 +47,17 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
-# HBM bytes per launch of the scorer from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of `bench.py --only score_grouped` (profiles/score_packed_c3_hbm_counters.txt
-# holds the commands, the raw counters and the calibration), keyed by workload;
-# None until a counter run for that workload has been recorded there.  The profiler
-# cannot run inside this process, so the figure is a recorded one and says so.
-MEASURED_TRAFFIC_BYTES = {"c3": int(187240 * 1024 * 2.000 + 65618 * 1024 * 1.000)}
+# HBM bytes per launch of the scorer from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --workload W --only score_grouped` (profiles/score_flat_c3_hbm_counters.txt and
+# profiles/score_flat_c5_hbm_counters.txt hold the commands, the raw counters and the
+# calibration), keyed by workload; None until a counter run for that workload has been
+# recorded there.  The profiler cannot run inside this process, so the figure is a
+# recorded one and says so.
+MEASURED_TRAFFIC_BYTES = {"c3": int(175940.4 * 1024 * 2.000 + 65569.8 * 1024 * 1.000),
+                          "c5": int(150077.5 * 1024 * 2.000 + 94275.5 * 1024 * 1.000)}
 MEASURED_TRAFFIC_SOURCE = ("recorded, not measured in this run: rocprofv3 --pmc FETCH_SIZE (x2.000, calibrated on a 1 GiB "
-                           "read stream of the same request width) + WRITE_SIZE (x1.000, device copy); "
-                           "profiles/score_packed_c3_hbm_counters.txt")
+                           "read stream of the same request width) + WRITE_SIZE (x1.000, device copy) of "
+                           "score_flat_kernel; profiles/score_flat_{w}_hbm_counters.txt")
 
 
 def algorithmic_bytes(w, lens=None, budgets=None):
@@ -744,11 +746,12 @@ def main():
         "data": "synthetic",
         "config": {"workload": rec["workload"], "layers_timed": 1,
                    "new_keys_hashed_per_step": rec["new_keys_hashed_per_step"], "launch": rec["launch"]},
-        "roofline": {"kernel": "score_packed_kernel", "bound": "hbm",
+        "roofline": {"kernel": "score_flat_kernel" if st.use_grouped else "score_packed_kernel", "bound": "hbm",
                      "achieved": round(ab["score"] / per["score"] / 1e3, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(ab["score"] / per["score"] / 1e3 / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
-                     "traffic_source": MEASURED_TRAFFIC_SOURCE if MEASURED_TRAFFIC_BYTES.get(w.name) else None},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(w.name) if st.use_grouped else None,
+                     "traffic_source": (MEASURED_TRAFFIC_SOURCE.format(w=w.name)
+                                        if MEASURED_TRAFFIC_BYTES.get(w.name) and st.use_grouped else None)},
         "kernels": rec["kernels"],
         "kernel_timing": rec["kernel_timing"],
         "power_state": rec["power_state"],
