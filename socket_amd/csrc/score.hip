@@ -217,7 +217,11 @@ __device__ __forceinline__ void score_tile(
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
     int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf,
     int n_tiles, uint32_t bf16_one, uint32_t* __restrict__ row_range, int hsplit, int pair, int tile,
-    bool table_resident, int red_off) {
+    bool table_resident, int red_off, int tile_tokens) {
+  // tile_tokens: tokens between the starts of two tiles, a multiple of 4 and at most the
+  // 4 * KT4 * THREADS a workgroup can hold (less: the lanes past it stay idle, so that a
+  // context which overhangs a whole number of tiles by a little is cut into one more, equal,
+  // tile per row rather than scored by half as many workgroups of the next size up)
   // MODE: 0 = table in the reference layout [B,Hq,L,R], interleaved while staged;
   // 1 = grouped table, copied through registers; 2 = grouped table, copied from
   // global memory straight into LDS
@@ -249,11 +253,13 @@ __device__ __forceinline__ void score_tile(
   const int tid = threadIdx.x;
   const int len = lens ? min(lens[b], T) : T;
 
-  if (tile * TW >= len) {
+  const int tile0 = tile * tile_tokens;               // first token of the tile
+  const int tile_end = min(T, tile0 + tile_tokens);   // one past its last
+  if (tile0 >= len) {
     // nothing cached this far out for this sequence: the tile is all masked
     for (int g = 0; g < G; ++g) {
-      float* dst = scores + ((int64_t)(head0 + g)) * score_stride + tile * TW;
-      const int n = min(TW, T - tile * TW);
+      float* dst = scores + ((int64_t)(head0 + g)) * score_stride + tile0;
+      const int n = tile_end - tile0;
       for (int t = tid * 4; t < n; t += THREADS * 4) {
         if (t + 4 <= n) {
           store_stream16(dst + t, -INFINITY, -INFINITY, -INFINITY, -INFINITY);
@@ -283,9 +289,9 @@ __device__ __forceinline__ void score_tile(
   bool live[KT4];
 #pragma unroll
   for (int j = 0; j < KT4; ++j) {
-    tbase[j] = tile * TW + j * (CT * 4) + tid * 4;
-    live[j] = tid < CT && tbase[j] < T;
-    tsafe[j] = live[j] ? tbase[j] : tile * TW;
+    tbase[j] = tile0 + j * (CT * 4) + tid * 4;
+    live[j] = tid < CT && tbase[j] < tile_end;
+    tsafe[j] = live[j] ? tbase[j] : tile0;
   }
 
   // The value norms of the lane's tokens are requested now and used in the epilogue:
@@ -320,7 +326,7 @@ __device__ __forceinline__ void score_tile(
   // gather (a ragged batch; a context that overhangs the last full tile by a
   // little): it only takes its share of the table copies and meets the barriers.
   // The test is wave-uniform and made once, outside the gather loop.
-  const bool wave_active = !DMA || tile * TW + (tid >> 6) * 256 < len;
+  const bool wave_active = !DMA || tile0 + (tid >> 6) * 256 < min(len, tile_end);
   if (!wave_active) {
     const int chunk_tables_ = chunk_words * cpw;
     if (!table_resident) {
@@ -736,7 +742,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     float* __restrict__ scores, int Hq, int Hkv, int G, int L, int P_rt, int R, int T,
     int64_t Tcap, int64_t score_stride, int NW, int chunk_words, int nbuf, int n_pairs,
     int n_tiles, int n_launch_tiles, int xcd_remap, uint32_t bf16_one, uint32_t* __restrict__ row_range,
-    int hsplit, int red_off) {
+    int hsplit, int red_off, int tile_tokens) {
   // Workgroup -> (pair, tile).  Workgroups are dealt to the 8 XCDs round-robin
   // by linear id; with the remap all tiles of one (b, kv head), and all the
   // workgroups that share its query heads out between them, land on one XCD: its
@@ -759,7 +765,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
   if (pair >= n_pairs) return;
   score_tile<GP, TT, KT4, THREADS, PT, MODE>(q_probs, codes, v_norm, lens, scores, Hq, Hkv, G, L, P_rt, R, T, Tcap,
                                              score_stride, NW, chunk_words, nbuf, n_tiles, bf16_one, row_range,
-                                             hsplit, pair, tile, false, red_off);
+                                             hsplit, pair, tile, false, red_off, tile_tokens);
   // A short last tile is not given a workgroup of its own (a whole extra round of
   // them on a full chip): the workgroup of the tile before it, with the table
   // still in LDS, does it as well.  Only where one workgroup holds a whole table.
@@ -767,7 +773,7 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
     if (n_launch_tiles < n_tiles && tile == n_launch_tiles - 1)
       score_tile<GP, TT, KT4, THREADS, PT, MODE>(q_probs, codes, v_norm, lens, scores, Hq, Hkv, G, L, P_rt, R, T,
                                                  Tcap, score_stride, NW, chunk_words, nbuf, n_tiles, bf16_one,
-                                                 row_range, hsplit, pair, tile + 1, true, red_off);
+                                                 row_range, hsplit, pair, tile + 1, true, red_off, tile_tokens);
   }
 }
 
@@ -1157,7 +1163,21 @@ int launch_score_packed(const ScoreArgs& a) {
       return SOCKET_ERR_LAUNCH;
   }
   constexpr int TW = THREADS * 4 * KT4;
-  const int n_tiles = (a.T + TW - 1) / TW;
+  // Tokens per tile: what a workgroup holds -- unless that leaves CUs without a workgroup
+  // and cutting every row into as many equal tiles as there are CUs for it keeps more than
+  // half of each workgroup's waves in work (a 65536-token context grown by a few hundred
+  // tokens: 17 tiles of 4096 per row on 136 of 256 CUs, or 29 of 2304 on 232).  Only where
+  // idle lanes cost nothing else: one token group per lane, slices copied global -> LDS.
+  int tile_tokens = TW;
+  if (KT4 == 1 && DMA && GP > 1 && !a.row_range) {
+    const int64_t rows = (int64_t)a.B * a.Hkv * ((G + GP - 1) / GP);
+    const int per_row = (int)(lim.cu_count / rows);
+    if (rows * ((a.T + TW - 1) / TW) < lim.cu_count && per_row > (a.T + TW - 1) / TW) {
+      const int even = (((a.T + per_row - 1) / per_row) + 255) / 256 * 256;
+      if (even < TW && 2 * even > TW) tile_tokens = even;
+    }
+  }
+  const int n_tiles = (a.T + tile_tokens - 1) / tile_tokens;
   if (a.row_range && a.range_parts != n_tiles) return SOCKET_ERR_SHAPE;
   const int hsplit = (G + GP - 1) / GP;
   const int n_pairs = a.B * a.Hkv * hsplit;
@@ -1170,7 +1190,7 @@ int launch_score_packed(const ScoreArgs& a) {
   hipLaunchKernelGGL(kern, dim3(n_wg), dim3(THREADS), lds_bytes, a.stream, (const TE*)a.q_probs,
                      a.codes, a.v_norm, a.lens, a.scores, a.Hq, a.Hkv, G, a.L, a.P, a.R, a.T, a.Tcap,
                      a.score_stride, NW, chunk_words, nbuf, n_pairs, n_tiles, n_launch_tiles, xcd_remap,
-                     0x3f80u, a.row_range, hsplit, (int)table_bytes);
+                     0x3f80u, a.row_range, hsplit, (int)table_bytes, tile_tokens);
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }

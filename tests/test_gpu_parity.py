@@ -797,6 +797,9 @@ def test_bf16_soft_hash_against_the_reference_dtype_chain(dev, name, Hq, Hkv, L,
     (8, 32, 8, 60, 10, 70000, torch.bfloat16),   # a tile for every CU: slices go straight from global memory to LDS
     (8, 56, 8, 20, 10, 33000, torch.float32),    # the same with fp32 entries and split head groups
     (16, 16, 16, 7, 8, 9000, torch.bfloat16),    # ... and one head per group, P = 8
+    (1, 32, 8, 60, 10, 65792, torch.bfloat16),   # a context that overhangs 16 tiles of 4096 by a little: 29 even tiles per row
+    (1, 32, 8, 60, 10, 100000, torch.float32),   # ... 25 tiles of 4096 on 200 CUs, or 31 of 3328
+    (2, 14, 2, 48, 10, 50000, torch.bfloat16),   # ... with two head parts per kv head
 ])
 def test_grouped_table_layout_gives_identical_scores(dev, B, Hq, Hkv, L, P, T, dtype):
     """The grouped table (converter and fused producer) is a relayout only: the
@@ -821,6 +824,11 @@ def test_grouped_table_layout_gives_identical_scores(dev, B, Hq, Hkv, L, P, T, d
     packed = _packed_cache(codes, P, Tcap, dev)
     a, ra = hash_cache.score_packed(q_probs, packed, vn.to(dev), T, P, lens=lens, with_range=True)
     b, rb = hash_cache.score_packed(table, packed, vn.to(dev), T, P, lens=lens, with_range=True, n_heads=Hq)
+    # without the key ranges the launch is free to cut the rows otherwise (even tiles for a
+    # context that overhangs a whole number of them, the persistent launch): same scores
+    c = hash_cache.score_packed(table, packed, vn.to(dev), T, P, lens=lens, n_heads=Hq)
+    assert torch.equal(torch.isinf(c), torch.isinf(b))
+    assert ((c - b).abs() / b.abs().clamp_min(1e-30)).nan_to_num(0).max() <= (0.0 if dtype == torch.float32 else 2e-6)
     # A short context with few kv heads is scored from the [B,Hq,L,R] table one
     # head per workgroup, with plain fp32 adds; the grouped table always goes
     # through the several-heads-at-once accumulate, whose last-place rounding can
