@@ -799,18 +799,21 @@ __global__ __launch_bounds__(THREADS) void score_packed_kernel(
 // full (L a multiple of 32/P), a word count that is a multiple of the ring depth,
 // at most 64 sequences (one wave ranks their lengths).
 // ---------------------------------------------------------------------------
-constexpr int kFlatUnit = 512;
-constexpr int kFlatTileUnits = 16;
+constexpr int kFlatTileUnits = 16;   // waves of a workgroup: units of a full tile
 constexpr int kFlatPrefetch = 4;
 
-template <int GP, class TT, int PT>
+// KT4: token groups (of 256) per wave and tile: 2 (units of 512, tiles of 8192) where every CU
+// has a tile or more, 1 (units of 256, tiles of 4096) below that, so that the waves of a
+// workgroup stay in work when there are fewer tokens per CU.
+template <int GP, class TT, int PT, int KT4>
 __global__ __launch_bounds__(1024) void score_flat_kernel(
     const typename TT::elem* __restrict__ q_table, const uint32_t* __restrict__ codes,
     const uint16_t* __restrict__ v_norm, const int32_t* __restrict__ lens, float* __restrict__ scores,
     int B, int Hq, int Hkv, int G, int L, int R, int T, int64_t Tcap, int64_t score_stride, int NW,
     int chunk_words, int hsplit, uint32_t bf16_one, int fill_masked, int spread) {
   typedef typename TT::elem TE;
-  constexpr int THREADS = 1024, KT4 = 2, kPrefetch = kFlatPrefetch;
+  constexpr int THREADS = 1024, kPrefetch = kFlatPrefetch;
+  constexpr int kFlatUnit = 256 * KT4;               // tokens one wave scores in a tile
   constexpr int CPW = 32 / PT, EB = GP * (int)sizeof(TE);
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const Bf16Select sel = make_bf16_select(bf16_one);
@@ -818,7 +821,7 @@ __global__ __launch_bounds__(1024) void score_flat_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int VS = Hkv * hsplit;                      // rows of the flattened space per sequence
   const int chunk_elems = chunk_words * CPW * R * GP;
-  const int offl = wave * kFlatUnit + lane * 4;      // the lane's first token in a tile (group 1: + 256)
+  const int offl = wave * kFlatUnit + lane * 4;      // the lane's first token in a tile (group j: + 256 j)
 
   // ---- this workgroup's stretch of the flattened unit space -----------------------------
   int len_l = 0;                                     // lane l: cached length of sequence l
@@ -1311,10 +1314,14 @@ int flat_chunk_words(size_t bytes_per_word, int NW, size_t lds_budget) {
   return cw;
 }
 
-// Whether the persistent kernel serves this call: the operands it is written for, and
-// at least one 8192-token tile for every CU (below that the launches that shrink the
-// tile to fill the chip do better).
-bool flat_serves(const ScoreArgs& a, size_t elem_bytes) {
+// Whether the persistent kernel serves this call: the operands it is written for, and at
+// least a quarter of an 8192-token tile for every CU (measured against the tiled launches on
+// 256 CUs, bf16 table of 4 heads x 60 tables: 8 rows x 131072 tokens 24.4 against 26.4 us,
+// 16 rows x 65536 24.4 against 27.5, 8 rows x 65536 19.1 against 20.3; below that the
+// launches that shrink the workgroup with the tile do as well).
+constexpr int kFlatMinTilesNum = 4;
+// (groups_out: token groups per wave the launch should use)
+bool flat_serves(const ScoreArgs& a, size_t elem_bytes, int* groups_out = nullptr) {
   const SocketDeviceLimits& lim = socket_device_limits();
   const int G = a.Hq / a.Hkv;
   if (!a.grouped || a.row_range || G < 2 || a.B > 64 || (a.P != 8 && a.P != 10)) return false;
@@ -1324,10 +1331,11 @@ bool flat_serves(const ScoreArgs& a, size_t elem_bytes) {
   const size_t bytes_per_word = (size_t)cpw * a.R * width * elem_bytes;
   if (flat_chunk_words(bytes_per_word, NW, (size_t)lim.max_lds_per_block - kScoreScratchBytes) < 1) return false;
   const int64_t tiles = (int64_t)a.B * a.Hkv * hsplit * ((a.T + 8191) / 8192);
-  return tiles >= lim.cu_count;
+  if (groups_out) *groups_out = tiles >= lim.cu_count ? 2 : 1;
+  return kFlatMinTilesNum * tiles >= lim.cu_count;
 }
 
-template <int GP, class TT, int PT>
+template <int GP, class TT, int PT, int KT4>
 int launch_score_flat(const ScoreArgs& a) {
   typedef typename TT::elem TE;
   const SocketDeviceLimits& lim = socket_device_limits();
@@ -1337,7 +1345,7 @@ int launch_score_flat(const ScoreArgs& a) {
   const size_t bytes_per_word = (size_t)cpw * a.R * GP * sizeof(TE);
   const int chunk_words = flat_chunk_words(bytes_per_word, NW, (size_t)lim.max_lds_per_block - kScoreScratchBytes);
   const size_t lds_bytes = 2 * bytes_per_word * chunk_words;
-  auto kern = score_flat_kernel<GP, TT, PT>;
+  auto kern = score_flat_kernel<GP, TT, PT, KT4>;
   if (lds_bytes > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                           (int)lds_bytes) != hipSuccess)
@@ -1366,7 +1374,10 @@ int dispatch_flat(const ScoreArgs& a) {
   if constexpr (GP == 1) {
     return SOCKET_ERR_UNSUPPORTED;
   } else {
-    return a.P == 10 ? launch_score_flat<GP, TT, 10>(a) : launch_score_flat<GP, TT, 8>(a);
+    int groups = 2;
+    flat_serves(a, sizeof(typename TT::elem), &groups);
+    if (groups == 2) return a.P == 10 ? launch_score_flat<GP, TT, 10, 2>(a) : launch_score_flat<GP, TT, 8, 2>(a);
+    return a.P == 10 ? launch_score_flat<GP, TT, 10, 1>(a) : launch_score_flat<GP, TT, 8, 1>(a);
   }
 }
 

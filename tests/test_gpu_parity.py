@@ -931,10 +931,14 @@ def _definition_scores(qp, codes, vn, lens, T, G):
     (64, 2, 3, 12, 10, 17000, torch.bfloat16, "ragged"),   # the most sequences one wave ranks, a padded head group
     (4, 8, 4, 60, 10, 65536, torch.bfloat16, "none"),      # no lengths: every row full
     (2, 16, 4, 60, 10, 70001, torch.float32, "full"),
+    (1, 8, 4, 60, 10, 131072, torch.bfloat16, "ragged"),   # half a tile per CU: one token group per wave
+    (2, 8, 4, 60, 10, 40000, torch.float32, "edges"),      # ... a third
+    (1, 8, 4, 60, 10, 65792, torch.bfloat16, "full"),      # ... a quarter, and a context that overhangs the tiles
+    (3, 4, 7, 48, 10, 50000, torch.bfloat16, "ragged"),    # ... with two head parts
 ])
 def test_persistent_scorer_on_ragged_batches(dev, B, Hkv, G, L, P, T, dt, lens_kind):
     """Calls large enough for the one-workgroup-per-CU launch that is dealt from the
-    cached lengths (a tile for every CU and more, grouped table, full packed words):
+    cached lengths (a quarter of a tile for every CU and more, grouped table, full packed words):
     sequences of length 0, 1, around the 512-token unit and the 8192-token tile, equal
     to the context, or absent; with and without the -inf fill past the lengths.
     Scores equal the definition (bit for bit with an fp32 table)."""
