@@ -1315,11 +1315,13 @@ int flat_chunk_words(size_t bytes_per_word, int NW, size_t lds_budget) {
 }
 
 // Whether the persistent kernel serves this call: the operands it is written for, and at
-// least a quarter of an 8192-token tile for every CU (measured against the tiled launches on
-// 256 CUs, bf16 table of 4 heads x 60 tables: 8 rows x 131072 tokens 24.4 against 26.4 us,
-// 16 rows x 65536 24.4 against 27.5, 8 rows x 65536 19.1 against 20.3; below that the
-// launches that shrink the workgroup with the tile do as well).
-constexpr int kFlatMinTilesNum = 4;
+// least a sixteenth of an 8192-token tile for every CU, i.e. two waves' worth of tokens per
+// workgroup (measured against the tiled launches on 256 CUs, bf16 table of 4 heads x 60
+// tables, rows x tokens: 8 x 131072 24.6 against 26.4 us, 16 x 65536 24.5 against 27.5,
+// 8 x 65536 17.3 against 20.3, 8 x 32768 16.6 against 18.6, 8 x 16384 15.9 against 18.0;
+// 8 x 8192 the same 17.6: there every launch is the ~17 us it takes to pass the table
+// through LDS in seven slices, one copy latency and one barrier each).
+constexpr int kFlatMinTilesNum = 16;
 // (groups_out: token groups per wave the launch should use)
 bool flat_serves(const ScoreArgs& a, size_t elem_bytes, int* groups_out = nullptr) {
   const SocketDeviceLimits& lim = socket_device_limits();
