@@ -375,7 +375,8 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
                        v_cache: torch.Tensor, codes: torch.Tensor, v_norm: torch.Tensor, T: int, P: int,
                        sink: int, window: int, M: int, lens: Optional[torch.Tensor] = None,
                        budgets: Optional[torch.Tensor] = None,
-                       return_details: bool = False, one_launch: Optional[bool] = None):
+                       return_details: bool = False, one_launch: Optional[bool] = None,
+                       scores_buf: Optional[torch.Tensor] = None):
     """One decode step of sparse attention for one layer: score every cached key,
     select top-M + sink + window, attend over the selected rows.
 
@@ -392,13 +393,18 @@ def sparse_decode_step(q: torch.Tensor, q_probs: torch.Tensor, k_cache: torch.Te
     output, bit for bit).  Replays of graphs that hold this step must not overlap
     on one GPU.  True forces the one-launch form (the caller answers for the
     serialisation), False forbids it.
+
+    `scores_buf`: an fp32 [B, Hq, T rounded up to 4] tensor to score into (67 MB at
+    4 x 32 heads x 131072 tokens); without it the step allocates one per call, which an
+    eager serving loop may want to avoid (under graph capture the allocation is the
+    graph pool's and costs nothing per replay).
     """
     # (no per-tile key ranges from the scorer: the selection draws its threshold from a
     # sample of the row and only a row whose sample misleads it falls back to a pass
     # that would use them; tracking them costs the scorer more than that pass saves)
     # (positions past a sequence's length are written only when the caller gets the scores back:
     # the selection reads a row up to the same `lens`)
-    scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens, n_heads=q.shape[1],
+    scores = score_packed(q_probs, codes, v_norm, T, P, lens=lens, n_heads=q.shape[1], out=scores_buf,
                           skip_masked=not return_details)
     sparse_list, sparse_len = select_list(scores, sink, window, M, lens=lens, budgets=budgets)
     B, Hq, D = q.shape
