@@ -435,6 +435,17 @@ int socket_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t 
 int socket_gemv_bf16(const void* x, int64_t x_stride, const void* w, const void* w_gate, void* y,
                      int64_t y_stride, int M, int N, int K, void* stream);
 
+/* socket_add_rmsnorm followed by socket_gemv_bf16 on its output, as one launch: every
+ * workgroup works out h = x + residual and RMSNorm(h) * norm_weight for itself (the same
+ * arithmetic in the same order: results equal the two launches bit for bit) and multiplies
+ * from there.  x, residual, h_out [M,K] and y [M,N] contiguous bf16, K <= 8192; residual and
+ * h_out are given together or not at all (without them h is x), and h_out must not overlap
+ * x or residual (other workgroups are still reading them when it is written).  Replaces
+ * RMSNorm + nn.Linear of a decode step (GPT-FAST/model.py:603-614 with :436 and :599-600). */
+int socket_norm_gemv_bf16(const void* x, const void* residual, const void* norm_weight, float eps,
+                          void* h_out, const void* w, const void* w_gate, void* y, int M, int N, int K,
+                          void* stream);
+
 /* Block-sparse prefill attention: out[b,h,row,:] = softmax over the listed key
  * blocks (causal inside them) of q.k^T / sqrt(D), times v.  q, k, v, out are
  * [B,H,T,D] views (element strides for dims 0-2, last dim contiguous), bf16 or

@@ -68,6 +68,7 @@ SIGNATURES = {
     "socket_add_rmsnorm": (_I, [_P, _P, _P, _P, _P, _I, _L, _I, c_float, _P]),
     "socket_silu_mul": (_I, [_P, _P, _P, _I, _L, _P]),
     "socket_gemv_bf16": (_I, [_P, _L, _P, _P, _P, _L, _I, _I, _I, _P]),
+    "socket_norm_gemv_bf16": (_I, [_P, _P, _P, c_float, _P, _P, _P, _P, _I, _I, _I, _P]),
     "socket_attend_stage1": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L,
                                   _P, _L, _L, _P, _L, _L, _P, _P,
                                   _I, _I, _I, _I, _I, _I, _I, _I, _P]),

@@ -219,6 +219,7 @@ __global__ void silu_mul_kernel(const void* __restrict__ a, const void* __restri
 constexpr int kGemvThreads = 256;
 constexpr int kGemvUnroll = 4;
 constexpr int kGemvStep = 64 * 8;  // elements of a row per wave and step
+constexpr int kGemvWgPerCu = 4;    // workgroups per CU of the persistent launch
 
 template <int M, bool GATE>
 __global__ __launch_bounds__(kGemvThreads) void gemv_bf16_kernel(
@@ -276,6 +277,176 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_bf16_kernel(
       y[(int64_t)m * y_stride + n] = f32_to_bf16_bits(r);
     }
   }
+}
+
+// The product with the RMSNorm that feeds it (and the residual add before that) in the same
+// launch.  The vector is RMSNorm(x + r) * nw, worked out by every workgroup for itself while
+// its first weight vectors are on their way -- h = x + r, xn = round(h * rsqrt(mean(h^2) + eps))
+// * nw, rounded: lane for lane and sum for sum what add_rmsnorm_kernel computes -- and kept in
+// LDS (M rows of K).  So that few workgroups pay for it the launch is persistent: a few
+// workgroups per CU, wave g of the launch takes output features g, g + waves, g + 2 waves, ...;
+// its weight vectors run through two register buffers, the next 2048 elements of its row -- or
+// the first of its next row -- requested before the current ones are multiplied, so a wave
+// streams without a gap from its first row to its last.  A lane adds its products in the
+// order of gemv_bf16_kernel: the result equals the two launches bit for bit.  Workgroup 0
+// writes h.  (On 256 CUs, one row of 4096: 6144 outputs 11.6 against 13.7 us for the two
+// launches, 2 x 14336 gated 39.8 against 41.9; one workgroup per four outputs, as
+// gemv_bf16_kernel has them, pays for the norm 1536 and 3584 times and is no faster than
+// two launches; without a norm to share, the short-lived workgroups of gemv_bf16_kernel are
+// the faster form by 0.5-1 us.)
+template <int M, bool GATE>
+__global__ __launch_bounds__(kGemvThreads) void norm_gemv_rows_kernel(
+    const uint16_t* __restrict__ x, int64_t x_stride, const uint16_t* __restrict__ r,
+    const uint16_t* __restrict__ nw, float eps, uint16_t* __restrict__ h_out, const uint16_t* __restrict__ w,
+    const uint16_t* __restrict__ wg, uint16_t* __restrict__ y, int64_t y_stride, int N, int K) {
+  static_assert(kGemvThreads == kNormThreads, "the norm's lane map");
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  typedef DType_bf16 DT;
+  constexpr int E = DT::kPer16B;
+  constexpr int kChunk = kGemvStep * kGemvUnroll;
+  extern __shared__ __attribute__((aligned(16))) uint16_t xs[];   // [M][K]
+  __shared__ float red[M][kNormThreads / SOCKET_WAVE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int waves = gridDim.x * (kGemvThreads / 64);
+  int n = blockIdx.x * (kGemvThreads / 64) + wave;   // (wave-uniform)
+  const int nk = K / kChunk;
+  u32x4 wa[kGemvUnroll], ga[kGemvUnroll], wb[kGemvUnroll], gb[kGemvUnroll];
+  auto fetch = [&](u32x4 (&wv)[kGemvUnroll], u32x4 (&gv)[kGemvUnroll], int row, int kc) __attribute__((always_inline)) {
+    const int64_t at = (int64_t)row * K + kc * kChunk + lane * 8;
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      wv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(w + at + u * kGemvStep));
+      if (GATE) gv[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wg + at + u * kGemvStep));
+    }
+  };
+  if (n < N) fetch(wa, ga, n, 0);
+  // ---- the vector into LDS ----
+  const int nvec = K / E;
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    const int64_t row = (int64_t)m * x_stride;
+    float hreg[kNormVecs][E];
+    uint4 wraw[kNormVecs];   // (the norm's weights, requested with the row instead of after the barrier)
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < kNormVecs; ++k) {
+      const int v = tid + k * kNormThreads;
+      if (v < nvec) wraw[k] = *reinterpret_cast<const uint4*>(nw + (int64_t)v * E);
+    }
+#pragma unroll
+    for (int k = 0; k < kNormVecs; ++k) {
+      const int v = tid + k * kNormThreads;
+      if (v < nvec) {
+        unpack16<DT>(*reinterpret_cast<const uint4*>(x + row + (int64_t)v * E), hreg[k]);
+        if (r) {
+          float rr[E];
+          unpack16<DT>(*reinterpret_cast<const uint4*>(r + row + (int64_t)v * E), rr);
+#pragma unroll
+          for (int e = 0; e < E; ++e) hreg[k][e] = rnd<DT>(hreg[k][e] + rr[e]);
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) ss += hreg[k][e] * hreg[k][e];
+      }
+    }
+    ss = wave_reduce_to_last<false>(ss);
+    if (lane == 63) red[m][wave] = ss;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int k = 0; k < kNormThreads / SOCKET_WAVE; ++k) tot += red[m][k];
+    const float rs = rsqrtf(tot / (float)K + eps);
+#pragma unroll
+    for (int k = 0; k < kNormVecs; ++k) {
+      const int v = tid + k * kNormThreads;
+      if (v < nvec) {
+        float ww[E], yn[E];
+        unpack16<DT>(wraw[k], ww);
+#pragma unroll
+        for (int e = 0; e < E; ++e) yn[e] = rnd<DT>(hreg[k][e] * rs) * ww[e];
+        if (h_out && blockIdx.x == 0) store16<DT>(h_out, row + (int64_t)v * E, hreg[k]);
+        store16<DT>(xs, (int64_t)m * K + (int64_t)v * E, yn);
+      }
+    }
+  }
+  __syncthreads();
+  // ---- the rows of this wave ----
+  float acc[M], accg[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) acc[m] = accg[m] = 0.f;
+  int kc = 0;
+  // one chunk: request the one after it into the other buffers, multiply this one, and at a
+  // row's end reduce over the lanes and store
+  auto step = [&](u32x4 (&cw)[kGemvUnroll], u32x4 (&cg)[kGemvUnroll], u32x4 (&nwv)[kGemvUnroll],
+                  u32x4 (&ngv)[kGemvUnroll]) __attribute__((always_inline)) {
+    const bool row_ends = kc + 1 == nk;
+    const int n2 = row_ends ? n + waves : n, kc2 = row_ends ? 0 : kc + 1;
+    if (n2 < N) fetch(nwv, ngv, n2, kc2);
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const uint4 xv = *reinterpret_cast<const uint4*>(xs + (int64_t)m * K + kc * kChunk + lane * 8 + u * kGemvStep);
+        const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float x0 = __uint_as_float(xw[i] << 16), x1 = __uint_as_float(xw[i] & 0xffff0000u);
+          acc[m] = fmaf(__uint_as_float(cw[u][i] << 16), x0, acc[m]);
+          acc[m] = fmaf(__uint_as_float(cw[u][i] & 0xffff0000u), x1, acc[m]);
+          if (GATE) {
+            accg[m] = fmaf(__uint_as_float(cg[u][i] << 16), x0, accg[m]);
+            accg[m] = fmaf(__uint_as_float(cg[u][i] & 0xffff0000u), x1, accg[m]);
+          }
+        }
+      }
+    }
+    if (row_ends) {
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float o = wave_reduce_to_last<false>(acc[m]);
+        if (GATE) {
+          const float gsum = wave_reduce_to_last<false>(accg[m]);
+          const float a = rnd<DType_bf16>(o);
+          o = rnd<DType_bf16>(a / (1.f + expf(-a))) * rnd<DType_bf16>(gsum);
+        }
+        if (lane == 63) y[(int64_t)m * y_stride + n] = f32_to_bf16_bits(o);
+        acc[m] = accg[m] = 0.f;
+      }
+    }
+    n = n2;
+    kc = kc2;
+  };
+  while (n < N) {
+    step(wa, ga, wb, gb);
+    if (n >= N) break;
+    step(wb, gb, wa, ga);
+  }
+}
+
+template <int M>
+int launch_norm_gemv_rows(const uint16_t* x, int64_t xs, const uint16_t* r, const uint16_t* nw, float eps,
+                          uint16_t* h_out, const uint16_t* w, const uint16_t* wg, uint16_t* y, int64_t ys, int N,
+                          int K, hipStream_t s) {
+  const SocketDeviceLimits& lim = socket_device_limits();
+  const size_t lds = (size_t)M * K * 2;
+  if (lds + 256 > (size_t)lim.max_lds_per_block) return SOCKET_ERR_UNSUPPORTED;
+  // kGemvWgPerCu workgroups per CU (2: 12.1 / 41.4 us for the two shapes above, 3: 12.0 / 41.0,
+  // 4: 11.6 / 39.8), each wave with two chunks of its rows in flight; never more waves than rows
+  int n_wg = lim.cu_count * kGemvWgPerCu;
+  const int by_rows = (N + kGemvThreads / 64 - 1) / (kGemvThreads / 64);
+  if (n_wg > by_rows) n_wg = by_rows;
+  const dim3 grid((unsigned)n_wg), block(kGemvThreads);
+#define SOCKET_GR(GATE)                                                                                          \
+  do {                                                                                                           \
+    auto kern = norm_gemv_rows_kernel<M, GATE>;                                                                 \
+    if (lds > 48 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                              \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+      return SOCKET_ERR_LAUNCH;                                                                                  \
+    hipLaunchKernelGGL(kern, grid, block, lds, s, x, xs, r, nw, eps, h_out, w, wg, y, ys, N, K);                 \
+  } while (0)
+  if (wg) SOCKET_GR(true);
+  else SOCKET_GR(false);
+#undef SOCKET_GR
+  return SOCKET_OK;
 }
 
 template <int M>
@@ -375,6 +546,38 @@ extern "C" int socket_gemv_bf16(const void* x, int64_t x_stride, const void* w, 
     case 3: launch_gemv<3>(xp, x_stride, wp, gp, yp, y_stride, N, K, s); break;
     default: launch_gemv<4>(xp, x_stride, wp, gp, yp, y_stride, N, K, s); break;
   }
+  SOCKET_LAUNCH_CHECK();
+  return SOCKET_OK;
+}
+
+extern "C" int socket_norm_gemv_bf16(const void* x, const void* residual, const void* norm_weight, float eps,
+                                     void* h_out, const void* w, const void* w_gate, void* y, int M, int N, int K,
+                                     void* stream) {
+  SOCKET_REQUIRE(x && norm_weight && w && y, SOCKET_ERR_NULL);
+  SOCKET_REQUIRE((residual == nullptr) == (h_out == nullptr), SOCKET_ERR_NULL);
+  SOCKET_REQUIRE(M >= 1 && N >= 1 && K >= 1, SOCKET_ERR_SHAPE);
+  SOCKET_REQUIRE(M <= 4 && K % (kGemvStep * kGemvUnroll) == 0 && K <= kNormThreads * kNormVecs * 8,
+                 SOCKET_ERR_UNSUPPORTED);
+  SOCKET_REQUIRE(socket_aligned16(x) && socket_aligned16(norm_weight) && socket_aligned16(w) &&
+                     (!w_gate || socket_aligned16(w_gate)) && (!residual || socket_aligned16(residual)) &&
+                     (!h_out || socket_aligned16(h_out)),
+                 SOCKET_ERR_ALIGN);
+  hipStream_t s = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* rp = (const uint16_t*)residual;
+  const uint16_t* np = (const uint16_t*)norm_weight;
+  const uint16_t* wp = (const uint16_t*)w;
+  const uint16_t* gp = (const uint16_t*)w_gate;
+  uint16_t* hp = (uint16_t*)h_out;
+  uint16_t* yp = (uint16_t*)y;
+  int rc;
+  switch (M) {
+    case 1: rc = launch_norm_gemv_rows<1>(xp, K, rp, np, eps, hp, wp, gp, yp, N, N, K, s); break;
+    case 2: rc = launch_norm_gemv_rows<2>(xp, K, rp, np, eps, hp, wp, gp, yp, N, N, K, s); break;
+    case 3: rc = launch_norm_gemv_rows<3>(xp, K, rp, np, eps, hp, wp, gp, yp, N, N, K, s); break;
+    default: rc = launch_norm_gemv_rows<4>(xp, K, rp, np, eps, hp, wp, gp, yp, N, N, K, s); break;
+  }
+  if (rc != SOCKET_OK) return rc;
   SOCKET_LAUNCH_CHECK();
   return SOCKET_OK;
 }

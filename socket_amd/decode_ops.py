@@ -95,3 +95,31 @@ def linear_rows(x: torch.Tensor, weight: torch.Tensor, gate_weight: torch.Tensor
     check("socket_gemv_bf16", lib().socket_gemv_bf16(ptr(x), K, ptr(weight), ptr(gate_weight),
                                                      ptr(y), N, rows, N, K, stream_ptr(x.device)))
     return y
+
+
+@torch.no_grad()
+def norm_linear_rows(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor],
+                     weight: torch.Tensor, gate_weight: torch.Tensor = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(h, y) with h, xn = add_rmsnorm(x, norm_weight, eps, residual) and y = linear_rows(xn,
+    weight, gate_weight): one launch where the matrix-vector kernel takes the shape (every
+    workgroup normalises the row for itself; same values bit for bit), the two calls otherwise."""
+    rows = x.numel() // x.shape[-1]
+    K, N = x.shape[-1], weight.shape[0]
+    fits = (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+            and norm_weight.dtype == torch.bfloat16 and norm_weight.is_contiguous()
+            and rows <= (1 if gate_weight is None else 4)
+            and K % 2048 == 0 and K <= 8192 and weight.is_contiguous() and x.is_contiguous()
+            and (residual is None or (residual.shape == x.shape and residual.dtype == x.dtype
+                                      and residual.is_contiguous()))
+            and (gate_weight is None or (gate_weight.is_contiguous() and gate_weight.shape == weight.shape
+                                         and gate_weight.dtype == torch.bfloat16)))
+    if not fits:
+        h, xn = add_rmsnorm(x, norm_weight, eps, residual=residual)
+        return h, linear_rows(xn, weight, gate_weight)
+    h = x if residual is None else torch.empty_like(x)
+    y = torch.empty(*x.shape[:-1], N, dtype=x.dtype, device=x.device)
+    check("socket_norm_gemv_bf16", lib().socket_norm_gemv_bf16(
+        ptr(x), ptr(residual), ptr(norm_weight), float(eps), ptr(h) if residual is not None else None,
+        ptr(weight), ptr(gate_weight), ptr(y), rows, N, K, stream_ptr(x.device)))
+    return h, y
+

@@ -389,10 +389,11 @@ class TransformerBlock(nn.Module):
         the previous block's FFN output, None for the first); returns the new
         residual stream and this block's FFN output, not yet added."""
         an, fn, ff = self.attention_norm, self.ffn_norm, self.feed_forward
-        x, y = decode_ops.add_rmsnorm(x, an.weight, an.eps, residual=pending)
-        a = self.attention._run_fused(y, input_pos, sparse, step)
-        h, y = decode_ops.add_rmsnorm(x, fn.weight, fn.eps, residual=a)
-        return h, decode_ops.linear_rows(decode_ops.linear_rows(y, ff.w1.weight, ff.w3.weight), ff.w2.weight)
+        # (each norm runs inside the launch of the product it feeds)
+        x, qkv = decode_ops.norm_linear_rows(x, an.weight, an.eps, pending, self.attention.wqkv.weight)
+        a = self.attention._run_fused_qkv(qkv, input_pos, sparse, step)
+        h, g = decode_ops.norm_linear_rows(x, fn.weight, fn.eps, a, ff.w1.weight, ff.w3.weight)
+        return h, decode_ops.linear_rows(g, ff.w2.weight)
 
     def forward(self, x: Tensor, input_pos: Tensor, freqs_cis: Tensor, mask: Tensor = None) -> Tensor:
         return self._run(x, input_pos, freqs_cis, False, None)
@@ -508,9 +509,12 @@ class Attention(nn.Module):
     def _run_fused(self, x: Tensor, input_pos: Tensor, sparse: bool, step: "DecodeStep") -> Tensor:
         """The decode step of `_run` with rotary embedding, K/V append and length
         update in one launch (same values)."""
-        bsz = x.shape[0]
+        return self._run_fused_qkv(decode_ops.linear_rows(x, self.wqkv.weight), input_pos, sparse, step)
+
+    def _run_fused_qkv(self, qkv: Tensor, input_pos: Tensor, sparse: bool, step: "DecodeStep") -> Tensor:
+        """`_run_fused` from the projected row on (`qkv` = wqkv applied to the normalised input)."""
+        bsz = qkv.shape[0]
         cache = self.kv_cache
-        qkv = decode_ops.linear_rows(x, self.wqkv.weight)
         if sparse and _sparse_is_slower(self.config, cache, self.n_head):
             # below the crossover: the dense kernel, with the new key still hashed so that the
             # cache's hash state stays complete

@@ -438,6 +438,36 @@ def test_linear_rows_equals_the_fp32_product_rounded_once(dev, rows, N, K):
     assert torch.equal(decode_ops.linear_rows(x5, w), torch.nn.functional.linear(x5, w))
 
 
+@pytest.mark.parametrize("rows,N,K,gate,res", [
+    (1, 6144, 4096, False, True), (1, 6144, 4096, False, False), (1, 14336, 4096, True, True),
+    (4, 1001, 2048, True, True), (3, 515, 8192, True, False), (2, 4099, 4096, True, True),
+])
+def test_norm_linear_rows_equals_the_two_launches(dev, rows, N, K, gate, res):
+    """RMSNorm (with the residual add before it) inside the matrix-vector launch: h and
+    the product equal add_rmsnorm followed by linear_rows bit for bit, also twice in a
+    row and for an output count that does not fill the last workgroup; shapes the
+    kernel does not take go through the two calls."""
+    from socket_amd import decode_ops
+    g = torch.Generator().manual_seed(N * 3 + K + rows)
+    x = torch.randn(rows, 1, K, generator=g).to(torch.bfloat16).to(dev)
+    r = torch.randn(rows, 1, K, generator=g).to(torch.bfloat16).to(dev) if res else None
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16).to(dev)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    wg = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16).to(dev) if gate else None
+    x0, r0 = x.clone(), None if r is None else r.clone()
+    h_want, xn = decode_ops.add_rmsnorm(x, nw, 1e-5, residual=r)
+    y_want = decode_ops.linear_rows(xn, w, wg)
+    for _ in range(2):
+        h, y = decode_ops.norm_linear_rows(x, nw, 1e-5, r, w, wg)
+        assert torch.equal(h, h_want) and torch.equal(y, y_want)
+        assert (h is x) == (r is None)
+    assert torch.equal(x, x0) and (r is None or torch.equal(r, r0))     # inputs untouched
+    if not gate:
+        x2 = torch.randn(2, 1, K, generator=g).to(torch.bfloat16).to(dev)
+        h2, y2 = decode_ops.norm_linear_rows(x2, nw, 1e-5, None, w)
+        assert torch.equal(y2, decode_ops.linear_rows(decode_ops.add_rmsnorm(x2, nw, 1e-5)[1], w))
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)])
 @pytest.mark.parametrize("sparse", [True, False])
 def test_fused_decode_step_equals_the_plain_one(dev, dtype, tol, sparse):
