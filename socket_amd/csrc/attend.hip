@@ -134,9 +134,21 @@ constexpr int kMergeThreads = 256;
 // largest log-sum-exp first, then the lanes, four output coordinates each and
 // 256 / (D/4) splits side by side, add up weight * partial with independent
 // loads, and LDS folds the side-by-side groups.
-template <int D, bool COHERENT = false>
+constexpr int kMergeEarly = 4;   // rounds of splits a lane of stage2_kernel requests before it knows the row's length
+
+// EARLY (stage2_kernel): the lane's first log-sum-exp of the maximum sweep and its first
+// kMergeEarly rounds of (log-sum-exp, partial) were requested by the caller for every split
+// that exists, before the row's length was known -- one memory round trip instead of three
+// dependent ones; what lies past `nblk` is ignored here.  Same arithmetic in the same order.
+struct MergeEarly {
+  float m0;
+  float lse[kMergeEarly];
+  float4 o[kMergeEarly];
+};
+
+template <int D, bool COHERENT = false, bool EARLY = false>
 __device__ __forceinline__ void merge_splits(const float* mo, const float* ml, int nblk, void* __restrict__ out,
-                                             int out_dtype, int64_t out_off) {
+                                             int out_dtype, int64_t out_off, const MergeEarly* early = nullptr) {
   constexpr int LPD = D / 4;                    // lanes across the head dimension
   constexpr int NG = kMergeThreads / LPD;       // splits handled side by side
   constexpr int kW = kMergeThreads / SOCKET_WAVE;
@@ -147,7 +159,12 @@ __device__ __forceinline__ void merge_splits(const float* mo, const float* ml, i
   const int lane = tid & 63, wave = tid >> 6;
 
   float m = -INFINITY;
-  for (int s = tid; s < nblk; s += kMergeThreads) m = fmaxf(m, COHERENT ? load_coherent(ml + s) : ml[s]);
+  if (EARLY) {
+    if (tid < nblk) m = fmaxf(m, early->m0);
+    for (int s = tid + kMergeThreads; s < nblk; s += kMergeThreads) m = fmaxf(m, ml[s]);
+  } else {
+    for (int s = tid; s < nblk; s += kMergeThreads) m = fmaxf(m, COHERENT ? load_coherent(ml + s) : ml[s]);
+  }
   m = wave_reduce_to_last<true>(m);
   if (lane == 63) red[wave] = m;
   __syncthreads();
@@ -158,11 +175,24 @@ __device__ __forceinline__ void merge_splits(const float* mo, const float* ml, i
   const int grp = tid / LPD, d4 = (tid % LPD) * 4;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   float sum = 0.f;
-  for (int s = grp; s < nblk; s += NG) {
-    const float lse = COHERENT ? load_coherent(ml + s) : ml[s];
-    // a split without a live row has lse = -inf and weight 0; so has every split
-    // when nothing at all was attended (m = -inf), which leaves 0/0 below
+  // (a split without a live row has lse = -inf and weight 0; so has every split
+  // when nothing at all was attended (m = -inf), which leaves 0/0 below)
+  auto add = [&](float lse, const float4& o) __attribute__((always_inline)) {
     const float w = (lse == -INFINITY) ? 0.f : fast_exp(lse - m);
+    acc.x += w * o.x;
+    acc.y += w * o.y;
+    acc.z += w * o.z;
+    acc.w += w * o.w;
+    sum += w;
+  };
+  int s = grp;
+  if (EARLY) {
+#pragma unroll
+    for (int it = 0; it < kMergeEarly; ++it, s += NG)
+      if (s < nblk) add(early->lse[it], early->o[it]);
+  }
+  for (; s < nblk; s += NG) {
+    const float lse = COHERENT ? load_coherent(ml + s) : ml[s];
     float4 o;
     if (COHERENT) {
       const float* src = mo + (int64_t)s * D + d4;
@@ -170,11 +200,7 @@ __device__ __forceinline__ void merge_splits(const float* mo, const float* ml, i
     } else {
       o = *reinterpret_cast<const float4*>(mo + (int64_t)s * D + d4);
     }
-    acc.x += w * o.x;
-    acc.y += w * o.y;
-    acc.z += w * o.z;
-    acc.w += w * o.w;
-    sum += w;
+    add(lse, o);
   }
   part[grp][d4] = acc.x;
   part[grp][d4 + 1] = acc.y;
@@ -204,12 +230,25 @@ __global__ __launch_bounds__(kMergeThreads) void stage2_kernel(
     const int32_t* __restrict__ sparse_len, int64_t len_sb, int64_t len_sh, void* __restrict__ out,
     int out_dtype, int64_t out_sb, int64_t out_sh, int Hq, int nsplit, int block_seq) {
   const int h = blockIdx.x, b = blockIdx.y;
+  const float* mo = mid_o + ((int64_t)b * Hq + h) * nsplit * D;
+  const float* ml = mid_lse + ((int64_t)b * Hq + h) * nsplit;
+  // the partials of every split that exists are requested together with the length (those past the
+  // row's length hold whatever the workspace held and are ignored)
+  constexpr int LPD = D / 4, NG = kMergeThreads / LPD;
+  const int tid = threadIdx.x, grp = tid / LPD, d4 = (tid % LPD) * 4;
+  MergeEarly early;
+  early.m0 = tid < nsplit ? ml[tid] : -INFINITY;
+#pragma unroll
+  for (int it = 0; it < kMergeEarly; ++it) {
+    const int s = min(grp + it * NG, nsplit - 1);
+    early.lse[it] = ml[s];
+    early.o[it] = *reinterpret_cast<const float4*>(mo + (int64_t)s * D + d4);
+  }
   const int len = sparse_len[b * len_sb + h * len_sh];
   // (a length beyond nsplit * block_seq is cut to the splits that exist)
   int nblk = len <= 0 ? 0 : (len + block_seq - 1) / block_seq;
   nblk = min(nblk, nsplit);
-  merge_splits<D>(mid_o + ((int64_t)b * Hq + h) * nsplit * D, mid_lse + ((int64_t)b * Hq + h) * nsplit, nblk, out,
-                  out_dtype, b * out_sb + h * out_sh);
+  merge_splits<D, false, true>(mo, ml, nblk, out, out_dtype, b * out_sb + h * out_sh, &early);
 }
 
 // FINISH: the workgroup that completes a row's last outstanding split also merges
