@@ -687,7 +687,11 @@ def main():
                           "gbs": round(read_ceiling_gbs(dev), 1)}))
         return
     if args.only == "decode":
-        print(json.dumps({"only": "decode", "ctx_128k": decode_tok_s(dev, 131072 - 128, 128)}))
+        if args.workload == "c4":
+            print(json.dumps({"only": "decode", "c4_prompt_65536": decode_tok_s(
+                dev, 65536, 256, kinds=("sparse", "dense", "sparse_or_dense"))}))
+        else:
+            print(json.dumps({"only": "decode", "ctx_128k": decode_tok_s(dev, 131072 - 128, 128)}))
         return
     w = WORKLOADS[args.workload]
     iters = max(args.steps, 1)

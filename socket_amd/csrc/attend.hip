@@ -236,15 +236,15 @@ __global__ __launch_bounds__(kMergeThreads) void stage2_kernel(
   // row's length hold whatever the workspace held and are ignored)
   constexpr int LPD = D / 4, NG = kMergeThreads / LPD;
   const int tid = threadIdx.x, grp = tid / LPD, d4 = (tid % LPD) * 4;
+  const int len = sparse_len[b * len_sb + h * len_sh];   // (a scalar load: on its way while the rest is requested)
   MergeEarly early;
-  early.m0 = tid < nsplit ? ml[tid] : -INFINITY;
+  early.m0 = ml[min(tid, nsplit - 1)];   // (unconditional: a load under a condition is waited for on the spot)
 #pragma unroll
   for (int it = 0; it < kMergeEarly; ++it) {
     const int s = min(grp + it * NG, nsplit - 1);
     early.lse[it] = ml[s];
     early.o[it] = *reinterpret_cast<const float4*>(mo + (int64_t)s * D + d4);
   }
-  const int len = sparse_len[b * len_sb + h * len_sh];
   // (a length beyond nsplit * block_seq is cut to the splits that exist)
   int nblk = len <= 0 ? 0 : (len + block_seq - 1) / block_seq;
   nblk = min(nblk, nsplit);

@@ -147,7 +147,9 @@ __device__ __forceinline__ void soft_hash_block(
       if (i < G * D) {
         sh_load4<DT>(q, b * q_sb + (int64_t)(kvh * G + i / D) * q_sh + i % D, qv[u]);
         if constexpr (kRope) {
-          if (rope_on) sh_load4<FT>(freqs, (rope_pos * (D / 2) + (i % D) / 2) * 2, fv[u]);
+          // (always fetched, from row 0 when the position is outside the table: a load under a
+          // condition would make the compiler wait for every load issued so far, one by one)
+          sh_load4<FT>(freqs, ((rope_on ? rope_pos : 0) * (D / 2) + (i % D) / 2) * 2, fv[u]);
         }
       }
     }
@@ -526,9 +528,11 @@ __global__ __launch_bounds__(kSHThreads) void decode_prologue_kernel(
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const int e0 = ks * 32 + quarter * 8;
+      // (all three fetched whether needed or not -- the angles from row 0 for a position outside
+      // the table, the value row by every wave: loads under a condition are waited for one by one)
       raw[ks] = *reinterpret_cast<const uint4*>(krow + e0);
-      if (rope_on) sh_load8<FT>(freqs, p * D + e0, f[ks]);   // ((p * D/2) + e0/2) * 2
-      if (first) vf[ks].u = *reinterpret_cast<const uint4*>(vrow + e0);
+      sh_load8<FT>(freqs, (rope_on ? p : 0) * D + e0, f[ks]);   // ((p * D/2) + e0/2) * 2
+      vf[ks].u = *reinterpret_cast<const uint4*>(vrow + e0);
     }
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
