@@ -344,13 +344,18 @@ __device__ __forceinline__ void soft_hash_block(
       }
   }
   reduce(sm, false);
+  // (one reciprocal per head and a product per bucket where there were sixteen divisions a lane:
+  // the last write sweep was the longest phase of the workgroup)
+  float inv[GC];
+#pragma unroll
+  for (int g = 0; g < GC; ++g) inv[g] = 1.f / sm[g];
   for (int r0 = tid * 4; r0 < R; r0 += kSHThreads * 4) {
     if (!keep) logits4(r0, lg);
 #pragma unroll
     for (int g = 0; g < GC; ++g)
 #pragma unroll
       for (int i = 0; i < 4; ++i)   // now probabilities
-        lg[g][i] = (g < G) ? (keep ? lg[g][i] : expf(lg[g][i] - mx[g])) / sm[g] : 0.f;
+        lg[g][i] = (g < G) ? (keep ? lg[g][i] : expf(lg[g][i] - mx[g])) * inv[g] : 0.f;
     if (parts == 0) {
       // reference layout [B,Hq,L,R]
 #pragma unroll
